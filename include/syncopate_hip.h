@@ -1,0 +1,200 @@
+/*
+ * syncopate_hip.h — C ABI of libsyncopate_hip.so (MI355X / gfx950).
+ *
+ * Hand-written CDNA4 kernels for the per-rank chunk-scheduled compute path of
+ * Syncopate: the AG+GEMM consumer, the GEMM+RS producer and its chunked ring
+ * reduce, the chunked-KV flash attention, and the tiny stream-side flag
+ * primitives a single-GPU producer needs.  Every entry point takes plain
+ * pointers and sizes (device pointers unless a parameter says "host"), never
+ * allocates device memory, launches on the stream it is given and returns
+ * 0 on success, a negative SYN_E* code for rejected arguments, or a positive
+ * hipError_t.
+ *
+ * Units follow the reference's generated-kernel convention: wave sizes and
+ * offsets are in ELEMENTS and are divided by the block sizes inside the
+ * kernel (syncopate/computation/gemm/template.py:82-87,
+ * syncopate/computation/transform/transformer.py:616-621).
+ */
+#ifndef SYNCOPATE_HIP_H
+#define SYNCOPATE_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element types */
+#define SYN_DTYPE_BF16 0
+#define SYN_DTYPE_FP16 1
+
+/* argument errors (negative so they never collide with hipError_t) */
+#define SYN_EINVAL (-22)   /* malformed argument / unsupported configuration */
+#define SYN_ERANGE (-34)   /* wave table addresses tiles outside the operand  */
+#define SYN_EALIGN (-75)   /* pointer or extent not aligned as the kernel needs */
+
+/* device-side status words (int32[SYN_STATUS_WORDS], caller-zeroed) */
+#define SYN_STATUS_WORDS 4
+#define SYN_STATUS_OK 0
+#define SYN_STATUS_SPIN_TIMEOUT 1   /* [1]=wave index, [2]=program id, [3]=signal offset */
+
+/* gemm option bits */
+#define SYN_GEMM_XCD_REMAP 1u       /* permute hardware workgroup ids so that consecutive
+                                       logical program ids share an XCD (and its L2)      */
+
+typedef void* syn_stream_t;        /* hipStream_t */
+
+/*
+ * Wave table of a GEMM launch: num_waves rows, row w = one wave (one arrived
+ * chunk).  wave_sizes[w] = {rows, cols} and wave_offsets[w] = {row0, col0} of
+ * the C region the wave covers, in elements; signal_offsets[w] = index of the
+ * flag word that gates (consumer) or publishes (producer) the wave, or -1.
+ * Produced by RawSchedule.gen_block_shape_lists / gen_block_offset_lists /
+ * gen_signal_lists (syncopate/interface/tile_schedule.py:90-115).
+ */
+typedef struct syn_gemm_desc {
+    const void* a;                  /* [M, K] row-major                                    */
+    const void* b;                  /* [N, K] row-major (K contiguous), template.py:53-58  */
+    void* c;                        /* [M, N] row-major                                    */
+    uint64_t* flags;                /* flag words, value 1 = set                           */
+    const int32_t* wave_sizes;      /* device, [num_waves, 2]                              */
+    const int32_t* wave_offsets;    /* device, [num_waves, 2]                              */
+    const int32_t* signal_offsets;  /* device, [num_waves]                                 */
+    int32_t* counters;              /* producer only: device int32[num_waves], zeroed      */
+    int32_t* visit_log;             /* optional device int32[num_tiles, 4]:
+                                       {program id, wave, pid_m, pid_n} per tile id         */
+    int32_t* status;                /* optional device int32[SYN_STATUS_WORDS]             */
+    int32_t num_waves;
+    int32_t M, N, K;
+    int32_t dtype;                  /* SYN_DTYPE_*                                         */
+    int32_t block_m, block_n, block_k;
+    int32_t group_m;                /* GROUP_SIZE_M of get_pid_mn, template.py:10-18       */
+    int32_t num_sms;                /* NUM_SMS: tile id stride of the persistent walk      */
+    int64_t cum_tiles;              /* sum rows*cols over waves (elements); 0 = M*N        */
+    int64_t spin_timeout_us;        /* <=0: default (2 s); flag waits give up after this   */
+    uint32_t options;               /* SYN_GEMM_* bits                                     */
+} syn_gemm_desc;
+
+/*
+ * AG+GEMM consumer: C = A * B^T with fp32 accumulation, output tiles visited
+ * in wave order by a persistent grid; before the first tile of a wave whose
+ * signal offset is >= 0 the workgroup spins (acquire) until that flag == 1.
+ * Replaces kernel_gemm_consumer / gemm_consumer
+ * (syncopate/computation/gemm/template.py:21-220) and the generated
+ * consumer form (syncopate/computation/transform/transformer.py:759-879).
+ */
+int syn_gemm_consumer(const syn_gemm_desc* desc, syn_stream_t stream);
+
+/*
+ * GEMM+RS producer: same GEMM and walk; after each C tile of a wave with a
+ * signal offset >= 0 the workgroup does counters[wave]++ (release) and the
+ * one that observes rows*cols/(BM*BN) - 1 sets flags[signal] = 1.
+ * Replaces kernel_gemm_producer / gemm_producer
+ * (syncopate/computation/gemm/template.py:224-412).
+ */
+int syn_gemm_producer(const syn_gemm_desc* desc, syn_stream_t stream);
+
+/*
+ * Host-only check of a GEMM wave table against the operand shapes, block
+ * sizes and flag-array length; the launch entry points cannot do it because
+ * the tables they get live in device memory.  All pointers are HOST pointers.
+ * Returns 0, SYN_EINVAL or SYN_ERANGE.  No reference counterpart: the
+ * reference launches unchecked (template.py:177-185 asserts shapes only).
+ */
+int syn_gemm_check_waves(const int32_t* wave_sizes, const int32_t* wave_offsets,
+                         const int32_t* signal_offsets, int32_t num_waves,
+                         int32_t M, int32_t N, int32_t K,
+                         int32_t block_m, int32_t block_n, int32_t block_k,
+                         int64_t cum_tiles, int64_t num_flags);
+
+/* Number of workgroups syn_gemm_* will launch: min(num_sms, tiles)
+ * (template.py:193-197). */
+int syn_gemm_grid(int64_t cum_tiles, int32_t M, int32_t N, int32_t block_m,
+                  int32_t block_n, int32_t num_sms);
+
+/*
+ * Chunked ring reduce of GEMM+RS:
+ *   out[m, n] = local[rank*Mr + m, n] + sum_{i=1..W-1} recv[(rank+i) % W, m, n]
+ * added left to right.  acc_mode 0 rounds the running sum to the element type
+ * after every add (what the reference's `accum += data` on dtype tensors does,
+ * tests/test_gemm_rs.py:64-70); acc_mode 1 keeps the running sum in fp32 and
+ * rounds once.  recv is [W, Mr, N] (slot `rank` is never read), local is
+ * [W*Mr, N], out is [Mr, N]; Mr*N must be a multiple of 8.
+ * Replaces kernel_ring_reduce_tma / ring_reduce_tma (tests/test_gemm_rs.py:22-121).
+ */
+int syn_ring_reduce(const void* recv, const void* local, void* out,
+                    int32_t world, int32_t rank, int64_t rows_per_rank, int64_t N,
+                    int32_t dtype, int32_t acc_mode, syn_stream_t stream);
+
+/*
+ * Chunked-KV flash attention forward.  One workgroup per tile id; tile id ->
+ * (wave, z, h, q block, kv block range) exactly as the reference's wave lookup
+ * (syncopate/computation/attn/template.py:39-44,80-121; generated form
+ * transformer.py:555-660).  Table rows are {Z, H, Q, KV} sizes/offsets in
+ * ELEMENTS along Q and KV (divided by block_m / block_n in the kernel) and
+ * cum_wave_sizes is the inclusive prefix sum of Z*H*Q elements.  Each program
+ * computes its partial (O, lse2) with a base-2 online softmax and merges it
+ * into o / lse under a per-q-block lock (template.py:307-361).  With
+ * causal != 0, kv blocks wholly above the diagonal are skipped and the
+ * diagonal block is masked (col > row); q and kv positions are global
+ * sequence positions, so it needs Sq == Skv indexing (q row i attends kv <= i).
+ * lse is fp32 [Z, H, Sq] (base-2 log-sum-exp), lock and first are zeroed
+ * int32 [Z, H, Sq / block_m] scratch owned by the caller.
+ */
+typedef struct syn_attn_desc {
+    const void* q;                  /* [Z, H, Sq, D]                                      */
+    const void* k;                  /* [Z, H, Skv, D]                                     */
+    const void* v;                  /* [Z, H, Skv, D]                                     */
+    void* o;                        /* [Z, H, Sq, D]                                      */
+    float* lse;                     /* [Z, H, Sq]                                         */
+    int32_t* lock;                  /* [Z, H, Sq/block_m], zeroed                         */
+    int32_t* first;                 /* [Z, H, Sq/block_m], zeroed                         */
+    uint64_t* flags;
+    const int32_t* wave_offsets;    /* device, [num_waves, 4]                             */
+    const int32_t* wave_sizes;      /* device, [num_waves, 4]                             */
+    const int32_t* cum_wave_sizes;  /* device, [num_waves]                                */
+    const int32_t* signal_offsets;  /* device, [num_waves]                                */
+    int32_t* visit_log;             /* optional device int32[num_tiles, 8]:
+                                       {wave, z, h, q_block, kv_lo, kv_hi, signal, program}      */
+    int32_t* status;                /* optional device int32[SYN_STATUS_WORDS]            */
+    int32_t num_waves;
+    int32_t Z, H, Sq, Skv, D;
+    int32_t dtype;
+    int32_t block_m, block_n;
+    int32_t causal;
+    int32_t num_programs;           /* persistent grid: workgroup b runs tiles b, b+grid, ...;
+                                       <= 0 launches one workgroup per tile as the reference */
+    float sm_scale;
+    int64_t cum_tiles;              /* total Z*H*Q elements over all waves                */
+    int64_t spin_timeout_us;
+} syn_attn_desc;
+
+int syn_attn_fwd(const syn_attn_desc* desc, syn_stream_t stream);
+
+/* Host-only check of an attention wave table (HOST pointers). */
+int syn_attn_check_waves(const int32_t* wave_offsets, const int32_t* wave_sizes,
+                         const int32_t* cum_wave_sizes, const int32_t* signal_offsets,
+                         int32_t num_waves, int32_t Z, int32_t H, int32_t Sq, int32_t Skv,
+                         int32_t block_m, int32_t block_n, int64_t cum_tiles,
+                         int64_t num_flags);
+
+/*
+ * Stream-side primitives of the single-GPU producer; counterparts of the
+ * reference runtime's cudaMemcpyAsync / cuStreamWriteValue / cuStreamWaitValue
+ * calls (syncopate/communication/comm_runtime/communication_context.py:129-160).
+ */
+int syn_copy_async(void* dst, const void* src, int64_t nbytes, syn_stream_t stream);
+int syn_flag_set(uint64_t* flag, uint64_t value, syn_stream_t stream);
+int syn_flag_wait(const uint64_t* flag, uint64_t value, int64_t spin_timeout_us,
+                  int32_t* status, syn_stream_t stream);
+/* Occupy the stream for about `us` microseconds with one sleeping wavefront
+ * (models a slow link in front of a chunk copy). */
+int syn_delay_us(int64_t us, syn_stream_t stream);
+
+/* Library/ABI version: major*10000 + minor*100 + patch. */
+int syn_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SYNCOPATE_HIP_H */

@@ -1,0 +1,134 @@
+"""Helpers shared by the kernel launchers: status words, wave-table checks, pointers."""
+
+from __future__ import annotations
+
+import ctypes
+import weakref
+from typing import Dict, Optional, Sequence, Tuple, Union
+
+import torch
+
+from .. import _lib
+
+TableLike = Union[torch.Tensor, Sequence]
+
+# One int32[SYN_STATUS_WORDS] block per device.  A kernel whose flag wait times
+# out records (code, wave, program id, signal offset) here and exits.
+_status: Dict[int, torch.Tensor] = {}
+
+
+def status_words(device: torch.device) -> torch.Tensor:
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    buf = _status.get(idx)
+    if buf is None:
+        buf = torch.zeros(_lib.SYN_STATUS_WORDS, dtype=torch.int32, device=torch.device("cuda", idx))
+        _status[idx] = buf
+    return buf
+
+
+class FlagWaitTimeout(RuntimeError):
+    """A kernel gave up spinning on a flag word that was never set."""
+
+
+def check_status(device: Optional[torch.device] = None, *, reset: bool = True) -> None:
+    """Synchronise `device` and raise if a kernel reported a flag-wait time-out."""
+    devices = list(_status) if device is None else [
+        device.index if device.index is not None else torch.cuda.current_device()
+    ]
+    for idx in devices:
+        buf = _status.get(idx)
+        if buf is None:
+            continue
+        torch.cuda.synchronize(idx)
+        words = buf.tolist()
+        if words[0] != 0:
+            if reset:
+                buf.zero_()
+            if words[0] == _lib.SYN_STATUS_SPIN_TIMEOUT:
+                raise FlagWaitTimeout(
+                    f"flag wait timed out on cuda:{idx}: wave {words[1]}, program {words[2]}, "
+                    f"signal offset {words[3]}"
+                )
+            raise RuntimeError(f"kernel status {words} on cuda:{idx}")
+
+
+def as_device_table(table: TableLike, device: torch.device, width: Optional[int]) -> torch.Tensor:
+    """int32, contiguous, on `device`; `width` = row length (None for 1-D tables)."""
+    if isinstance(table, torch.Tensor):
+        t = table
+        if t.dtype != torch.int32:
+            raise TypeError(f"wave tables must be int32, got {t.dtype}")
+        if t.device != device:
+            t = t.to(device)
+    else:
+        t = torch.tensor(table, dtype=torch.int32, device=device)
+    t = t.contiguous()
+    if width is None:
+        if t.dim() != 1:
+            raise ValueError(f"expected a 1-D table, got shape {tuple(t.shape)}")
+    else:
+        if t.numel() % width:
+            raise ValueError(f"table of {t.numel()} entries is not rows of {width}")
+        t = t.view(-1, width)
+    return t
+
+
+def host_copy(t: torch.Tensor) -> torch.Tensor:
+    return t.detach().to("cpu", copy=True).contiguous()
+
+
+# Tables that passed the host-side check are remembered per tensor OBJECT (weak
+# reference + in-place version counter), never per address: the caching
+# allocator hands the address of a freed table to the next one.  A table given
+# as a list or CPU tensor is checked on every call (its host copy is free).
+_checked: Dict[Tuple[int, ...], Tuple[Tuple, Tuple[int, ...], Tuple]] = {}
+
+
+def already_checked(tensors: Sequence[torch.Tensor], params: Tuple) -> bool:
+    entry = _checked.get(tuple(id(t) for t in tensors))
+    if entry is None:
+        return False
+    refs, versions, seen_params = entry
+    if seen_params != params:
+        return False
+    for t, ref, ver in zip(tensors, refs, versions):
+        if ref() is not t or t._version != ver:
+            return False
+    return True
+
+
+def remember_checked(tensors: Sequence[torch.Tensor], params: Tuple) -> None:
+    if len(_checked) > 1024:
+        _checked.clear()
+    _checked[tuple(id(t) for t in tensors)] = (
+        tuple(weakref.ref(t) for t in tensors),
+        tuple(t._version for t in tensors),
+        params,
+    )
+
+
+def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def host_ptr(t: torch.Tensor) -> ctypes.c_void_p:
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def require_cuda(*tensors: torch.Tensor) -> torch.device:
+    dev = tensors[0].device
+    for t in tensors:
+        if not t.is_cuda:
+            raise ValueError("operands must live in GPU memory (the kernels have no CPU path)")
+        if t.device != dev:
+            raise ValueError("operands must be on the same device")
+    return dev
+
+
+def flag_buffer(signal_buffer: torch.Tensor) -> torch.Tensor:
+    """Flag arrays are 8-byte words (value 1 = set); int64 and uint64 are both accepted."""
+    if signal_buffer.element_size() != 8 or signal_buffer.is_floating_point():
+        raise TypeError(f"signal buffer must hold 64-bit integer words, got {signal_buffer.dtype}")
+    if not signal_buffer.is_contiguous():
+        raise ValueError("signal buffer must be contiguous")
+    return signal_buffer

@@ -1,0 +1,201 @@
+"""Launchers of the chunked-KV flash-attention kernel (MI355X HIP, through the C ABI).
+
+Two call forms, as in the reference:
+
+* ``attention(q, k, v, sm_scale, wave_dicts)`` — the hand-written template's
+  launcher (syncopate/computation/attn/template.py:366-439).  Table entries
+  along Q and KV are in BLOCKS, `cum_wave_sizes` counts programs, tables may be
+  padded with zero rows to a power of two (template.py:567-641).
+* ``attention_forward(q, k, v, sm_scale, *, wave_offsets, wave_sizes,
+  cum_wave_sizes, signal_ptr, signal_offsets, NUM_WAVES, cum_tiles)`` — the
+  launcher the transform pass generates (syncopate/computation/transform/
+  transformer.py:1125-1137; used in tests/test_allgather_attn_transform.py:206-214).
+  Table entries along Q and KV are in ELEMENTS and `cum_wave_sizes`/`cum_tiles`
+  count Z*H*Q elements.
+
+Layout: q, o [Z, H, Sq, D]; k, v [Z, H, Skv, D]; D = 128; bf16 or fp16.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Dict, Optional
+
+import torch
+
+from ... import _lib
+from .._launch import (
+    TableLike,
+    already_checked,
+    as_device_table,
+    flag_buffer,
+    host_copy,
+    host_ptr,
+    remember_checked,
+    require_cuda,
+    status_words,
+)
+
+BLOCK_M = 128
+BLOCK_N = 128
+DEFAULT_SPIN_TIMEOUT_US = 2_000_000
+
+
+def attention_forward(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    sm_scale: float,
+    *,
+    wave_offsets: TableLike,
+    wave_sizes: TableLike,
+    cum_wave_sizes: TableLike,
+    signal_ptr: torch.Tensor,
+    signal_offsets: TableLike,
+    NUM_WAVES: Optional[int] = None,
+    cum_tiles: Optional[int] = None,
+    causal: bool = False,
+    num_programs: int = 0,
+    out: Optional[torch.Tensor] = None,
+    return_lse: bool = False,
+    visit_log: Optional[torch.Tensor] = None,
+    spin_timeout_us: int = DEFAULT_SPIN_TIMEOUT_US,
+    stream: Optional[torch.cuda.Stream] = None,
+):
+    """Chunk-gated attention forward; returns o (and the base-2 lse if asked).
+
+    `causal` is an extension over the reference (which is non-causal): kv blocks
+    above the diagonal are skipped, the diagonal block is masked.
+    `num_programs` > 0 runs that many persistent workgroups over the tile ids
+    instead of one workgroup per tile.
+    """
+    dev = require_cuda(q, k, v, signal_ptr)
+    if not (q.dtype == k.dtype == v.dtype):
+        raise TypeError("q, k and v must share one element type")
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise ValueError("q, k, v must be [Z, H, S, D]")
+    HEAD_DIM_Q, HEAD_DIM_K, HEAD_DIM_V = q.shape[-1], k.shape[-1], v.shape[-1]
+    assert HEAD_DIM_Q == HEAD_DIM_K and HEAD_DIM_K == HEAD_DIM_V
+    if HEAD_DIM_K != 128:
+        raise ValueError("the gfx950 kernel is specialised for head_dim 128")
+    Z, H, Sq, D = q.shape
+    if k.shape[:2] != q.shape[:2] or v.shape != k.shape:
+        raise ValueError("k and v must be [Z, H, Skv, D] with q's Z and H")
+    Skv = k.shape[2]
+    if not (q.is_contiguous() and k.is_contiguous() and v.is_contiguous()):
+        raise ValueError("q, k and v must be contiguous (views of a contiguous comm buffer are fine)")
+    flags = flag_buffer(signal_ptr)
+
+    offs = as_device_table(wave_offsets, dev, 4)
+    sizes = as_device_table(wave_sizes, dev, 4)
+    cums = as_device_table(cum_wave_sizes, dev, None)
+    sigs = as_device_table(signal_offsets, dev, None)
+    num_waves = cums.numel() if NUM_WAVES is None else int(NUM_WAVES)
+    if min(offs.shape[0], sizes.shape[0], cums.numel(), sigs.numel()) < num_waves:
+        raise ValueError("wave tables are shorter than NUM_WAVES")
+
+    lib = _lib.load()
+    tables = (wave_offsets, wave_sizes, cum_wave_sizes, signal_offsets)   # the caller's objects
+    caller_owned = all(isinstance(t, torch.Tensor) and t.is_cuda
+                       for t in (wave_offsets, wave_sizes, cum_wave_sizes, signal_offsets))
+    params = (num_waves, Z, H, Sq, Skv, cum_tiles, flags.numel())
+    if cum_tiles is None or not (caller_owned and already_checked(tables, params)):
+        ho, hs, hc, hg = host_copy(offs), host_copy(sizes), host_copy(cums), host_copy(sigs)
+        if cum_tiles is None:
+            cum_tiles = int(hc[:num_waves].max().item())
+        _lib.check(
+            "syn_attn_check_waves",
+            lib.syn_attn_check_waves(host_ptr(ho), host_ptr(hs), host_ptr(hc), host_ptr(hg), num_waves,
+                                     Z, H, Sq, Skv, BLOCK_M, BLOCK_N, int(cum_tiles), flags.numel()),
+        )
+        if caller_owned:
+            remember_checked(tables, (num_waves, Z, H, Sq, Skv, cum_tiles, flags.numel()))
+
+    o = torch.empty_like(q) if out is None else out
+    if o.shape != q.shape or o.dtype != q.dtype or not o.is_contiguous():
+        raise ValueError("out must match q")
+    # lse (base 2), lock and first-writer marker: the reference's M / guard / first
+    # (template.py:382-384), one lock per 128-row q block
+    lse = torch.empty((Z, H, Sq), device=dev, dtype=torch.float32)
+    scratch = torch.zeros((2, Z, H, Sq // BLOCK_M), device=dev, dtype=torch.int32)
+    tiles = int(cum_tiles) // BLOCK_M
+    if visit_log is not None:
+        if visit_log.dtype != torch.int32 or visit_log.numel() < 8 * tiles or not visit_log.is_contiguous():
+            raise ValueError(f"visit_log must be a contiguous int32 tensor of at least {8 * tiles} words")
+
+    desc = _lib.AttnDesc(
+        q=q.data_ptr(), k=k.data_ptr(), v=v.data_ptr(), o=o.data_ptr(), lse=lse.data_ptr(),
+        lock=scratch[0].data_ptr(), first=scratch[1].data_ptr(), flags=flags.data_ptr(),
+        wave_offsets=offs.data_ptr(), wave_sizes=sizes.data_ptr(), cum_wave_sizes=cums.data_ptr(),
+        signal_offsets=sigs.data_ptr(),
+        visit_log=None if visit_log is None else visit_log.data_ptr(),
+        status=status_words(dev).data_ptr(),
+        num_waves=num_waves, Z=Z, H=H, Sq=Sq, Skv=Skv, D=D, dtype=_lib.dtype_code(q.dtype),
+        block_m=BLOCK_M, block_n=BLOCK_N, causal=1 if causal else 0, num_programs=int(num_programs),
+        sm_scale=float(sm_scale), cum_tiles=int(cum_tiles), spin_timeout_us=int(spin_timeout_us),
+    )
+    with torch.cuda.device(dev):
+        _lib.check("syn_attn_fwd", lib.syn_attn_fwd(ctypes.byref(desc), _lib.stream_handle(stream)))
+    return (o, lse) if return_lse else o
+
+
+def attention(q, k, v, sm_scale, wave_dicts: Dict, BLOCK_M=128, BLOCK_N=128, NUM_BUFFERS=2,
+              NUM_MMA_WARPS=8, NUM_MMA_GROUPS=2, **kwargs):
+    """Hand-template call form (template.py:366-439): tables in block units."""
+    if BLOCK_M != 128 or BLOCK_N != 128:
+        raise ValueError("the gfx950 kernel uses 128x128 blocks")
+    dev = q.device
+    offs = as_device_table(wave_dicts["wave_offsets"], dev, 4).clone()
+    sizes = as_device_table(wave_dicts["wave_sizes"], dev, 4).clone()
+    cums = as_device_table(wave_dicts["cum_wave_sizes"], dev, None).clone()
+    # blocks -> elements along Q and KV; programs -> Z*H*Q elements
+    scale = torch.tensor([1, 1, BLOCK_M, BLOCK_N], dtype=torch.int32, device=dev)
+    offs *= scale
+    sizes *= scale
+    cums *= BLOCK_M
+    signal_ptr = wave_dicts["signal_ptr"]
+    if signal_ptr.element_size() != 8:
+        # the reference's "everything resident" helper hands out int32 ones (template.py:622)
+        signal_ptr = signal_ptr.to(torch.int64)
+    return attention_forward(
+        q, k, v, sm_scale,
+        wave_offsets=offs, wave_sizes=sizes, cum_wave_sizes=cums,
+        signal_ptr=signal_ptr, signal_offsets=wave_dicts["signal_offsets"],
+        NUM_WAVES=wave_dicts.get("CUM_CHUNK_BLOCK"), **kwargs)
+
+
+def build_waves_and_signals_divisible(Z, H, N_CTX_Q, N_CTX_KV, *, BLOCK_M=128, BLOCK_N=128, w=4,
+                                      device="cuda"):
+    """Split only along KV into `w` equal waves, everything resident (all flags set):
+    the table shape of the reference's `_build_waves_and_signals_divisible`
+    (template.py:567-641), block units, padded with zero rows to a power of two.
+    """
+    if N_CTX_Q % BLOCK_M or N_CTX_KV % BLOCK_N or w <= 0:
+        raise ValueError("sequence lengths must be multiples of the block sizes and w positive")
+    nq = N_CTX_Q // BLOCK_M
+    nkv = N_CTX_KV // BLOCK_N
+    if nkv % w:
+        raise ValueError(f"(N_CTX_KV/BLOCK_N)={nkv} must be divisible by w({w})")
+    per = nkv // w
+    padded = 1 if w <= 1 else 1 << ((w - 1).bit_length())
+    offsets, sizes, cums = [], [], []
+    for i in range(w):
+        offsets.append([0, 0, 0, i * per])
+        sizes.append([Z, H, nq, per])
+        cums.append((i + 1) * Z * H * nq)
+    for _ in range(padded - w):
+        offsets.append([0, 0, 0, 0])
+        sizes.append([0, 0, 0, 0])
+        cums.append(0)
+    return dict(
+        wave_offsets=torch.tensor(offsets, dtype=torch.int32, device=device).flatten(),
+        wave_sizes=torch.tensor(sizes, dtype=torch.int32, device=device).flatten(),
+        cum_wave_sizes=torch.tensor(cums, dtype=torch.int32, device=device),
+        signal_ptr=torch.ones(padded, dtype=torch.int64, device=device),
+        signal_offsets=torch.zeros(padded, dtype=torch.int32, device=device),
+        CUM_CHUNK_BLOCK=padded,
+        num_pid_q=nq,
+        num_pid_kv_total=nkv,
+        kv_per_wave=per,
+        w=w,
+    )

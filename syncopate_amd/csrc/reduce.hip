@@ -1,0 +1,113 @@
+// Chunked ring reduce of GEMM+RS for gfx950 (tests/test_gemm_rs.py:22-72 of the reference):
+//   out[e] = local[rank*chunk + e] + sum_{i=1..W-1} recv[((rank+i) % W)*chunk + e]
+// A pure HBM stream: W reads and one write of 16 bytes per lane, all W loads of
+// an element group issued before the first add so that each lane keeps W
+// 128-bit requests in flight.
+#include "common.h"
+
+namespace syn {
+
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kReduceThreads = 256;
+constexpr int kMaxWorld = 16;
+
+template <typename T>
+__device__ __forceinline__ float to_f32(T x) { return (float)x; }
+
+template <typename T, bool ROUND_EACH>
+__device__ __forceinline__ u32x4_t add8(const u32x4_t* parts, int count) {
+    typedef T vec8 __attribute__((ext_vector_type(8)));
+    float acc[8];
+    {
+        const vec8 v = __builtin_bit_cast(vec8, parts[0]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = (float)v[e];
+    }
+    for (int i = 1; i < count; ++i) {
+        const vec8 v = __builtin_bit_cast(vec8, parts[i]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            float s = acc[e] + (float)v[e];
+            // fp32 add followed by round-to-nearest-even equals a correctly
+            // rounded add in the 16-bit type (both operands have <= 11 bits)
+            if (ROUND_EACH) s = (float)(T)s;
+            acc[e] = s;
+        }
+    }
+    vec8 r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] = (T)acc[e];
+    return __builtin_bit_cast(u32x4_t, r);
+}
+
+template <typename T, bool ROUND_EACH, int W>
+__global__ void __launch_bounds__(kReduceThreads)
+ring_reduce_kernel(const u32x4_t* __restrict__ recv, const u32x4_t* __restrict__ local,
+                   u32x4_t* __restrict__ out, int world, int rank, int64_t chunk_vecs) {
+    // W > 0: world known at compile time (fully unrolled loads); W == 0: generic
+    const int w = W > 0 ? W : world;
+    const int64_t stride = (int64_t)gridDim.x * kReduceThreads;
+    for (int64_t v = (int64_t)blockIdx.x * kReduceThreads + threadIdx.x; v < chunk_vecs; v += stride) {
+        u32x4_t parts[W > 0 ? W : kMaxWorld];
+        parts[0] = __builtin_nontemporal_load(local + (int64_t)rank * chunk_vecs + v);
+#pragma unroll
+        for (int i = 1; i < (W > 0 ? W : kMaxWorld); ++i) {
+            if (i < w) {
+                int src = rank + i;
+                if (src >= w) src -= w;
+                parts[i] = __builtin_nontemporal_load(recv + (int64_t)src * chunk_vecs + v);
+            }
+        }
+        const u32x4_t r = add8<T, ROUND_EACH>(parts, w);
+        __builtin_nontemporal_store(r, out + v);
+    }
+}
+
+template <typename T, bool ROUND_EACH>
+static int launch_reduce(const void* recv, const void* local, void* out, int world, int rank,
+                         int64_t chunk_vecs, hipStream_t stream) {
+    // one 16-byte group per lane and pass; enough workgroups to cover the chunk
+    // up to 16 per CU, beyond that lanes loop
+    int64_t blocks = (chunk_vecs + kReduceThreads - 1) / kReduceThreads;
+    const int64_t cap = 256 * 16;
+    if (blocks > cap) blocks = cap;
+    if (blocks < 1) blocks = 1;
+    const dim3 grid((unsigned)blocks), block(kReduceThreads);
+    const u32x4_t* r = reinterpret_cast<const u32x4_t*>(recv);
+    const u32x4_t* l = reinterpret_cast<const u32x4_t*>(local);
+    u32x4_t* o = reinterpret_cast<u32x4_t*>(out);
+    switch (world) {
+        case 2: hipLaunchKernelGGL((ring_reduce_kernel<T, ROUND_EACH, 2>), grid, block, 0, stream, r, l, o, world, rank, chunk_vecs); break;
+        case 4: hipLaunchKernelGGL((ring_reduce_kernel<T, ROUND_EACH, 4>), grid, block, 0, stream, r, l, o, world, rank, chunk_vecs); break;
+        case 8: hipLaunchKernelGGL((ring_reduce_kernel<T, ROUND_EACH, 8>), grid, block, 0, stream, r, l, o, world, rank, chunk_vecs); break;
+        default: hipLaunchKernelGGL((ring_reduce_kernel<T, ROUND_EACH, 0>), grid, block, 0, stream, r, l, o, world, rank, chunk_vecs); break;
+    }
+    return (int)hipGetLastError();
+}
+
+}  // namespace syn
+
+extern "C" int syn_ring_reduce(const void* recv, const void* local, void* out, int32_t world,
+                               int32_t rank, int64_t rows_per_rank, int64_t N, int32_t dtype,
+                               int32_t acc_mode, syn_stream_t stream) {
+    using namespace syn;
+    if (!recv || !local || !out) return SYN_EINVAL;
+    if (world < 1 || world > kMaxWorld || rank < 0 || rank >= world) return SYN_EINVAL;
+    if (rows_per_rank <= 0 || N <= 0) return SYN_EINVAL;
+    if (acc_mode != 0 && acc_mode != 1) return SYN_EINVAL;
+    const int64_t elems = rows_per_rank * N;
+    if (elems % 8) return SYN_EALIGN;
+    if (!aligned16(recv) || !aligned16(local) || !aligned16(out)) return SYN_EALIGN;
+    const int64_t vecs = elems / 8;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (dtype == SYN_DTYPE_BF16) {
+        return acc_mode == 0 ? launch_reduce<__bf16, true>(recv, local, out, world, rank, vecs, s)
+                             : launch_reduce<__bf16, false>(recv, local, out, world, rank, vecs, s);
+    }
+    if (dtype == SYN_DTYPE_FP16) {
+        return acc_mode == 0 ? launch_reduce<_Float16, true>(recv, local, out, world, rank, vecs, s)
+                             : launch_reduce<_Float16, false>(recv, local, out, world, rank, vecs, s);
+    }
+    return SYN_EINVAL;
+}

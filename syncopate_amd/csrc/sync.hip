@@ -1,0 +1,70 @@
+// Stream-side primitives of the single-GPU producer: the counterparts of the
+// reference runtime's cudaMemcpyAsync, cuStreamWriteValue and cuStreamWaitValue
+// (syncopate/communication/comm_runtime/communication_context.py:129-160),
+// written as one-wavefront kernels so they order with the copies on a stream.
+#include "common.h"
+
+namespace syn {
+
+__global__ void __launch_bounds__(64) flag_set_kernel(uint64_t* flag, uint64_t value) {
+    if (threadIdx.x == 0)
+        __hip_atomic_store(flag, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+__global__ void __launch_bounds__(64)
+flag_wait_kernel(const uint64_t* flag, uint64_t value, int64_t budget_ticks, int32_t* status) {
+    if (threadIdx.x == 0) {
+        if (!spin_until_equal(flag, value, budget_ticks))
+            report_status(status, SYN_STATUS_SPIN_TIMEOUT, -1, -1, -1);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+}
+
+__global__ void __launch_bounds__(64) delay_kernel(int64_t ticks) {
+    if (threadIdx.x == 0) {
+        const uint64_t t0 = wall_clock64();
+        while ((int64_t)(wall_clock64() - t0) < ticks) __builtin_amdgcn_s_sleep(16);
+    }
+}
+
+}  // namespace syn
+
+extern "C" {
+
+int syn_copy_async(void* dst, const void* src, int64_t nbytes, syn_stream_t stream) {
+    if (nbytes < 0 || (nbytes > 0 && (!dst || !src))) return SYN_EINVAL;
+    if (nbytes == 0) return 0;
+    return (int)hipMemcpyAsync(dst, src, (size_t)nbytes, hipMemcpyDeviceToDevice,
+                               reinterpret_cast<hipStream_t>(stream));
+}
+
+int syn_flag_set(uint64_t* flag, uint64_t value, syn_stream_t stream) {
+    if (!flag) return SYN_EINVAL;
+    hipLaunchKernelGGL(syn::flag_set_kernel, dim3(1), dim3(64), 0,
+                       reinterpret_cast<hipStream_t>(stream), flag, value);
+    return (int)hipGetLastError();
+}
+
+int syn_flag_wait(const uint64_t* flag, uint64_t value, int64_t spin_timeout_us, int32_t* status,
+                  syn_stream_t stream) {
+    if (!flag) return SYN_EINVAL;
+    hipLaunchKernelGGL(syn::flag_wait_kernel, dim3(1), dim3(64), 0,
+                       reinterpret_cast<hipStream_t>(stream), flag, value,
+                       syn::timeout_ticks(spin_timeout_us), status);
+    return (int)hipGetLastError();
+}
+
+int syn_delay_us(int64_t us, syn_stream_t stream) {
+    if (us < 0 || us > 1000000) return SYN_EINVAL;   // a delay is a model of link time, not a sleep
+    int dev = 0, khz = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess || khz <= 0)
+        khz = 100000;
+    hipLaunchKernelGGL(syn::delay_kernel, dim3(1), dim3(64), 0,
+                       reinterpret_cast<hipStream_t>(stream), us * (int64_t)khz / 1000);
+    return (int)hipGetLastError();
+}
+
+int syn_version(void) { return 100; }
+
+}  // extern "C"

@@ -1,0 +1,104 @@
+"""GPU parity of the chunked-KV flash attention against the CPU oracle (through the C ABI)."""
+
+import pytest
+import torch
+
+from oracle import numerics, visit_order
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-2
+
+
+def _qkv(Z, H, Sq, Skv, dtype, seed=0):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    q = torch.randn(Z, H, Sq, 128, generator=g).to(dtype)
+    k = torch.randn(Z, H, Skv, 128, generator=g).to(dtype)
+    v = torch.randn(Z, H, Skv, 128, generator=g).to(dtype)
+    return q, k, v
+
+
+def _kv_waves(Z, H, Sq, chunks, signals):
+    """One wave per kv chunk (element units), all of q against it."""
+    offsets, sizes, cums, total = [], [], [], 0
+    for lo, hi in chunks:
+        offsets.append([0, 0, 0, lo])
+        sizes.append([Z, H, Sq, hi - lo])
+        total += Z * H * Sq
+        cums.append(total)
+    return offsets, sizes, cums, list(signals), total
+
+
+def _rel(out, ref):
+    return ((out.float().cpu() - ref).abs().max() / ref.abs().max()).item()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("num_programs", [0, 5])
+def test_chunked_kv_matches_sdpa_and_oracle(hip, dtype, num_programs):
+    from syncopate_amd.computation.attn import attention_forward
+    from syncopate_amd.computation._launch import check_status
+
+    Z, H, Sq, Skv = 1, 3, 256, 1024
+    q, k, v = _qkv(Z, H, Sq, Skv, dtype)
+    chunks = [(512, 768), (0, 256), (768, 1024), (256, 512)]          # arrival order
+    offsets, sizes, cums, signals, total = _kv_waves(Z, H, Sq, chunks, [-1, 0, 1, 2])
+    flags = torch.ones(3, dtype=torch.int64, device="cuda")
+    sm_scale = 128 ** -0.5
+    log = torch.full((total // 128, 8), -1, dtype=torch.int32, device="cuda")
+    o, lse = attention_forward(q.cuda(), k.cuda(), v.cuda(), sm_scale, wave_offsets=offsets,
+                               wave_sizes=sizes, cum_wave_sizes=cums, signal_ptr=flags,
+                               signal_offsets=signals, NUM_WAVES=4, cum_tiles=total,
+                               num_programs=num_programs, return_lse=True, visit_log=log)
+    check_status()
+    ref = numerics.sdpa_fp32(q, k, v, sm_scale)
+    assert _rel(o, ref) <= REL_TOL
+    want_o, want_lse = numerics.chunked_attention(q, k, v, sm_scale, chunks)
+    assert _rel(o, want_o.float()) <= REL_TOL
+    assert (lse.cpu() - want_lse).abs().max().item() <= 2e-2
+    # lse2 is the base-2 log-sum-exp of the scaled scores
+    s = (q.float() @ k.float().transpose(-1, -2)) * sm_scale
+    assert (lse.cpu() - torch.logsumexp(s, dim=-1) / 0.6931471805599453).abs().max().item() <= 2e-2
+    rows = log.cpu().tolist()
+    for t, got in enumerate(rows):
+        w = visit_order.attn_tile_work(t, offsets, sizes, cums, signals)
+        assert got[:7] == [w["wave"], w["z"], w["h"], w["q_block"], w["kv_lo"], w["kv_hi"], w["signal"]]
+
+
+def test_causal_extension_matches_sdpa(hip):
+    from syncopate_amd.computation.attn import attention_forward
+    from syncopate_amd.computation._launch import check_status
+
+    Z, H, S = 2, 2, 512
+    q, k, v = _qkv(Z, H, S, S, torch.bfloat16, seed=4)
+    chunks = [(0, 128), (128, 384), (384, 512)]
+    offsets, sizes, cums, signals, total = _kv_waves(Z, H, S, chunks, [-1, -1, -1])
+    flags = torch.ones(1, dtype=torch.int64, device="cuda")
+    for scale in (128 ** -0.5, 1.0):
+        o = attention_forward(q.cuda(), k.cuda(), v.cuda(), scale, wave_offsets=offsets, wave_sizes=sizes,
+                              cum_wave_sizes=cums, signal_ptr=flags, signal_offsets=signals,
+                              cum_tiles=total, causal=True)
+        check_status()
+        ref = numerics.sdpa_fp32(q, k, v, scale, causal=True)
+        assert _rel(o, ref) <= REL_TOL
+
+
+def test_hand_template_form_resident(hip):
+    """attention(q, k, v, sm_scale, wave_dicts) with the everything-resident table
+    (reference: syncopate/computation/attn/template.py:442-497, kv_divide waves)."""
+    from syncopate_amd.computation.attn import attention, build_waves_and_signals_divisible
+    from syncopate_amd.computation._launch import check_status
+
+    Z, H, N_CTX = 2, 2, 768
+    g = torch.Generator(device="cpu").manual_seed(20)
+    q = (0.5 * torch.randn(Z, H, N_CTX, 128, generator=g)).half()
+    k = (0.5 * torch.randn(Z, H, N_CTX, 128, generator=g)).half()
+    v = (0.5 * torch.randn(Z, H, N_CTX, 128, generator=g)).half()
+    wave_dicts = build_waves_and_signals_divisible(Z, H, N_CTX, N_CTX, w=3)
+    assert wave_dicts["CUM_CHUNK_BLOCK"] == 4
+    o = attention(q.cuda(), k.cuda(), v.cuda(), 0.5, wave_dicts)
+    check_status()
+    p = torch.softmax((q.float() @ k.float().transpose(2, 3)) * 0.5, dim=-1)
+    ref = p @ v.float()
+    torch.testing.assert_close(o.float().cpu(), ref, atol=5e-2, rtol=0)   # the reference's bound (:486)
+    assert _rel(o, ref) <= REL_TOL

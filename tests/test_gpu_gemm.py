@@ -1,0 +1,200 @@
+"""GPU parity of the chunk-scheduled GEMM kernels against the CPU oracle (through the C ABI)."""
+
+import pytest
+import torch
+
+from oracle import numerics, visit_order
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-2  # max |err| / max |ref| against torch fp32, the bound the path is specified to
+
+
+def _inputs(M, N, K, dtype, seed=0, scale=0.02):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    a = (scale * torch.randn(M, K, generator=g)).to(dtype)
+    b = (scale * torch.randn(N, K, generator=g)).to(dtype)
+    return a, b
+
+
+def _row_waves(M, N, world, rank):
+    """AG-GEMM wave table of `rank`: chunk (rank+k) % world arrives k-th, flag k-1."""
+    rows = M // world
+    sizes = [[rows, N] for _ in range(world)]
+    offsets = [[((rank + k) % world) * rows, 0] for k in range(world)]
+    signals = [-1] + list(range(world - 1))
+    return sizes, offsets, signals
+
+
+def _max_rel_err(out, ref):
+    return ((out.float().cpu() - ref).abs().max() / ref.abs().max()).item()
+
+
+def _check_visits(log, sizes, offsets, signals, M, N, BM, BN, group_m, num_sms, cum_tiles, remap):
+    from syncopate_amd.computation._launch import check_status  # noqa: F401
+
+    want = visit_order.gemm_tile_visits(sizes, offsets, signals, M=M, N=N, BM=BM, BN=BN,
+                                        group_m=group_m, num_sms=num_sms, cum_tiles=cum_tiles)
+    got = log.cpu().view(-1, 4).tolist()
+    assert len(got) >= len(want)
+    for v in want:
+        pid, wave, pm, pn = got[v["tile_id"]]
+        assert (pid, wave, pm, pn) == (v["pid"], v["wave"], v["pid_m"], v["pid_n"]), v
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("BM,BN", [(128, 128), (128, 256), (256, 128), (256, 256)])
+def test_consumer_resident_matches_fp32_and_visit_order(hip, dtype, BM, BN):
+    from syncopate_amd.computation.gemm import gemm_consumer
+    from syncopate_amd.computation._launch import check_status
+
+    M, N, K, world, rank = 2048, 1024, 512, 4, 1
+    a, b = _inputs(M, N, K, dtype)
+    sizes, offsets, signals = _row_waves(M, N, world, rank)
+    ref = numerics.gemm_fp32(a, b)
+    ad, bd = a.cuda(), b.cuda()
+    c = torch.zeros(M, N, dtype=dtype, device="cuda")
+    flags = torch.ones(world, dtype=torch.int64, device="cuda")
+    tiles = (M // BM) * (N // BN)
+    for num_sms, remap in [(256, True), (24, False), (7, True)]:
+        c.zero_()
+        log = torch.full((tiles, 4), -1, dtype=torch.int32, device="cuda")
+        gemm_consumer(ad, bd, c, flags, sizes, offsets, signals, world, num_sms, BM, BN, 64, 8,
+                      cum_tiles=M * N, visit_log=log, xcd_remap=remap)
+        check_status()
+        assert _max_rel_err(c, ref) <= REL_TOL
+        _check_visits(log, sizes, offsets, signals, M, N, BM, BN, 8, num_sms, M * N, remap)
+
+
+def test_consumer_group_size_and_column_waves(hip):
+    """Waves that split N as well as M, ragged groups (GROUP_SIZE_M does not divide the wave)."""
+    from syncopate_amd.computation.gemm import gemm
+    from syncopate_amd.computation._launch import check_status
+
+    M, N, K, BM, BN = 1536, 1024, 256, 128, 128
+    a, b = _inputs(M, N, K, torch.bfloat16, seed=3)
+    ref = numerics.gemm_fp32(a, b)
+    sizes = [[640, 512], [896, 512], [640, 512], [896, 512]]
+    offsets = [[0, 512], [640, 0], [0, 0], [640, 512]]
+    signals = [1, -1, 0, 2]
+    cum = sum(s[0] * s[1] for s in sizes)
+    assert cum == M * N
+    flags = torch.ones(3, dtype=torch.int64, device="cuda")
+    c = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
+    for group_m, num_sms in [(3, 17), (8, 256), (1, 5)]:
+        c.zero_()
+        log = torch.full((cum // (BM * BN), 4), -1, dtype=torch.int32, device="cuda")
+        gemm(a.cuda(), b.cuda(), c, 1, num_sms, BM, BN, 64, group_m, cur_wave_sizes=sizes,
+             wave_offsets=offsets, signal_ptr=flags, signal_offsets=signals, cum_tiles=cum,
+             visit_log=log)
+        check_status()
+        assert _max_rel_err(c, ref) <= REL_TOL
+        _check_visits(log, sizes, offsets, signals, M, N, BM, BN, group_m, num_sms, cum, True)
+
+
+def test_consumer_gated_by_side_stream_producer(hip):
+    """Chunks land in the symmetric buffer on a side stream (copy, then flag) while the
+    consumer is already running; the result must be bitwise the resident one."""
+    from syncopate_amd import _lib
+    from syncopate_amd.computation.gemm import gemm_consumer
+    from syncopate_amd.computation._launch import check_status
+
+    M, N, K, world, rank, BM, BN = 4096, 1024, 1024, 8, 3, 128, 256
+    a, b = _inputs(M, N, K, torch.bfloat16, seed=5)
+    sizes, offsets, signals = _row_waves(M, N, world, rank)
+    staged = a.cuda()
+    bd = b.cuda()
+    flags = torch.ones(world - 1, dtype=torch.int64, device="cuda")
+    c_res = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
+    gemm_consumer(staged, bd, c_res, flags, sizes, offsets, signals, world, 200, BM, BN, cum_tiles=M * N)
+    torch.cuda.synchronize()
+
+    rows = M // world
+    symm = torch.full((M, K), float("nan"), dtype=torch.bfloat16, device="cuda")   # poison
+    symm[rank * rows:(rank + 1) * rows].copy_(staged[rank * rows:(rank + 1) * rows])
+    flags.zero_()
+    c = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    main = torch.cuda.current_stream()
+    side.wait_stream(main)
+    # consumer first, with head-room of 56 CUs for the copies
+    gemm_consumer(symm, bd, c, flags, sizes, offsets, signals, world, 200, BM, BN, cum_tiles=M * N,
+                  spin_timeout_us=3_000_000)
+    nbytes = rows * K * 2
+    for k in range(1, world):
+        chunk = (rank + k) % world
+        _lib.check("syn_delay_us", hip.syn_delay_us(200, _lib.stream_handle(side)))
+        _lib.check("syn_copy_async", hip.syn_copy_async(symm.data_ptr() + chunk * nbytes,
+                                                        staged.data_ptr() + chunk * nbytes, nbytes,
+                                                        _lib.stream_handle(side)))
+        _lib.check("syn_flag_set", hip.syn_flag_set(flags.data_ptr() + 8 * (k - 1), 1,
+                                                    _lib.stream_handle(side)))
+    main.wait_stream(side)
+    check_status()
+    assert flags.tolist() == [1] * (world - 1)
+    assert torch.equal(c, c_res)
+    assert _max_rel_err(c, numerics.gemm_fp32(a, b)) <= REL_TOL
+
+
+def test_consumer_flag_never_set_times_out_cleanly(hip):
+    from syncopate_amd.computation.gemm import gemm_consumer
+    from syncopate_amd.computation._launch import FlagWaitTimeout, check_status
+
+    M, N, K, world = 512, 256, 128, 2
+    a, b = _inputs(M, N, K, torch.bfloat16)
+    sizes, offsets, signals = _row_waves(M, N, world, 0)
+    flags = torch.zeros(1, dtype=torch.int64, device="cuda")
+    c = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
+    gemm_consumer(a.cuda(), b.cuda(), c, flags, sizes, offsets, signals, world, 64, 128, 128,
+                  cum_tiles=M * N, spin_timeout_us=20_000)
+    with pytest.raises(FlagWaitTimeout):
+        check_status()
+    check_status()  # status words were reset
+
+
+def test_bad_tables_are_rejected_before_launch(hip):
+    from syncopate_amd import _lib
+    from syncopate_amd.computation.gemm import gemm_consumer
+
+    M, N, K = 512, 256, 128
+    a, b = _inputs(M, N, K, torch.bfloat16)
+    c = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
+    flags = torch.ones(1, dtype=torch.int64, device="cuda")
+    cases = [
+        ([[256, 256], [256, 256]], [[0, 0], [512, 0]], [-1, 0]),   # rows beyond M
+        ([[256, 256], [256, 256]], [[0, 0], [256, 0]], [-1, 1]),   # flag index beyond the array
+        ([[256, 256], [200, 256]], [[0, 0], [256, 0]], [-1, 0]),   # not a multiple of the block
+        ([[256, 256]], [[0, 0]], [-1]),                            # covers half of cum_tiles
+    ]
+    for sizes, offsets, signals in cases:
+        with pytest.raises(_lib.SyncopateHipError):
+            gemm_consumer(a.cuda(), b.cuda(), c, flags, sizes, offsets, signals, 2, 64, 128, 128,
+                          cum_tiles=M * N)
+
+
+@pytest.mark.parametrize("BM,BN", [(128, 256), (256, 256)])
+def test_producer_counters_flags_and_result(hip, BM, BN):
+    """GEMM+RS producer: wave order (r+1..r+W-1, r), every counter == tiles of its wave,
+    every flag == 1 (reference: tests/computation/gemm/test_gemm_producer.py:34-36)."""
+    from syncopate_amd.computation.gemm import gemm_producer
+
+    M, N, K, world, rank = 2048, 1024, 512, 8, 2
+    a, b = _inputs(M, N, K, torch.bfloat16, seed=7)
+    rows = M // world
+    order = [(rank + k + 1) % world for k in range(world)]
+    sizes = [[rows, N]] * world
+    offsets = [[ch * rows, 0] for ch in order]
+    signals = list(range(world))
+    flags = torch.zeros(world, dtype=torch.int64, device="cuda")
+    counters = torch.zeros(world, dtype=torch.int32, device="cuda")
+    c = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
+    log = torch.full(((M // BM) * (N // BN), 4), -1, dtype=torch.int32, device="cuda")
+    gemm_producer(a.cuda(), b.cuda(), c, flags, sizes, offsets, signals, 256, BM, BN,
+                  cum_tiles=M * N, counter_buffer=counters, visit_log=log)
+    torch.cuda.synchronize()
+    per_wave = (rows // BM) * (N // BN)
+    assert counters.tolist() == [per_wave] * world
+    assert flags.tolist() == [1] * world
+    assert _max_rel_err(c, numerics.gemm_fp32(a, b)) <= REL_TOL
+    _check_visits(log, sizes, offsets, signals, M, N, BM, BN, 8, 256, M * N, True)

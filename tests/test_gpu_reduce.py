@@ -1,0 +1,70 @@
+"""GPU parity of the chunked ring reduce against the CPU oracle: bit-exact."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import numerics
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(world, rows, N, dtype, seed):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    recv = torch.randn(world, rows, N, generator=g).to(dtype)
+    local = torch.randn(world * rows, N, generator=g).to(dtype)
+    return recv, local
+
+
+@pytest.mark.parametrize("dtype,name", [(torch.bfloat16, "bf16"), (torch.float16, "fp16")])
+@pytest.mark.parametrize("world,rows,N", [(8, 128, 512), (4, 64, 256), (2, 8, 8), (3, 40, 72),
+                                           (16, 16, 128), (1, 16, 64)])
+@pytest.mark.parametrize("acc_mode", ["dtype", "fp32"])
+def test_ring_reduce_bit_exact(hip, dtype, name, world, rows, N, acc_mode):
+    from syncopate_amd.computation.reduce import ring_reduce
+
+    for rank in sorted({0, world - 1, world // 2}):
+        recv, local = _case(world, rows, N, dtype, seed=world * 100 + rank)
+        want = numerics.ring_reduce(recv.float().numpy(), local.float().numpy(), rank, dtype=name,
+                                    round_each_add=(acc_mode == "dtype"))
+        recv_d = recv.cuda()
+        # the slot of the rank itself is never read: poison it
+        recv_d[rank].fill_(float("nan"))
+        out = torch.empty(rows, N, dtype=dtype, device="cuda")
+        ring_reduce(recv_d, out, local.cuda(), rank, acc_mode=acc_mode)
+        got = out.float().cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_ring_reduce_full_size_properties(hip):
+    """BASELINE size (8 x (1024, 8192) bf16): integer-valued inputs make every partial sum
+    exact, so the result must equal the integer sum whatever the order or rounding."""
+    from syncopate_amd.computation.reduce import ring_reduce
+
+    world, rows, N, rank = 8, 1024, 8192, 5
+    g = torch.Generator(device="cpu").manual_seed(11)
+    recv = torch.randint(-8, 9, (world, rows, N), generator=g).to(torch.bfloat16)
+    local = torch.randint(-8, 9, (world * rows, N), generator=g).to(torch.bfloat16)
+    want = local[rank * rows:(rank + 1) * rows].float()
+    for i in range(1, world):
+        want = want + recv[(rank + i) % world].float()
+    out = torch.empty(rows, N, dtype=torch.bfloat16, device="cuda")
+    for mode in ("dtype", "fp32"):
+        ring_reduce(recv.cuda(), out, local.cuda(), rank, acc_mode=mode)
+        assert torch.equal(out.float().cpu(), want)
+
+
+def test_ring_reduce_rejects_bad_arguments(hip):
+    from syncopate_amd import _lib
+    from syncopate_amd.computation.reduce import ring_reduce
+
+    recv = torch.zeros(4, 3, 5, dtype=torch.bfloat16, device="cuda")     # 15 elements: not 8-divisible
+    local = torch.zeros(12, 5, dtype=torch.bfloat16, device="cuda")
+    out = torch.zeros(3, 5, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(_lib.SyncopateHipError):
+        ring_reduce(recv, out, local, 0)
+    recv = torch.zeros(4, 8, 8, dtype=torch.bfloat16, device="cuda")
+    local = torch.zeros(32, 8, dtype=torch.bfloat16, device="cuda")
+    out = torch.zeros(8, 8, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(_lib.SyncopateHipError):
+        ring_reduce(recv, out, local, 4)                                  # rank out of range
