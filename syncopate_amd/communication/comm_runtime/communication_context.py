@@ -1,0 +1,190 @@
+"""Single-GPU executor of a CommInfo: replays one rank's op list on side streams.
+
+Counterpart of the reference runtime
+(syncopate/communication/comm_runtime/communication_context.py: `__init__`
+:31-76, `reset_signals` :90-96, `start_after`/`end_before` :98-106, `execute`
+:108-235, `get_graph` :242-249), with the other ranks simulated on the same
+MI355X: every rank's "symmetric" buffers and flag arrays are ordinary device
+tensors of this process, a cross-rank copy is a hipMemcpyAsync between two of
+them, a flag write is a one-wavefront kernel doing a system-scope release
+store and a flag wait is a one-wavefront kernel spinning (with a time-out) on
+the word.  Only the ops of `rank` are executed, in exactly the order the op
+list prescribes, so a consumer kernel launched on the compute stream really
+overlaps with data arriving chunk by chunk.
+
+On a multi-GPU node the same op list would be replayed with the peers'
+buffers mapped through IPC and one stream per peer link; that path is not
+built here.
+"""
+
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from ... import _lib
+from ..descriptor import ReduceOp, SignalType
+from .operations import (
+    CollectiveComm,
+    CommInfo,
+    CopyEngineOp,
+    IntraNodeSignal,
+    SMCopyOp,
+    WaitIntraNodeSignal,
+)
+
+SIGNAL_DTYPE = torch.int64   # 8-byte flag words, value 1 = set
+
+
+class CommContext:
+    rank: int
+    info: CommInfo
+    recv_signal_bufs: List[torch.Tensor]
+    transit_signal_bufs: List[torch.Tensor]
+    compute_signal_bufs: List[torch.Tensor]
+    comm_buffers: Dict[str, List[torch.Tensor]]
+    streams: List[torch.cuda.Stream]
+
+    def __init__(self, rank: int, info: CommInfo, multi_info: bool = False, *,
+                 device: Optional[torch.device] = None, link_delay_us: int = 0,
+                 wait_timeout_us: int = 2_000_000) -> None:
+        if info.local_world_size <= 0:
+            info.local_world_size = info.world_size
+        if info.local_world_size != info.world_size:
+            raise NotImplementedError("the single-GPU executor simulates one node: "
+                                      "local_world_size must equal world_size")
+        if not 0 <= rank < info.world_size:
+            raise ValueError(f"rank {rank} outside world of {info.world_size}")
+        self.rank = rank
+        self.local_rank = rank % info.local_world_size
+        self.node_id = rank // info.local_world_size
+        self.info = info
+        self.device = torch.device("cuda", torch.cuda.current_device()) if device is None else device
+        self.link_delay_us = int(link_delay_us)
+        self.wait_timeout_us = int(wait_timeout_us)
+        self._lib = _lib.load()
+        world = info.local_world_size
+
+        def flag_arrays(count: int) -> List[torch.Tensor]:
+            if count <= 0:
+                return []
+            return [torch.zeros((count,), dtype=SIGNAL_DTYPE, device=self.device) for _ in range(world)]
+
+        self.recv_signal_bufs = flag_arrays(info.recv_signal_num)
+        self.transit_signal_bufs = flag_arrays(info.transit_signal_num)
+        self.compute_signal_bufs = flag_arrays(info.compute_signal_num)
+        self.comm_buffers = {
+            name: [torch.zeros(tuple(shape), dtype=dtype, device=self.device) for _ in range(world)]
+            for name, (shape, dtype) in info.comm_buffer_sizes.items()
+        }
+        self.status = torch.zeros(_lib.SYN_STATUS_WORDS, dtype=torch.int32, device=self.device)
+        self.streams = [torch.cuda.Stream(device=self.device) for _ in info.operations[self.rank]]
+        self.compute_stream = None
+
+    # ---- flags and stream ordering -------------------------------------------
+
+    def reset_signals(self) -> None:
+        for group in (self.recv_signal_bufs, self.transit_signal_bufs, self.compute_signal_bufs):
+            if group:
+                group[self.local_rank].fill_(0)
+
+    def start_after(self, stream: Optional[torch.cuda.Stream] = None) -> None:
+        """Communication streams start once `stream` has reached this point."""
+        stream = torch.cuda.current_stream(self.device) if stream is None else stream
+        for comm_stream in self.streams:
+            comm_stream.wait_stream(stream)
+
+    def end_before(self, stream: Optional[torch.cuda.Stream] = None) -> None:
+        """`stream` continues only after all communication streams have drained."""
+        stream = torch.cuda.current_stream(self.device) if stream is None else stream
+        for comm_stream in self.streams:
+            stream.wait_stream(comm_stream)
+
+    # ---- replay --------------------------------------------------------------
+
+    def _flags(self, signal_type: SignalType, rank: int) -> torch.Tensor:
+        if signal_type == SignalType.COMPUTE_DONE:
+            return self.compute_signal_bufs[rank]
+        if signal_type == SignalType.RECEIVE_DATA:
+            return self.recv_signal_bufs[rank]
+        raise NotImplementedError(f"Signal type {signal_type} not implemented yet.")
+
+    def execute(self, neglect_local: bool = False) -> None:
+        """Enqueue this rank's ops, stream by stream, in list order."""
+        lib = self._lib
+        world = self.info.local_world_size
+        for stream, ops in zip(self.streams, self.info.operations[self.rank]):
+            handle = int(stream.cuda_stream)
+            for op in ops:
+                if isinstance(op, CopyEngineOp):
+                    assert op.src_rank == self.rank or op.dst_rank == self.rank
+                    if op.src_rank == op.dst_rank and neglect_local:
+                        continue
+                    src = self.comm_buffers[op.src][op.src_rank % world]
+                    dst = self.comm_buffers[op.dst][op.dst_rank % world]
+                    assert src.is_contiguous() and dst.is_contiguous()
+                    nbytes_src = src.numel() * src.element_size()
+                    nbytes_dst = dst.numel() * dst.element_size()
+                    if op.src_offset + op.size > nbytes_src or op.dst_offset + op.size > nbytes_dst:
+                        raise ValueError(f"{op} runs past the end of its buffer")
+                    if self.link_delay_us and op.src_rank != op.dst_rank:
+                        _lib.check("syn_delay_us", lib.syn_delay_us(self.link_delay_us, handle))
+                    _lib.check("syn_copy_async",
+                               lib.syn_copy_async(dst.data_ptr() + op.dst_offset,
+                                                  src.data_ptr() + op.src_offset, op.size, handle))
+                elif isinstance(op, IntraNodeSignal):
+                    assert op.signal_type == SignalType.RECEIVE_DATA
+                    flags = self.recv_signal_bufs[op.rank % world]
+                    if not 0 <= op.offset < flags.numel():
+                        raise ValueError(f"{op} is outside the flag array")
+                    _lib.check("syn_flag_set", lib.syn_flag_set(flags.data_ptr() + 8 * op.offset, 1, handle))
+                elif isinstance(op, WaitIntraNodeSignal):
+                    flags = self._flags(op.signal_type, op.rank % world)
+                    if not 0 <= op.offset < flags.numel():
+                        raise ValueError(f"{op} is outside the flag array")
+                    _lib.check("syn_flag_wait",
+                               lib.syn_flag_wait(flags.data_ptr() + 8 * op.offset, 1, self.wait_timeout_us,
+                                                 self.status.data_ptr(), handle))
+                elif isinstance(op, SMCopyOp):
+                    assert op.src_rank == self.rank or op.dst_rank == self.rank
+                    if op.src_rank == op.dst_rank and neglect_local:
+                        continue
+                    src = self.comm_buffers[op.src][op.src_rank % world]
+                    dst = self.comm_buffers[op.dst][op.dst_rank % world]
+                    src_box = src[tuple(slice(ax.start, ax.end) for ax in op.src_slice)]
+                    dst_box = dst[tuple(slice(ax.start, ax.end) for ax in op.dst_slice)]
+                    with torch.cuda.stream(stream):
+                        if op.reduce_op is None:
+                            dst_box.copy_(src_box.reshape(dst_box.shape))
+                        elif op.reduce_op == ReduceOp.SUM:
+                            dst_box.add_(src_box.reshape(dst_box.shape))
+                        else:
+                            raise NotImplementedError(f"reduce op {op.reduce_op} in a box copy")
+                elif isinstance(op, CollectiveComm):
+                    raise NotImplementedError(
+                        "library collectives need the other ranks to be real processes; "
+                        "the single-GPU executor replays copy/flag op lists only")
+                else:
+                    raise TypeError(f"unknown op record {type(op).__name__}")
+
+    def check_status(self) -> None:
+        """Synchronise and raise if a stream-side flag wait gave up."""
+        torch.cuda.synchronize(self.device)
+        words = self.status.tolist()
+        if words[0] != 0:
+            self.status.zero_()
+            raise RuntimeError(f"communication stream flag wait timed out (status {words})")
+
+    def get_comm_sms(self) -> int:
+        return self.info.num_copy_sms
+
+    def get_graph(self) -> torch.cuda.CUDAGraph:
+        """Capture start_after / execute / end_before into a HIP graph.  The op list
+        consists of memcpy nodes and small kernels only (no memset nodes)."""
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            self.start_after(torch.cuda.current_stream(self.device))
+            self.execute()
+            self.end_before(torch.cuda.current_stream(self.device))
+        return graph

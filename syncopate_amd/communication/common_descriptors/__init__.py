@@ -1,0 +1,18 @@
+"""Plan builders for the collectives the chunk-scheduled kernels are fused with."""
+
+from .all_gather import (
+    build_all_gather_plan_1d_swizzle,
+    build_double_ring_all_gather_plan,
+    build_ring_all_gather_plan,
+)
+from .all_to_all import build_all_to_all_plan, build_all_to_all_plan_dim
+from .reduce_scatter import build_reduce_scatter_direct_reduce_plan
+
+__all__ = [
+    "build_all_gather_plan_1d_swizzle",
+    "build_ring_all_gather_plan",
+    "build_double_ring_all_gather_plan",
+    "build_all_to_all_plan",
+    "build_all_to_all_plan_dim",
+    "build_reduce_scatter_direct_reduce_plan",
+]
