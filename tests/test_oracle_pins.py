@@ -119,17 +119,18 @@ def test_attention_tile_work_covers_every_q_kv_pair_once():
 # ---------------------------------------------------------------- rounding and ring reduce
 
 def test_bf16_rounding_is_round_to_nearest_even():
-    x = np.array([1.0, 1.00390625, 1.01171875, 1.0078125 + 2 ** -9, -3.0e38, 1e-40], dtype=np.float32)
-    #                 tie -> even (down)   tie -> even (up)     above tie
-    want = np.array([1.0, 1.0, 1.015625, 1.015625, -3.0e38, 1e-40], dtype=np.float32)
-    got = numerics.round_to(x, "bf16")
-    assert got[0] == 1.0 and got[1] == 1.0 and got[2] == 1.015625 and got[3] == 1.015625
+    # bf16 has 8 significand bits: ulp(1.0) = 2^-7
+    x = np.array([1.0, 1 + 2.0 ** -8, 1 + 2.0 ** -7 + 2.0 ** -8, 1 + 2.0 ** -7 + 2.0 ** -9,
+                  1 + 2.0 ** -7 + 2.0 ** -8 + 2.0 ** -12], dtype=np.float32)
+    #             exact  tie -> even (down)  tie -> even (up)          below the tie
+    #             above the tie
+    want = np.array([1.0, 1.0, 1 + 2.0 ** -6, 1 + 2.0 ** -7, 1 + 2.0 ** -6], dtype=np.float32)
+    assert np.array_equal(numerics.round_to(x, "bf16"), want)
     rng = np.random.default_rng(1)
     r = (rng.standard_normal(200000) * np.exp(rng.uniform(-20, 20, 200000))).astype(np.float32)
     assert np.array_equal(numerics.round_to(r, "bf16"), torch.from_numpy(r).bfloat16().float().numpy())
     assert np.array_equal(numerics.round_to(r, "fp16")[np.abs(r) < 6e4],
                           torch.from_numpy(r).half().float().numpy()[np.abs(r) < 6e4])
-    assert want.dtype == np.float32
 
 
 @pytest.mark.parametrize("dtype,tdtype", [("bf16", torch.bfloat16), ("fp16", torch.float16)])
