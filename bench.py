@@ -1,0 +1,267 @@
+"""Benchmark of the chunk-scheduled AG+GEMM on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one fused all-gather+GEMM iteration of rank 0 of a simulated mesh of 8
+(BASELINE configuration 2): flags reset, the 7 peer chunks of A (1024 x 8192 bf16 each)
+copied into the symmetric buffer on a side stream in the order the lowered schedule
+prescribes (copy, then flag), the consumer GEMM (8192 x 8192 x 3584) on the compute stream
+waiting on each chunk's flag.  All operands are resident in HBM before the timed region.
+Prints ONE JSON line; see DESIGN.md for the meaning of every field.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+import torch  # noqa: E402
+
+MFMA_BF16_PEAK_TFLOPS = 2500.0      # MI355X dense bf16
+HBM_PEAK_GBPS = 8000.0
+
+# AG+GEMM, BASELINE configuration 2
+M, K, N, WORLD, RANK = 8192, 8192, 3584, 8, 0
+BM, BN, BK, GROUP_M = 256, 256, 64, 8
+NUM_SMS = 248                        # 8 of the 256 CUs stay free for the copy kernels of the producer
+
+
+def _events(n):
+    return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+
+
+def build_ag_gemm(device):
+    from syncopate_amd.communication.code_gen import CommGenerator
+    from syncopate_amd.communication.comm_runtime.communication_context import CommContext
+    from syncopate_amd.communication.common_descriptors import build_all_gather_plan_1d_swizzle
+    from syncopate_amd.interface import lower_comm_plan_to_raw_schedules
+    from syncopate_amd.interface.wave_tables import gemm_consumer_tables
+
+    t0 = time.perf_counter()
+    plans = {r: build_all_gather_plan_1d_swizzle((M, K), torch.bfloat16, 0, WORLD, r, "a", "pull")
+             for r in range(WORLD)}
+    gen = CommGenerator(plans)
+    gen.plan_signals()
+    schedule = lower_comm_plan_to_raw_schedules(gen)[RANK]["a"]
+    info = gen.generate_code_for_plan()
+    compile_ms = (time.perf_counter() - t0) * 1e3
+    info.local_world_size = info.world_size
+    tables = gemm_consumer_tables(schedule, N)
+
+    torch.manual_seed(0)
+    a = (0.02 * torch.randn(M, K, device=device)).bfloat16()
+    b = (0.02 * torch.randn(N, K, device=device)).bfloat16()
+    ctx = CommContext(RANK, info, device=device)
+    rows = M // WORLD
+    for r in range(WORLD):     # every rank's symmetric buffer holds its own shard
+        ctx.comm_buffers["a"][r][r * rows:(r + 1) * rows].copy_(a[r * rows:(r + 1) * rows])
+    dev_tables = dict(
+        cur_wave_sizes=torch.tensor(tables.block_shapes, dtype=torch.int32, device=device),
+        wave_offsets=torch.tensor(tables.block_offsets, dtype=torch.int32, device=device),
+        signal_offsets=torch.tensor(tables.signal_offsets, dtype=torch.int32, device=device),
+        cum_tiles=tables.cum_tiles,
+    )
+    c = torch.empty(M, N, dtype=torch.bfloat16, device=device)
+    return dict(a=a, b=b, c=c, ctx=ctx, tables=dev_tables, compile_ms=compile_ms)
+
+
+def run_ag_gemm(state, steps, warmup):
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.gemm import gemm
+
+    ctx, b, c, tables = state["ctx"], state["b"], state["c"], state["tables"]
+    symm = ctx.comm_buffers["a"][RANK]
+    flags = ctx.recv_signal_bufs[RANK]
+    stream = torch.cuda.current_stream()
+    rows = M // WORLD
+
+    def consumer(flag_words):
+        gemm(symm, b, c, WORLD, NUM_SMS, BM, BN, BK, GROUP_M, signal_ptr=flag_words, **tables)
+
+    def fused_step():
+        ctx.reset_signals()
+        ctx.start_after(stream)
+        ctx.execute()
+        consumer(flags)
+        ctx.end_before(stream)
+
+    # ---- gated run: the step the metric is quoted on ----
+    for _ in range(warmup):
+        fused_step()
+    torch.cuda.synchronize()
+    begin, end = _events(steps), _events(steps)
+    t0 = time.perf_counter()
+    for i in range(steps):
+        ctx.reset_signals()
+        ctx.start_after(stream)
+        ctx.execute()
+        begin[i].record(stream)
+        consumer(flags)
+        end[i].record(stream)
+        ctx.end_before(stream)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    gated_kernel_ms = sum(s.elapsed_time(e) for s, e in zip(begin, end)) / steps
+    check_status()
+    ctx.check_status()
+
+    # ---- same kernel, every chunk resident and every flag already set ----
+    resident_flags = torch.ones_like(flags)
+    for _ in range(warmup):
+        consumer(resident_flags)
+    torch.cuda.synchronize()
+    begin, end = _events(steps), _events(steps)
+    for i in range(steps):
+        begin[i].record(stream)
+        consumer(resident_flags)
+        end[i].record(stream)
+    torch.cuda.synchronize()
+    resident_kernel_ms = sum(s.elapsed_time(e) for s, e in zip(begin, end)) / steps
+    check_status()
+    return wall_ms, gated_kernel_ms, resident_kernel_ms
+
+
+def check_ag_gemm(state):
+    """Spot-check the last step's output against torch on the GPU (fp32 accumulate)."""
+    a, b, c = state["a"], state["b"], state["c"]
+    rows = torch.arange(0, M, 257, device=a.device)
+    ref = a[rows].float() @ b.float().t()
+    err = ((c[rows].float() - ref).abs().max() / ref.abs().max()).item()
+    gathered = torch.equal(state["ctx"].comm_buffers["a"][RANK], a)
+    return err, gathered
+
+
+def run_reduce(device, steps, warmup):
+    """GEMM+RS chunked reduce at BASELINE configuration 3: 8 x (1024, 8192) bf16 -> (1024, 8192)."""
+    from syncopate_amd.computation.reduce import ring_reduce
+
+    world, rows, n = 8, 1024, 8192
+    torch.manual_seed(1)
+    recv = torch.randn(world, rows, n, device=device).bfloat16()
+    local = torch.randn(world * rows, n, device=device).bfloat16()
+    out = torch.empty(rows, n, dtype=torch.bfloat16, device=device)
+    stream = torch.cuda.current_stream()
+    for _ in range(warmup):
+        ring_reduce(recv, out, local, RANK)
+    torch.cuda.synchronize()
+    begin, end = _events(steps), _events(steps)
+    for i in range(steps):
+        begin[i].record(stream)
+        ring_reduce(recv, out, local, RANK)
+        end[i].record(stream)
+    torch.cuda.synchronize()
+    ms = sum(s.elapsed_time(e) for s, e in zip(begin, end)) / steps
+    nbytes = (world + 1) * rows * n * 2          # 8 reads + 1 write of a (1024, 8192) bf16 block
+    return ms, nbytes
+
+
+def cpu_baseline(state):
+    """torch CPU matmul over the gathered operands (fp32 values of the same bf16 inputs):
+    a bounded sample of the same GEMM — a band of rows of A against all of B."""
+    from oracle import numerics
+
+    threads = min(16, os.cpu_count() or 1)
+    torch.set_num_threads(threads)
+    sample_rows = 1024
+    a = state["a"][:sample_rows].cpu()
+    b = state["b"].cpu()
+    numerics.gemm_fp32(a[:128], b)          # warm-up
+    reps, spent = 0, 0.0
+    while spent < 10.0 and reps < 8:
+        t0 = time.perf_counter()
+        numerics.gemm_fp32(a, b)
+        spent += time.perf_counter() - t0
+        reps += 1
+    flop = 2.0 * sample_rows * N * K * reps
+    return {
+        "value": flop / spent / 1e12,
+        "unit": "TFLOP/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"{reps} x torch CPU fp32 matmul of A[:{sample_rows}] (bf16 values) with all of B, "
+                  f"{spent:.1f} s",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one rank's share on ONE GPU: the other ranks of the mesh are "
+                 "simulated by a side-stream producer; run it with --gpus 1")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs the MI355X (no GPU visible)")
+    from syncopate_amd import _lib
+
+    _lib.load()      # fail loudly if the HIP library has not been built
+    device = torch.device("cuda", 0)
+    torch.cuda.set_device(device)
+
+    state = build_ag_gemm(device)
+    wall_ms, gated_ms, resident_ms = run_ag_gemm(state, args.steps, args.warmup)
+    err, gathered = check_ag_gemm(state)
+    reduce_ms, reduce_bytes = run_reduce(device, max(args.steps, 20), args.warmup)
+
+    flop = 2.0 * M * N * K
+    value = flop / (wall_ms * 1e-3) / 1e12
+    kernel_tflops = flop / (gated_ms * 1e-3) / 1e12
+    line = {
+        "metric": "AG-GEMM TFLOP/s",
+        "value": value,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": wall_ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": "AG-GEMM one rank's share, simulated mesh=8: A (8192,8192) bf16 arriving as 8 chunks "
+                        "of 1024 rows in swizzled order behind flags, B (8192,3584) bf16 stored [N,K], "
+                        "fp32 accumulate",
+            "tile": [BM, BN, BK],
+            "programs": NUM_SMS,
+            "producer": "side stream: hipMemcpyAsync + flag-set kernel per chunk",
+        },
+        "pct_bf16_mfma_peak": 100.0 * value / MFMA_BF16_PEAK_TFLOPS,
+        "flag_wait_overhead_pct": 100.0 * (gated_ms - resident_ms) / resident_ms,
+        "kernel_ms_gated": gated_ms,
+        "kernel_ms_resident": resident_ms,
+        "resident_tflops": flop / (resident_ms * 1e-3) / 1e12,
+        "rs_reduce_GBps": reduce_bytes / (reduce_ms * 1e-3) / 1e9,
+        "rs_reduce_us": reduce_ms * 1e3,
+        "rs_reduce_pct_hbm_peak": 100.0 * reduce_bytes / (reduce_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+        "host_compile_ms": state["compile_ms"],
+        "max_rel_err_vs_fp32": err,
+        "gathered_a_matches": gathered,
+        "roofline": {
+            "kernel": "gemm_wave_kernel<bf16,256,256,consumer>",
+            "bound": "mfma",
+            "achieved": kernel_tflops,
+            "peak": MFMA_BF16_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": kernel_tflops / MFMA_BF16_PEAK_TFLOPS,
+            "traffic": None,
+        },
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(state)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

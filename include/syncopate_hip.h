@@ -41,6 +41,9 @@ extern "C" {
 /* gemm option bits */
 #define SYN_GEMM_XCD_REMAP 1u       /* permute hardware workgroup ids so that consecutive
                                        logical program ids share an XCD (and its L2)      */
+#define SYN_GEMM_EIGHT_WAVES 2u     /* 512-thread workgroups (two wavefronts per SIMD)     */
+#define SYN_GEMM_PAIR_PIPE 4u       /* force the two-stage 64-deep pipeline (default: the
+                                       four-stage 32-deep ring whenever K % 128 == 0)      */
 
 typedef void* syn_stream_t;        /* hipStream_t */
 

@@ -24,6 +24,8 @@ SYN_EALIGN = -75
 SYN_STATUS_WORDS = 4
 SYN_STATUS_SPIN_TIMEOUT = 1
 SYN_GEMM_XCD_REMAP = 1
+SYN_GEMM_EIGHT_WAVES = 2
+SYN_GEMM_PAIR_PIPE = 4
 
 _ERRORS = {
     SYN_EINVAL: "SYN_EINVAL (malformed argument or unsupported configuration)",

@@ -52,6 +52,8 @@ def _launch(
     counter_buffer: Optional[torch.Tensor],
     visit_log: Optional[torch.Tensor],
     xcd_remap: bool,
+    eight_waves: bool,
+    pair_pipe: bool,
     spin_timeout_us: int,
     stream: Optional[torch.cuda.Stream],
 ) -> None:
@@ -130,7 +132,8 @@ def _launch(
         num_sms=num_gemm_sms,
         cum_tiles=int(cum_tiles),
         spin_timeout_us=int(spin_timeout_us),
-        options=_lib.SYN_GEMM_XCD_REMAP if xcd_remap else 0,
+        options=(_lib.SYN_GEMM_XCD_REMAP if xcd_remap else 0) | (_lib.SYN_GEMM_EIGHT_WAVES if eight_waves else 0)
+        | (_lib.SYN_GEMM_PAIR_PIPE if pair_pipe else 0),
     )
     with torch.cuda.device(dev):
         fn = lib.syn_gemm_producer if producer else lib.syn_gemm_consumer
@@ -157,6 +160,8 @@ def gemm_consumer(
     cum_tiles=0,
     visit_log=None,
     xcd_remap=True,
+    eight_waves=False,
+    pair_pipe=False,
     spin_timeout_us=DEFAULT_SPIN_TIMEOUT_US,
     stream=None,
 ):
@@ -172,7 +177,7 @@ def gemm_consumer(
     assert M_per_rank % BLOCK_SIZE_M == 0
     _launch(False, a, b, c, signal_buffer, cur_wave_size, wave_offset, signal_offsets, num_gemm_sms,
             BLOCK_SIZE_M, BLOCK_SIZE_N, BLOCK_SIZE_K, GROUP_SIZE_M, cum_tiles, None, visit_log,
-            xcd_remap, spin_timeout_us, stream)
+            xcd_remap, eight_waves, pair_pipe, spin_timeout_us, stream)
 
 
 def gemm_producer(
@@ -194,6 +199,8 @@ def gemm_producer(
     counter_buffer=None,
     visit_log=None,
     xcd_remap=True,
+    eight_waves=False,
+    pair_pipe=False,
     stream=None,
 ):
     """GEMM+RS producer: same GEMM; every finished tile bumps its wave's counter
@@ -203,7 +210,7 @@ def gemm_producer(
     """
     _launch(True, a, b, c, signal_buffer, cur_wave_size, wave_offset, signal_offsets, num_gemm_sms,
             BLOCK_SIZE_M, BLOCK_SIZE_N, BLOCK_SIZE_K, GROUP_SIZE_M, cum_tiles, counter_buffer,
-            visit_log, xcd_remap, DEFAULT_SPIN_TIMEOUT_US, stream)
+            visit_log, xcd_remap, eight_waves, pair_pipe, DEFAULT_SPIN_TIMEOUT_US, stream)
 
 
 def gemm(
@@ -226,6 +233,8 @@ def gemm(
     cum_tiles=0,
     visit_log=None,
     xcd_remap=True,
+    eight_waves=False,
+    pair_pipe=False,
     spin_timeout_us=DEFAULT_SPIN_TIMEOUT_US,
     stream=None,
 ):
@@ -236,4 +245,4 @@ def gemm(
     """
     _launch(counter_ptr is not None, a, b, c, signal_ptr, cur_wave_sizes, wave_offsets, signal_offsets,
             num_gemm_sms, BLOCK_SIZE_M, BLOCK_SIZE_N, BLOCK_SIZE_K, GROUP_SIZE_M, cum_tiles,
-            counter_ptr, visit_log, xcd_remap, spin_timeout_us, stream)
+            counter_ptr, visit_log, xcd_remap, eight_waves, pair_pipe, spin_timeout_us, stream)
