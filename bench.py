@@ -30,7 +30,9 @@ HBM_PEAK_GBPS = 8000.0
 # AG+GEMM, BASELINE configuration 2
 M, K, N, WORLD, RANK = 8192, 8192, 3584, 8, 0
 BM, BN, BK, GROUP_M = 256, 256, 64, 8
-NUM_SMS = 248                        # 8 of the 256 CUs stay free for the copy kernels of the producer
+NUM_SMS = 224                        # 448 tiles = 2 per program; 32 of the 256 CUs stay free for the
+                                     # copy kernels of the producer
+EIGHT_WAVES = True                   # 512-thread workgroups, two wavefronts per SIMD
 
 
 def _events(n):
@@ -83,7 +85,8 @@ def run_ag_gemm(state, steps, warmup):
     rows = M // WORLD
 
     def consumer(flag_words):
-        gemm(symm, b, c, WORLD, NUM_SMS, BM, BN, BK, GROUP_M, signal_ptr=flag_words, **tables)
+        gemm(symm, b, c, WORLD, NUM_SMS, BM, BN, BK, GROUP_M, signal_ptr=flag_words, xcd_remap=False,
+             eight_waves=EIGHT_WAVES, **tables)
 
     def fused_step():
         ctx.reset_signals()
@@ -169,12 +172,12 @@ def cpu_baseline(state):
 
     threads = min(16, os.cpu_count() or 1)
     torch.set_num_threads(threads)
-    sample_rows = 1024
+    sample_rows = M
     a = state["a"][:sample_rows].cpu()
     b = state["b"].cpu()
     numerics.gemm_fp32(a[:128], b)          # warm-up
     reps, spent = 0, 0.0
-    while spent < 10.0 and reps < 8:
+    while spent < 10.0 and reps < 40:
         t0 = time.perf_counter()
         numerics.gemm_fp32(a, b)
         spent += time.perf_counter() - t0
@@ -249,7 +252,7 @@ def main():
         "max_rel_err_vs_fp32": err,
         "gathered_a_matches": gathered,
         "roofline": {
-            "kernel": "gemm_wave_kernel<bf16,256,256,consumer>",
+            "kernel": "gemm_wave_kernel<bf16, RingPipe, 256x256, 8 wavefronts, consumer>",
             "bound": "mfma",
             "achieved": kernel_tflops,
             "peak": MFMA_BF16_PEAK_TFLOPS,

@@ -44,6 +44,10 @@ extern "C" {
 #define SYN_GEMM_EIGHT_WAVES 2u     /* 512-thread workgroups (two wavefronts per SIMD)     */
 #define SYN_GEMM_PAIR_PIPE 4u       /* force the two-stage 64-deep pipeline (default: the
                                        four-stage 32-deep ring whenever K % 128 == 0)      */
+#define SYN_GEMM_NO_K_STAGGER 8u    /* every tile sweeps K from 0 (default: neighbouring
+                                       tiles start 128 elements apart and wrap around, which
+                                       spreads lockstep programs over the memory channels;
+                                       the fp32 sums are then taken in rotated order)      */
 
 typedef void* syn_stream_t;        /* hipStream_t */
 
@@ -187,6 +191,12 @@ int syn_attn_check_waves(const int32_t* wave_offsets, const int32_t* wave_sizes,
  * calls (syncopate/communication/comm_runtime/communication_context.py:129-160).
  */
 int syn_copy_async(void* dst, const void* src, int64_t nbytes, syn_stream_t stream);
+/* The same copy done by `num_blocks` 256-thread workgroups with streaming (non-temporal)
+ * loads and stores; nbytes and both pointers must be multiples of 16.  Counterpart of the
+ * reference's SM-driven copy (comm_runtime/non_tma_persistent_copy.py:191-304) for the
+ * contiguous case. */
+int syn_copy_kernel_async(void* dst, const void* src, int64_t nbytes, int32_t num_blocks,
+                          syn_stream_t stream);
 int syn_flag_set(uint64_t* flag, uint64_t value, syn_stream_t stream);
 int syn_flag_wait(const uint64_t* flag, uint64_t value, int64_t spin_timeout_us,
                   int32_t* status, syn_stream_t stream);

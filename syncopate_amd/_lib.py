@@ -26,6 +26,7 @@ SYN_STATUS_SPIN_TIMEOUT = 1
 SYN_GEMM_XCD_REMAP = 1
 SYN_GEMM_EIGHT_WAVES = 2
 SYN_GEMM_PAIR_PIPE = 4
+SYN_GEMM_NO_K_STAGGER = 8
 
 _ERRORS = {
     SYN_EINVAL: "SYN_EINVAL (malformed argument or unsupported configuration)",
@@ -124,6 +125,7 @@ _SIGNATURES = {
          c_int32, c_int32, c_int64, c_int64],
     ),
     "syn_copy_async": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p]),
+    "syn_copy_kernel_async": (c_int32, [c_void_p, c_void_p, c_int64, c_int32, c_void_p]),
     "syn_flag_set": (c_int32, [c_void_p, c_uint64, c_void_p]),
     "syn_flag_wait": (c_int32, [c_void_p, c_uint64, c_int64, c_void_p, c_void_p]),
     "syn_delay_us": (c_int32, [c_int64, c_void_p]),

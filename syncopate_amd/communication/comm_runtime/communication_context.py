@@ -48,7 +48,7 @@ class CommContext:
 
     def __init__(self, rank: int, info: CommInfo, multi_info: bool = False, *,
                  device: Optional[torch.device] = None, link_delay_us: int = 0,
-                 wait_timeout_us: int = 2_000_000) -> None:
+                 wait_timeout_us: int = 2_000_000, copy_blocks: int = 0) -> None:
         if info.local_world_size <= 0:
             info.local_world_size = info.world_size
         if info.local_world_size != info.world_size:
@@ -63,6 +63,9 @@ class CommContext:
         self.device = torch.device("cuda", torch.cuda.current_device()) if device is None else device
         self.link_delay_us = int(link_delay_us)
         self.wait_timeout_us = int(wait_timeout_us)
+        # 0: contiguous copies go through hipMemcpyAsync; > 0: through a streaming copy kernel of
+        # that many 256-thread workgroups (16-byte aligned copies only)
+        self.copy_blocks = int(copy_blocks)
         self._lib = _lib.load()
         world = info.local_world_size
 
@@ -130,9 +133,13 @@ class CommContext:
                         raise ValueError(f"{op} runs past the end of its buffer")
                     if self.link_delay_us and op.src_rank != op.dst_rank:
                         _lib.check("syn_delay_us", lib.syn_delay_us(self.link_delay_us, handle))
-                    _lib.check("syn_copy_async",
-                               lib.syn_copy_async(dst.data_ptr() + op.dst_offset,
-                                                  src.data_ptr() + op.src_offset, op.size, handle))
+                    dst_ptr, src_ptr = dst.data_ptr() + op.dst_offset, src.data_ptr() + op.src_offset
+                    kernel_ok = self.copy_blocks > 0 and not (op.size % 16 or dst_ptr % 16 or src_ptr % 16)
+                    if kernel_ok:
+                        _lib.check("syn_copy_kernel_async",
+                                   lib.syn_copy_kernel_async(dst_ptr, src_ptr, op.size, self.copy_blocks, handle))
+                    else:
+                        _lib.check("syn_copy_async", lib.syn_copy_async(dst_ptr, src_ptr, op.size, handle))
                 elif isinstance(op, IntraNodeSignal):
                     assert op.signal_type == SignalType.RECEIVE_DATA
                     flags = self.recv_signal_bufs[op.rank % world]

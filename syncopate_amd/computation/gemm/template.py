@@ -54,6 +54,7 @@ def _launch(
     xcd_remap: bool,
     eight_waves: bool,
     pair_pipe: bool,
+    k_stagger: bool,
     spin_timeout_us: int,
     stream: Optional[torch.cuda.Stream],
 ) -> None:
@@ -133,7 +134,7 @@ def _launch(
         cum_tiles=int(cum_tiles),
         spin_timeout_us=int(spin_timeout_us),
         options=(_lib.SYN_GEMM_XCD_REMAP if xcd_remap else 0) | (_lib.SYN_GEMM_EIGHT_WAVES if eight_waves else 0)
-        | (_lib.SYN_GEMM_PAIR_PIPE if pair_pipe else 0),
+        | (_lib.SYN_GEMM_PAIR_PIPE if pair_pipe else 0) | (0 if k_stagger else _lib.SYN_GEMM_NO_K_STAGGER),
     )
     with torch.cuda.device(dev):
         fn = lib.syn_gemm_producer if producer else lib.syn_gemm_consumer
@@ -162,6 +163,7 @@ def gemm_consumer(
     xcd_remap=True,
     eight_waves=False,
     pair_pipe=False,
+    k_stagger=True,
     spin_timeout_us=DEFAULT_SPIN_TIMEOUT_US,
     stream=None,
 ):
@@ -177,7 +179,7 @@ def gemm_consumer(
     assert M_per_rank % BLOCK_SIZE_M == 0
     _launch(False, a, b, c, signal_buffer, cur_wave_size, wave_offset, signal_offsets, num_gemm_sms,
             BLOCK_SIZE_M, BLOCK_SIZE_N, BLOCK_SIZE_K, GROUP_SIZE_M, cum_tiles, None, visit_log,
-            xcd_remap, eight_waves, pair_pipe, spin_timeout_us, stream)
+            xcd_remap, eight_waves, pair_pipe, k_stagger, spin_timeout_us, stream)
 
 
 def gemm_producer(
@@ -201,6 +203,7 @@ def gemm_producer(
     xcd_remap=True,
     eight_waves=False,
     pair_pipe=False,
+    k_stagger=True,
     stream=None,
 ):
     """GEMM+RS producer: same GEMM; every finished tile bumps its wave's counter
@@ -210,7 +213,7 @@ def gemm_producer(
     """
     _launch(True, a, b, c, signal_buffer, cur_wave_size, wave_offset, signal_offsets, num_gemm_sms,
             BLOCK_SIZE_M, BLOCK_SIZE_N, BLOCK_SIZE_K, GROUP_SIZE_M, cum_tiles, counter_buffer,
-            visit_log, xcd_remap, eight_waves, pair_pipe, DEFAULT_SPIN_TIMEOUT_US, stream)
+            visit_log, xcd_remap, eight_waves, pair_pipe, k_stagger, DEFAULT_SPIN_TIMEOUT_US, stream)
 
 
 def gemm(
@@ -235,6 +238,7 @@ def gemm(
     xcd_remap=True,
     eight_waves=False,
     pair_pipe=False,
+    k_stagger=True,
     spin_timeout_us=DEFAULT_SPIN_TIMEOUT_US,
     stream=None,
 ):
@@ -245,4 +249,4 @@ def gemm(
     """
     _launch(counter_ptr is not None, a, b, c, signal_ptr, cur_wave_sizes, wave_offsets, signal_offsets,
             num_gemm_sms, BLOCK_SIZE_M, BLOCK_SIZE_N, BLOCK_SIZE_K, GROUP_SIZE_M, cum_tiles,
-            counter_ptr, visit_log, xcd_remap, eight_waves, pair_pipe, spin_timeout_us, stream)
+            counter_ptr, visit_log, xcd_remap, eight_waves, pair_pipe, k_stagger, spin_timeout_us, stream)

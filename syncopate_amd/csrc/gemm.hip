@@ -40,6 +40,7 @@ struct GemmParams {
     int32_t num_sms;
     int32_t num_tiles;
     int32_t xcd_remap;
+    int32_t k_stagger;
 };
 
 template <typename T>
@@ -191,7 +192,7 @@ struct PairPipe {
 
     static __device__ __forceinline__ void run(f32x16_t (&acc)[TM][TN], const unsigned char* a_slab,
                                                const unsigned char* b_slab, size_t row_bytes, int K,
-                                               int lane, int wave) {
+                                               int k_rot, int lane, int wave) {
         __shared__ __attribute__((aligned(1024))) unsigned char stage0[STAGE];
         __shared__ __attribute__((aligned(1024))) unsigned char stage1[STAGE];
         const int wm = wave / WGN, wn = wave % WGN;
@@ -203,9 +204,12 @@ struct PairPipe {
         const int a_rd = (wm * WM + (lane & 31)) * ROW;
         const int b_rd = A_BYTES + (wn * WN + (lane & 31)) * ROW;
         const int k_steps = K / BK;
+        const int rot = k_rot % k_steps;
+        // slab i of this tile's walk is slab (i + rot) mod k_steps of K
+        auto at = [&](int i) -> size_t { const int k = i + rot; return (size_t)(k >= k_steps ? k - k_steps : k) * ROW; };
 
-        dma_slab<BM, ROW, NW>(stage0, a_slab, lane_off, row_bytes, wave);
-        dma_slab<BN, ROW, NW>(stage0 + A_BYTES, b_slab, lane_off, row_bytes, wave);
+        dma_slab<BM, ROW, NW>(stage0, a_slab + at(0), lane_off, row_bytes, wave);
+        dma_slab<BN, ROW, NW>(stage0 + A_BYTES, b_slab + at(0), lane_off, row_bytes, wave);
         __syncthreads();                 // waits for the fills (vmcnt) and for every wavefront
 
         // two slabs per trip: fill the idle stage with slab ks+1 while slab ks is multiplied
@@ -213,8 +217,8 @@ struct PairPipe {
         // last slab re-fetches that slab (no branch in the loop body; nothing reads it).
         const int pairs = k_steps >> 1;
         for (int pr = 0; pr < pairs; ++pr) {
-            const size_t k_odd = (size_t)(2 * pr + 1) * ROW;
-            const size_t k_even = (size_t)min(2 * pr + 2, k_steps - 1) * ROW;
+            const size_t k_odd = at(2 * pr + 1);
+            const size_t k_even = at(min(2 * pr + 2, k_steps - 1));
             dma_slab<BM, ROW, NW>(stage1, a_slab + k_odd, lane_off, row_bytes, wave);
             dma_slab<BN, ROW, NW>(stage1 + A_BYTES, b_slab + k_odd, lane_off, row_bytes, wave);
             slab(acc, stage0, a_rd, b_rd, half, swz);
@@ -287,7 +291,7 @@ struct RingPipe {
 
     static __device__ __forceinline__ void run(f32x16_t (&acc)[TM][TN], const unsigned char* a_slab,
                                                const unsigned char* b_slab, size_t row_bytes, int K,
-                                               int lane, int wave) {
+                                               int k_rot, int lane, int wave) {
         __shared__ __attribute__((aligned(1024))) unsigned char st0[STAGE];
         __shared__ __attribute__((aligned(1024))) unsigned char st1[STAGE];
         __shared__ __attribute__((aligned(1024))) unsigned char st2[STAGE];
@@ -301,11 +305,14 @@ struct RingPipe {
         const int half = lane >> 5, swz = (lane >> 2) & 3;
         ln.chunk0 = ((0 + half) ^ swz) << 4;
         ln.chunk1 = ((2 + half) ^ swz) << 4;
-        const int last = K / BK - 1;
+        const int k_steps = K / BK, last = k_steps - 1;
+        const int rot = k_rot % k_steps;
+        // slab i of this tile's walk is slab (i + rot) mod k_steps of K
+        auto at = [&](int i) -> int { const int k = min(i, last) + rot; return k >= k_steps ? k - k_steps : k; };
 
-        fill(st0, a_slab, b_slab, 0, ln, row_bytes, wave);
-        fill(st1, a_slab, b_slab, min(1, last), ln, row_bytes, wave);
-        fill(st2, a_slab, b_slab, min(2, last), ln, row_bytes, wave);
+        fill(st0, a_slab, b_slab, at(0), ln, row_bytes, wave);
+        fill(st1, a_slab, b_slab, at(1), ln, row_bytes, wave);
+        fill(st2, a_slab, b_slab, at(2), ln, row_bytes, wave);
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(2 * FILLS, true));
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
@@ -313,10 +320,10 @@ struct RingPipe {
         load_frags<T, TM, TN, ROW>(fa0, fb0, st0, ln.a_rd, ln.b_rd, ln.chunk0);
 
         for (int s = 0; s <= last; s += 4) {
-            step(acc, fa0, fb0, st0, st1, st3, a_slab, b_slab, min(s + 3, last), ln, row_bytes, wave);
-            step(acc, fa0, fb0, st1, st2, st0, a_slab, b_slab, min(s + 4, last), ln, row_bytes, wave);
-            step(acc, fa0, fb0, st2, st3, st1, a_slab, b_slab, min(s + 5, last), ln, row_bytes, wave);
-            step(acc, fa0, fb0, st3, st0, st2, a_slab, b_slab, min(s + 6, last), ln, row_bytes, wave);
+            step(acc, fa0, fb0, st0, st1, st3, a_slab, b_slab, at(s + 3), ln, row_bytes, wave);
+            step(acc, fa0, fb0, st1, st2, st0, a_slab, b_slab, at(s + 4), ln, row_bytes, wave);
+            step(acc, fa0, fb0, st2, st3, st1, a_slab, b_slab, at(s + 5), ln, row_bytes, wave);
+            step(acc, fa0, fb0, st3, st0, st2, a_slab, b_slab, at(s + 6), ln, row_bytes, wave);
         }
         // drain the re-fetches of the last slab before anything refills the stages
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, true));
@@ -430,8 +437,13 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
 #pragma unroll
                 for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
+        // Tiles walk K cyclically, neighbouring tiles starting 128 elements apart.  With a
+        // power-of-two row pitch, programs that all sweep K from 0 in lockstep keep hitting the
+        // same few memory channels; four phases spread them while tiles that share a panel of A
+        // or B still stay within 512 elements of each other (L2 reuse).
+        const int k_rot = p.k_stagger ? ((pid_m + pid_n) & 3) * (128 / Pipe::BK) : 0;
         Pipe::run(acc, reinterpret_cast<const unsigned char*>(A + m0 * (size_t)K),
-                  reinterpret_cast<const unsigned char*>(B + n0 * (size_t)K), row_bytes, K, lane, wave);
+                  reinterpret_cast<const unsigned char*>(B + n0 * (size_t)K), row_bytes, K, k_rot, lane, wave);
 
         // Epilogue.  With B as the first MFMA operand a lane holds, for column m = lane % 32 of
         // D', rows n = 8g + 4*(lane/32) + 0..3: four consecutive elements of one row of C -> one
@@ -547,6 +559,7 @@ static int gemm_entry(const syn_gemm_desc* d, hipStream_t stream, bool producer)
     p.num_sms = d->num_sms;
     p.num_tiles = (int)tiles;
     p.xcd_remap = (d->options & SYN_GEMM_XCD_REMAP) ? 1 : 0;
+    p.k_stagger = (d->options & SYN_GEMM_NO_K_STAGGER) ? 0 : 1;
     const bool eight = (d->options & SYN_GEMM_EIGHT_WAVES) != 0;
     // the ring needs whole groups of four 32-deep slabs
     const bool ring = !(d->options & SYN_GEMM_PAIR_PIPE) && d->K % 128 == 0;

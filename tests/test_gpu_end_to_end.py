@@ -1,0 +1,262 @@
+"""Fused iterations on one MI355X, from plan builder to kernel: the op list of one rank is
+replayed on side streams by CommContext (the other ranks of the mesh are buffers of the same
+process) while the chunk-scheduled kernel runs on the compute stream.  The flows follow the
+reference's distributed scripts: tests/test_gemm_rs.py:196-233,
+tests/test_allgather_attn_transform.py:94-105 and tests/test_all2all_attn_transform.py:118-146.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import numerics
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-2
+
+
+def _rel(out, ref):
+    return ((out.float().cpu() - ref.float()).abs().max() / ref.float().abs().max()).item()
+
+
+def _compile(plans):
+    from syncopate_amd.communication.code_gen import CommGenerator
+    from syncopate_amd.interface import lower_comm_plan_to_raw_schedules
+
+    gen = CommGenerator(plans)
+    gen.plan_signals()
+    schedules = lower_comm_plan_to_raw_schedules(gen)
+    info = gen.generate_code_for_plan()
+    info.local_world_size = info.world_size
+    return schedules, info
+
+
+@pytest.mark.parametrize("rank", [0, 2])
+def test_gemm_rs_iteration(hip, rank):
+    """Producer GEMM -> comm stream waits on each wave's COMPUTE_DONE flag and pushes the chunk
+    to its owner -> ring reduce of the received partials."""
+    from syncopate_amd.communication.comm_runtime.communication_context import CommContext
+    from syncopate_amd.communication.common_descriptors import build_all_to_all_plan
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.gemm import gemm_producer
+    from syncopate_amd.computation.reduce import ring_reduce_tma
+    from syncopate_amd.interface.wave_tables import gemm_producer_tables
+
+    world, M, N, K, BM, BN = 4, 1024, 512, 256, 128, 128
+    rows = M // world
+    g = torch.Generator().manual_seed(11 + rank)
+    a = (0.1 * torch.randn(M, K, generator=g)).bfloat16()
+    b = (0.1 * torch.randn(N, K, generator=g)).bfloat16()
+    peer_partials = (0.5 * torch.randn(world, rows, N, generator=g)).bfloat16()
+
+    plans = {r: build_all_to_all_plan(shape=(M, N), dtype=torch.bfloat16, mesh_size=world, rank=r,
+                                      src_buffer="src", dst_buffer="dst", transfer_kind="push",
+                                      compute_producer=True) for r in range(world)}
+    schedules, info = _compile(plans)
+    tables = gemm_producer_tables(schedules[rank]["src"])
+    # the chunk a peer owns is computed (and shipped) before the rank's own chunk
+    assert [off[0] // rows for off in tables.block_offsets] == [(rank + 1 + i) % world for i in range(world)]
+
+    ctx = CommContext(rank, info)
+    src = ctx.comm_buffers["src"][rank]
+    dst = ctx.comm_buffers["dst"][rank]
+    src.fill_(float("nan"))          # a chunk shipped before its tiles were stored would carry NaNs
+    dst.copy_(peer_partials.cuda())  # what the peers pushed (they are not replayed here)
+    ad, bd = a.cuda(), b.cuda()
+    out = torch.empty(rows, N, dtype=torch.bfloat16, device="cuda")
+    comm_stream = torch.cuda.Stream()
+    main = torch.cuda.current_stream()
+
+    ctx.reset_signals()
+    comm_stream.wait_stream(main)
+    gemm_producer(ad, bd, src, ctx.compute_signal_bufs[rank], tables.block_shapes, tables.block_offsets,
+                  tables.signal_offsets, 13, BM, BN, 64, 8, cum_tiles=tables.cum_tiles)
+    ctx.start_after(comm_stream)
+    ctx.execute(neglect_local=True)
+    ctx.end_before(comm_stream)
+    main.wait_stream(comm_stream)
+    ring_reduce_tma(dst, out, src, rank)
+    check_status()
+    ctx.check_status()
+
+    partial = numerics.gemm_fp32(a, b)
+    assert _rel(src, partial) <= REL_TOL
+    assert ctx.compute_signal_bufs[rank].tolist() == [1] * world
+    for peer in range(world):
+        if peer == rank:
+            continue
+        # the peer's slot `rank` holds the rows it owns of this rank's partial result, bit for bit
+        got = ctx.comm_buffers["dst"][peer][rank]
+        assert torch.equal(got, src[peer * rows:(peer + 1) * rows])
+        peer_flags = ctx.recv_signal_bufs[peer].tolist()
+        assert sum(peer_flags) == 1
+    # neglect_local drops the local copy only: its flag is still written
+    assert ctx.recv_signal_bufs[rank].sum().item() == 1
+    assert torch.equal(dst.cpu(), peer_partials)
+    want = numerics.ring_reduce(dst.float().cpu().numpy(), src.float().cpu().numpy(), rank, dtype="bf16")
+    assert np.array_equal(out.float().cpu().numpy(), want)
+    total = partial[rank * rows:(rank + 1) * rows].double()
+    for peer in range(world):
+        if peer != rank:
+            total = total + peer_partials[peer].double()
+    assert _rel(out, total) <= 2e-2
+
+
+@pytest.mark.parametrize("rank", [1, 3])
+def test_allgather_attention_iteration(hip, rank):
+    """K/V chunks pulled from their owners on a side stream (copy, then flag) while the
+    attention kernel walks the waves of the lowered schedule; the local Q attends to the whole
+    sequence."""
+    from syncopate_amd.communication.comm_runtime.communication_context import CommContext
+    from syncopate_amd.communication.common_descriptors import build_all_gather_plan_1d_swizzle
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.attn import attention_forward
+    from syncopate_amd.interface.wave_tables import allgather_attn_tables, plan_layout_spec
+
+    world, B, H, SEQ, D = 4, 1, 2, 1024, 128
+    per_rank = SEQ // world
+    shape, seq_axis, axes = plan_layout_spec("bhsd", B, H, SEQ, D)
+    plans = {r: build_all_gather_plan_1d_swizzle(shape, torch.bfloat16, seq_axis, world, r, "kv", "pull")
+             for r in range(world)}
+    schedules, info = _compile(plans)
+    tables = allgather_attn_tables(schedules[rank]["kv"], per_rank, axes)
+    assert [off[3] // per_rank for off in tables.wave_offsets] == [(rank + i) % world for i in range(world)]
+    assert tables.signal_offsets == [-1, 0, 1, 2]    # the rank's own chunk needs no flag
+
+    g = torch.Generator().manual_seed(5)
+    kv = torch.randn(*shape, generator=g).bfloat16()
+    q = torch.randn(B, H, per_rank, D, generator=g).bfloat16()
+    ctx = CommContext(rank, info, link_delay_us=30)
+    for r in range(world):                           # every simulated rank holds its own slice
+        ctx.comm_buffers["kv"][r][:, :, :, r * per_rank:(r + 1) * per_rank].copy_(
+            kv[:, :, :, r * per_rank:(r + 1) * per_rank])
+    buf = ctx.comm_buffers["kv"][rank]
+    qd = q.cuda()
+    tiles = tables.cum_tiles // 128
+    log = torch.full((tiles, 8), -1, dtype=torch.int32, device="cuda")
+    main = torch.cuda.current_stream()
+
+    ctx.reset_signals()
+    ctx.start_after(main)
+    ctx.execute()
+    out = attention_forward(qd, buf[0], buf[1], D ** -0.5, wave_offsets=tables.wave_offsets,
+                            wave_sizes=tables.wave_sizes, cum_wave_sizes=tables.cum_wave_sizes,
+                            signal_ptr=ctx.recv_signal_bufs[rank], signal_offsets=tables.signal_offsets,
+                            NUM_WAVES=len(tables.signal_offsets), cum_tiles=tables.cum_tiles, visit_log=log)
+    ctx.end_before(main)
+    check_status()
+    ctx.check_status()
+
+    assert torch.equal(buf.cpu(), kv)                # the gather itself
+    want = numerics.sdpa_fp32(q, kv[0], kv[1], D ** -0.5)
+    assert _rel(out, want) <= REL_TOL
+    assert (log[:, 0] >= 0).all()                    # every tile of every wave ran
+
+
+def test_all2all_attention_iteration_with_graph_replay(hip):
+    """Ulysses exchange of stacked Q/K/V captured as a HIP graph (the reference captures the
+    comm side, tests/test_all2all_attn_transform.py:278) and replayed several times: every
+    replay, with eager work and synchronisation in between, must gather the same bytes and give
+    the same attention output as the eager run."""
+    from syncopate_amd.communication.comm_runtime.communication_context import CommContext
+    from syncopate_amd.communication.common_descriptors import build_all_to_all_plan_dim
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.attn import attention_forward
+    from syncopate_amd.interface.wave_tables import all2all_attn_tables
+
+    world, rank, B, H, S_local, D = 4, 1, 1, 8, 256, 128
+    H_local, SEQ = H // world, world * S_local
+    shape = (3, B, H, S_local, D)
+    plans = {r: build_all_to_all_plan_dim(shape=shape, dtype=torch.bfloat16, mesh_size=world, rank=r,
+                                          src_buffer="src", dst_buffer="dst", src_split_axis=3,
+                                          dst_split_axis=2, transfer_kind="pull", compute_producer=False)
+             for r in range(world)}
+    schedules, info = _compile(plans)
+    tables = all2all_attn_tables(schedules[rank]["dst"], {"batch": 1, "head": 2, "seq": 3})
+    assert len(tables.signal_offsets) == world * world
+
+    g = torch.Generator().manual_seed(9)
+    qkv = [torch.randn(*shape, generator=g).bfloat16() for _ in range(world)]     # per source rank
+    # what the exchange must leave on `rank`: its heads, the whole sequence
+    gathered = torch.cat([x[:, :, rank * H_local:(rank + 1) * H_local] for x in qkv], dim=3)
+    ctx = CommContext(rank, info)
+    for r in range(world):
+        ctx.comm_buffers["src"][r].copy_(qkv[r])
+    dst = ctx.comm_buffers["dst"][rank]
+    flags = ctx.recv_signal_bufs[rank]
+    main = torch.cuda.current_stream()
+
+    def attend():
+        return attention_forward(dst[0], dst[1], dst[2], D ** -0.5, wave_offsets=tables.wave_offsets,
+                                 wave_sizes=tables.wave_sizes, cum_wave_sizes=tables.cum_wave_sizes,
+                                 signal_ptr=flags, signal_offsets=tables.signal_offsets,
+                                 NUM_WAVES=len(tables.signal_offsets), cum_tiles=tables.cum_tiles)
+
+    # eager
+    dst.zero_()
+    ctx.reset_signals()
+    ctx.start_after(main)
+    ctx.execute()
+    eager = attend()
+    ctx.end_before(main)
+    check_status()
+    ctx.check_status()
+    assert torch.equal(dst.cpu(), gathered)
+    want = numerics.sdpa_fp32(gathered[0], gathered[1], gathered[2], D ** -0.5)
+    assert _rel(eager, want) <= REL_TOL
+
+    graph = ctx.get_graph()
+    comm_stream = torch.cuda.Stream()
+    for replay in range(3):
+        dst.zero_()
+        ctx.reset_signals()
+        torch.cuda.synchronize()
+        comm_stream.wait_stream(main)
+        with torch.cuda.stream(comm_stream):
+            graph.replay()
+        out = attend()
+        main.wait_stream(comm_stream)
+        check_status()
+        ctx.check_status()
+        assert torch.equal(dst.cpu(), gathered), f"replay {replay}"
+        # partial results of one q block merge in the order their workgroups take the lock, so
+        # two runs agree to rounding, not bit for bit
+        assert _rel(out, want) <= REL_TOL, f"replay {replay}"
+        assert flags.tolist() == [1] * world
+
+
+def test_copy_kernel_producer_matches_copy_engine(hip):
+    """The compute-unit copy path of CommContext (copy_blocks > 0) moves the same bytes."""
+    from syncopate_amd.communication.comm_runtime.communication_context import CommContext
+    from syncopate_amd.communication.common_descriptors import build_all_gather_plan_1d_swizzle
+
+    world, rank, M, K = 4, 3, 512, 384
+    plans = {r: build_all_gather_plan_1d_swizzle((M, K), torch.float16, 0, world, r, "a", "pull")
+             for r in range(world)}
+    _, info = _compile(plans)
+    g = torch.Generator().manual_seed(2)
+    a = torch.randn(M, K, generator=g).half()
+    rows = M // world
+    for blocks in (0, 8):
+        ctx = CommContext(rank, info, copy_blocks=blocks)
+        for r in range(world):
+            ctx.comm_buffers["a"][r][r * rows:(r + 1) * rows].copy_(a[r * rows:(r + 1) * rows])
+        ctx.reset_signals()
+        ctx.start_after()
+        ctx.execute()
+        ctx.end_before()
+        ctx.check_status()
+        assert torch.equal(ctx.comm_buffers["a"][rank].cpu(), a)
+        assert ctx.recv_signal_bufs[rank].tolist() == [1] * (world - 1)
+
+
+def test_copy_kernel_rejects_misaligned(hip):
+    buf = torch.zeros(256, dtype=torch.uint8, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+    from syncopate_amd import _lib
+
+    assert hip.syn_copy_kernel_async(buf.data_ptr() + 8, buf.data_ptr() + 128, 64, 4, s) == _lib.SYN_EALIGN
+    assert hip.syn_copy_kernel_async(buf.data_ptr(), buf.data_ptr() + 128, 60, 4, s) == _lib.SYN_EALIGN
+    assert hip.syn_copy_kernel_async(buf.data_ptr(), buf.data_ptr() + 128, 64, 0, s) == _lib.SYN_EINVAL
+    torch.cuda.synchronize()
