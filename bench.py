@@ -7,7 +7,7 @@ A step is one fused all-gather+GEMM iteration of rank 0 of a simulated mesh of 8
 copied into the symmetric buffer on a side stream in the order the lowered schedule
 prescribes (copy, then flag), the consumer GEMM (8192 x 8192 x 3584) on the compute stream
 waiting on each chunk's flag.  All operands are resident in HBM before the timed region.
-Prints ONE JSON line; see DESIGN.md for the meaning of every field.
+Prints ONE JSON line.
 """
 
 from __future__ import annotations
@@ -26,6 +26,11 @@ import torch  # noqa: E402
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0      # MI355X dense bf16
 HBM_PEAK_GBPS = 8000.0
+# Bytes one launch of the 256x256 consumer kernel moves between L2 and the fabric: FETCH_SIZE and
+# WRITE_SIZE of two counter runs of `bench.py --resident-only`, scaled by the readings of the
+# library's copy kernel (profiles/ag_gemm_8192x8192x3584_bench_hbm_traffic.txt).  Counter runs
+# serialise kernels, so this cannot be sampled while the benchmark itself runs.
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 996.5e6
 
 # AG+GEMM, BASELINE configuration 2
 M, K, N, WORLD, RANK = 8192, 8192, 3584, 8, 0
@@ -74,7 +79,7 @@ def build_ag_gemm(device):
     return dict(a=a, b=b, c=c, ctx=ctx, tables=dev_tables, compile_ms=compile_ms)
 
 
-def run_ag_gemm(state, steps, warmup):
+def run_ag_gemm(state, steps, warmup, resident_only=False):
     from syncopate_amd.computation._launch import check_status
     from syncopate_amd.computation.gemm import gemm
 
@@ -96,22 +101,27 @@ def run_ag_gemm(state, steps, warmup):
         ctx.end_before(stream)
 
     # ---- gated run: the step the metric is quoted on ----
-    for _ in range(warmup):
-        fused_step()
-    torch.cuda.synchronize()
-    begin, end = _events(steps), _events(steps)
-    t0 = time.perf_counter()
-    for i in range(steps):
-        ctx.reset_signals()
-        ctx.start_after(stream)
-        ctx.execute()
-        begin[i].record(stream)
-        consumer(flags)
-        end[i].record(stream)
-        ctx.end_before(stream)
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    gated_kernel_ms = sum(s.elapsed_time(e) for s, e in zip(begin, end)) / steps
+    wall_ms = gated_kernel_ms = None
+    if resident_only:
+        fused_step()                      # once, so that the gathered buffer is complete
+        torch.cuda.synchronize()
+    else:
+        for _ in range(warmup):
+            fused_step()
+        torch.cuda.synchronize()
+        begin, end = _events(steps), _events(steps)
+        t0 = time.perf_counter()
+        for i in range(steps):
+            ctx.reset_signals()
+            ctx.start_after(stream)
+            ctx.execute()
+            begin[i].record(stream)
+            consumer(flags)
+            end[i].record(stream)
+            ctx.end_before(stream)
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+        gated_kernel_ms = sum(s.elapsed_time(e) for s, e in zip(begin, end)) / steps
     check_status()
     ctx.check_status()
 
@@ -128,7 +138,24 @@ def run_ag_gemm(state, steps, warmup):
     torch.cuda.synchronize()
     resident_kernel_ms = sum(s.elapsed_time(e) for s, e in zip(begin, end)) / steps
     check_status()
+    if resident_only:
+        wall_ms = gated_kernel_ms = resident_kernel_ms
     return wall_ms, gated_kernel_ms, resident_kernel_ms
+
+
+def traffic_calibration(device):
+    """One launch of the library's plain copy kernel over 64 MiB: under a counter run its
+    FETCH_SIZE / WRITE_SIZE readings give the scale of those counters (65536 KiB each way)."""
+    from syncopate_amd import _lib
+
+    lib = _lib.load()
+    nbytes = 64 << 20
+    src = torch.empty(nbytes, dtype=torch.uint8, device=device).fill_(1)
+    dst = torch.empty_like(src)
+    _lib.check("syn_copy_kernel_async",
+               lib.syn_copy_kernel_async(dst.data_ptr(), src.data_ptr(), nbytes, 1024,
+                                         torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
 
 
 def check_ag_gemm(state):
@@ -142,25 +169,27 @@ def check_ag_gemm(state):
 
 
 def run_reduce(device, steps, warmup):
-    """GEMM+RS chunked reduce at BASELINE configuration 3: 8 x (1024, 8192) bf16 -> (1024, 8192)."""
+    """GEMM+RS chunked reduce at BASELINE configuration 3: 8 x (1024, 8192) bf16 -> (1024, 8192).
+    Launches rotate over three sets of operands (3 x 151 MB, more than the 256 MB of memory-side
+    cache) so that every launch streams from HBM; the batch is timed as a whole."""
     from syncopate_amd.computation.reduce import ring_reduce
 
-    world, rows, n = 8, 1024, 8192
+    world, rows, n, sets = 8, 1024, 8192, 3
     torch.manual_seed(1)
-    recv = torch.randn(world, rows, n, device=device).bfloat16()
-    local = torch.randn(world * rows, n, device=device).bfloat16()
-    out = torch.empty(rows, n, dtype=torch.bfloat16, device=device)
+    recv = [torch.randn(world, rows, n, device=device).bfloat16() for _ in range(sets)]
+    local = [torch.randn(world * rows, n, device=device).bfloat16() for _ in range(sets)]
+    out = [torch.empty(rows, n, dtype=torch.bfloat16, device=device) for _ in range(sets)]
     stream = torch.cuda.current_stream()
-    for _ in range(warmup):
-        ring_reduce(recv, out, local, RANK)
+    for i in range(max(warmup, sets)):
+        ring_reduce(recv[i % sets], out[i % sets], local[i % sets], RANK)
     torch.cuda.synchronize()
-    begin, end = _events(steps), _events(steps)
+    begin, end = _events(1)[0], _events(1)[0]
+    begin.record(stream)
     for i in range(steps):
-        begin[i].record(stream)
-        ring_reduce(recv, out, local, RANK)
-        end[i].record(stream)
+        ring_reduce(recv[i % sets], out[i % sets], local[i % sets], RANK)
+    end.record(stream)
     torch.cuda.synchronize()
-    ms = sum(s.elapsed_time(e) for s, e in zip(begin, end)) / steps
+    ms = begin.elapsed_time(end) / steps
     nbytes = (world + 1) * rows * n * 2          # 8 reads + 1 write of a (1024, 8192) bf16 block
     return ms, nbytes
 
@@ -199,6 +228,9 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--resident-only", action="store_true",
+                    help="skip the flag-gated steps (for hardware-counter runs, which serialise kernels: "
+                         "a gated consumer would wait for copies that can only start after it)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one rank's share on ONE GPU: the other ranks of the mesh are "
@@ -212,9 +244,10 @@ def main():
     torch.cuda.set_device(device)
 
     state = build_ag_gemm(device)
-    wall_ms, gated_ms, resident_ms = run_ag_gemm(state, args.steps, args.warmup)
+    wall_ms, gated_ms, resident_ms = run_ag_gemm(state, args.steps, args.warmup, args.resident_only)
+    traffic_calibration(device)
     err, gathered = check_ag_gemm(state)
-    reduce_ms, reduce_bytes = run_reduce(device, max(args.steps, 20), args.warmup)
+    reduce_ms, reduce_bytes = run_reduce(device, max(args.steps, 30), args.warmup)
 
     flop = 2.0 * M * N * K
     value = flop / (wall_ms * 1e-3) / 1e12
@@ -232,6 +265,7 @@ def main():
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
+        "resident_only": bool(args.resident_only),
         "config": {
             "workload": "AG-GEMM one rank's share, simulated mesh=8: A (8192,8192) bf16 arriving as 8 chunks "
                         "of 1024 rows in swizzled order behind flags, B (8192,3584) bf16 stored [N,K], "
@@ -258,7 +292,7 @@ def main():
             "peak": MFMA_BF16_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": kernel_tflops / MFMA_BF16_PEAK_TFLOPS,
-            "traffic": None,
+            "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH,
         },
     }
     if not args.no_cpu_baseline:
