@@ -42,8 +42,9 @@ extern "C" {
 #define SYN_GEMM_XCD_REMAP 1u       /* permute hardware workgroup ids so that consecutive
                                        logical program ids share an XCD (and its L2)      */
 #define SYN_GEMM_EIGHT_WAVES 2u     /* 512-thread workgroups (two wavefronts per SIMD)     */
-#define SYN_GEMM_PAIR_PIPE 4u       /* force the two-stage 64-deep pipeline (default: the
-                                       four-stage 32-deep ring whenever K % 128 == 0)      */
+#define SYN_GEMM_RING_PIPE 4u       /* four LDS stages of 32-deep K slabs instead of the default
+                                       two stages of 64-deep slabs; needs K % 128 == 0,
+                                       otherwise the default pipeline runs                 */
 #define SYN_GEMM_NO_K_STAGGER 8u    /* every tile sweeps K from 0 (default: neighbouring
                                        tiles start 128 elements apart and wrap around, which
                                        spreads lockstep programs over the memory channels;

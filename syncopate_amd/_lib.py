@@ -25,7 +25,7 @@ SYN_STATUS_WORDS = 4
 SYN_STATUS_SPIN_TIMEOUT = 1
 SYN_GEMM_XCD_REMAP = 1
 SYN_GEMM_EIGHT_WAVES = 2
-SYN_GEMM_PAIR_PIPE = 4
+SYN_GEMM_RING_PIPE = 4
 SYN_GEMM_NO_K_STAGGER = 8
 
 _ERRORS = {

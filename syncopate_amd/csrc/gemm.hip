@@ -3,16 +3,18 @@
 // A workgroup owns a BM x BN tile of C and walks tile ids pid, pid + NUM_SMS, ... in the
 // wave order of the schedule (syncopate/computation/gemm/template.py:69-136).  A and B are
 // both K-contiguous, so a k-slab of either is a set of short rows.  Slabs go from HBM
-// straight into an LDS ring with global_load_lds_dwordx4 (16 bytes per lane, no register
+// straight into LDS stages with global_load_lds_dwordx4 (16 bytes per lane, no register
 // staging); a wavefront-wide load fills 1 KB of consecutive LDS rows, and which 16-byte
 // chunk of its row a lane fetches is XOR-swizzled with the row number so that the 128-bit
 // fragment reads of v_mfma_f32_32x32x16 are bank-conflict free over the 64 LDS banks.
 //
-// Two pipelines over the same tile walk:
-//   ring   4 stages of 32-deep slabs; the fill of slab s+3 is issued while slab s is being
-//          multiplied, so three slabs are in flight and HBM/L2 latency is covered; one
-//          barrier per slab, with MFMA work on both sides of it.  Needs K % 128 == 0.
-//   pair   2 stages of 64-deep slabs (one in flight); any K % 64 == 0.
+// Two pipelines over the same tile walk, both with one barrier per slab and MFMA work on
+// both sides of it:
+//   pair   2 stages of 64-deep slabs: rows are whole 128-byte cache lines, one slab in flight
+//          while the other is multiplied; any K % 64 == 0.  The default.
+//   ring   4 stages of 32-deep slabs, three in flight; rows are half cache lines, which costs
+//          L1 fill bandwidth.  Needs K % 128 == 0.
+// A tile's first fills are issued before the previous tile's C is stored.
 //
 // Consumer form: before the first tile of a wave whose signal offset is >= 0 lane 0 spins on
 // the flag word, then the whole workgroup takes an acquire fence (template.py:121-128).
@@ -151,16 +153,67 @@ __device__ __forceinline__ void interleave_hint() {
     interleave_reads<0, READS, MFMAS>();
 }
 
+// The same with the fills spread out too: G groups of (MFMAs, fill, LDS read), every kind
+// divided as evenly as integers allow.  A wavefront issues in order, so a burst of fills that
+// outruns the vector-memory queue would hold its MFMAs back; one fill every few MFMAs never does.
+template <int G, int GROUPS, int READS, int MFMAS, int FILLS>
+__device__ __forceinline__ void spread_groups() {
+    if constexpr (G < GROUPS) {
+        constexpr int m = MFMAS * (G + 1) / GROUPS - MFMAS * G / GROUPS;
+        constexpr int r = READS * (G + 1) / GROUPS - READS * G / GROUPS;
+        constexpr int f = FILLS * (G + 1) / GROUPS - FILLS * G / GROUPS;
+        if constexpr (m > 0) __builtin_amdgcn_sched_group_barrier(kSgMfma, m, 0);
+        if constexpr (f > 0) __builtin_amdgcn_sched_group_barrier(kSgVmemRead, f, 0);
+        if constexpr (r > 0) __builtin_amdgcn_sched_group_barrier(kSgDsRead, r, 0);
+        spread_groups<G + 1, GROUPS, READS, MFMAS, FILLS>();
+    }
+}
+
+template <int READS, int MFMAS, int FILLS>
+__device__ __forceinline__ void spread_hint() {
+    constexpr int want = READS > FILLS ? READS : FILLS;
+    constexpr int groups = want < 1 ? 1 : (want > MFMAS ? MFMAS : want);
+    spread_groups<0, groups, READS, MFMAS, FILLS>();
+}
+
+// Fills FIRST..LAST-1 of a stage of BM rows of A followed by BN rows of B, in the numbering
+// of dma_slab (fill j of this wavefront is 1 KB block j * NW + wave of the stage).
+template <int FIRST, int LAST, int BM, int ROW_BYTES, int NW>
+__device__ __forceinline__ void dma_part(unsigned char* stage, const unsigned char* a_slab,
+                                         const unsigned char* b_slab, unsigned lane_off,
+                                         size_t row_bytes, int wave) {
+    constexpr int kRowsPerBlock = 1024 / ROW_BYTES;
+    constexpr int kABlocks = BM / kRowsPerBlock;
+#pragma unroll
+    for (int j = FIRST; j < LAST; ++j) {
+        const int blk = j * NW + wave;                 // block of the stage: A blocks, then B blocks
+        const unsigned char* src = blk < kABlocks
+            ? a_slab + (size_t)(blk * kRowsPerBlock) * row_bytes
+            : b_slab + (size_t)((blk - kABlocks) * kRowsPerBlock) * row_bytes;
+        __builtin_amdgcn_global_load_lds((global_void_ptr)(src + lane_off),
+                                         (lds_void_ptr)(stage + blk * 1024), 16, 0, 0);
+    }
+}
+
 // ------------------------------------------------------------------ pipelines
 //
-// Both take the accumulators, the uniform addresses of the tile's A and B row panels and
-// run the whole K loop.  On return every fill has landed and every wavefront has passed a
-// barrier, so the stages may be refilled at once.
+// Both are split in two: prologue() issues the first fills of a tile from the uniform addresses
+// of its A and B row panels; main() takes the accumulators and runs the whole K loop.  When
+// main() returns every fill has landed and every wavefront has passed a barrier, so the stages
+// may be refilled at once - the kernel issues the next tile's prologue before it stores C.
 
 // pair: two stages of 64-deep slabs.  LDS row r (128 bytes) keeps logical chunk c at physical
 // chunk c ^ ((r >> 1) & 7): a row covers half of the 64 banks (even rows the low half), a
 // 128-bit read is served 16 consecutive rows per cycle, and (r >> 1) & 7 gives the 8 rows that
-// share a half 8 distinct chunks.
+// share a half 8 distinct chunks.  Rows are whole 128-byte cache lines.
+//
+// Slab s lives in stage s % 2 and is multiplied in four k16 steps:
+//     steps 0-2: MFMAs of the step | read the fragments of the next step
+//     wait: own fills of slab s+1 landed, own LDS reads returned;  barrier
+//     step 3:    MFMAs             | read step 0 of slab s+1 | issue the fills of slab s+2
+//                                    into the stage slab s has just been read out of
+// so a barrier costs no LDS latency and a fill has one slab time to land.  Fills past the
+// last slab re-fetch it (nothing reads them).
 template <typename T, int BM, int BN, int WGM, int WGN>
 struct PairPipe {
     static constexpr int NW = WGM * WGN;
@@ -171,67 +224,114 @@ struct PairPipe {
     static constexpr int K_ALIGN = 64;
     typedef typename Mfma32<T>::frag_t frag_t;
 
-    static __device__ __forceinline__ void slab(f32x16_t (&acc)[TM][TN], const unsigned char* st,
-                                                int a_rd, int b_rd, int half, int swz) {
-        frag_t fa0[TM], fb0[TN], fa1[TM], fb1[TN];
-        load_frags<T, TM, TN, ROW>(fa0, fb0, st, a_rd, b_rd, ((0 + half) ^ swz) << 4);
-        __builtin_amdgcn_sched_group_barrier(kSgDsRead, TM + TN, 0);
-#pragma unroll
-        for (int kk = 0; kk < 4; kk += 2) {
-            load_frags<T, TM, TN, ROW>(fa1, fb1, st, a_rd, b_rd, (((kk + 1) * 2 + half) ^ swz) << 4);
-            mma_step<T, TM, TN>(acc, fa0, fb0);
-            if (kk == 0) interleave_hint<TM + TN, TM * TN, FILLS>();
-            else interleave_hint<TM + TN, TM * TN, 0>();
-            __builtin_amdgcn_sched_barrier(0);
-            if (kk + 2 < 4) load_frags<T, TM, TN, ROW>(fa0, fb0, st, a_rd, b_rd, (((kk + 2) * 2 + half) ^ swz) << 4);
-            mma_step<T, TM, TN>(acc, fa1, fb1);
-            if (kk + 2 < 4) interleave_hint<TM + TN, TM * TN, 0>();
-            __builtin_amdgcn_sched_barrier(0);
-        }
+    struct Lane {
+        unsigned lane_off;
+        int a_rd, b_rd, half, swz;
+    };
+
+    static __device__ __forceinline__ void fill(unsigned char* st, const unsigned char* a_slab,
+                                                const unsigned char* b_slab, size_t k_off, const Lane& ln,
+                                                size_t row_bytes, int wave) {
+        dma_part<0, FILLS, BM, ROW, NW>(st, a_slab + k_off, b_slab + k_off, ln.lane_off, row_bytes, wave);
     }
 
-    static __device__ __forceinline__ void run(f32x16_t (&acc)[TM][TN], const unsigned char* a_slab,
-                                               const unsigned char* b_slab, size_t row_bytes, int K,
-                                               int k_rot, int lane, int wave) {
-        __shared__ __attribute__((aligned(1024))) unsigned char stage0[STAGE];
-        __shared__ __attribute__((aligned(1024))) unsigned char stage1[STAGE];
+    // f0 holds the fragments of (cur, step 0) on entry and of (nxt, step 0) on exit
+    static __device__ __forceinline__ void slab(f32x16_t (&acc)[TM][TN], frag_t (&fa0)[TM], frag_t (&fb0)[TN],
+                                                unsigned char* cur, const unsigned char* nxt,
+                                                const unsigned char* a_slab, const unsigned char* b_slab,
+                                                size_t k_refill, const Lane& ln, size_t row_bytes, int wave) {
+        frag_t fa1[TM], fb1[TN];
+        load_frags<T, TM, TN, ROW>(fa1, fb1, cur, ln.a_rd, ln.b_rd, ((2 + ln.half) ^ ln.swz) << 4);
+        mma_step<T, TM, TN>(acc, fa0, fb0);
+        spread_hint<TM + TN, TM * TN, 0>();
+        __builtin_amdgcn_sched_barrier(0);
+
+        load_frags<T, TM, TN, ROW>(fa0, fb0, cur, ln.a_rd, ln.b_rd, ((4 + ln.half) ^ ln.swz) << 4);
+        mma_step<T, TM, TN>(acc, fa1, fb1);
+        spread_hint<TM + TN, TM * TN, 0>();
+        __builtin_amdgcn_sched_barrier(0);
+
+        load_frags<T, TM, TN, ROW>(fa1, fb1, cur, ln.a_rd, ln.b_rd, ((6 + ln.half) ^ ln.swz) << 4);
+        mma_step<T, TM, TN>(acc, fa0, fb0);
+        spread_hint<TM + TN, TM * TN, 0>();
+        __builtin_amdgcn_sched_barrier(0);
+
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, true));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+
+        fill(cur, a_slab, b_slab, k_refill, ln, row_bytes, wave);
+        load_frags<T, TM, TN, ROW>(fa0, fb0, nxt, ln.a_rd, ln.b_rd, ((0 + ln.half) ^ ln.swz) << 4);
+        mma_step<T, TM, TN>(acc, fa1, fb1);
+        spread_hint<TM + TN, TM * TN, FILLS>();
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // the stages are distinct objects: LDS reads of one never wait for fills of the other
+    template <int I>
+    static __device__ __forceinline__ unsigned char* stage() {
+        __shared__ __attribute__((aligned(1024))) unsigned char st[STAGE];
+        return st;
+    }
+
+    static __device__ __forceinline__ Lane make_lane(size_t row_bytes, int lane, int wave) {
         const int wm = wave / WGN, wn = wave % WGN;
+        Lane ln;
         const int ld_row = lane >> 3;
         // blocks this wavefront fills are wave, wave + NW, ... (NW even): block parity = wave parity
         const int ld_chunk = (lane & 7) ^ ((((wave & 1) << 3 | ld_row) >> 1) & 7);
-        const unsigned lane_off = (unsigned)(ld_row * row_bytes) + ld_chunk * 16;
-        const int half = lane >> 5, swz = (lane >> 1) & 7;
-        const int a_rd = (wm * WM + (lane & 31)) * ROW;
-        const int b_rd = A_BYTES + (wn * WN + (lane & 31)) * ROW;
-        const int k_steps = K / BK;
+        ln.lane_off = (unsigned)(ld_row * row_bytes) + ld_chunk * 16;
+        ln.half = lane >> 5;
+        ln.swz = (lane >> 1) & 7;
+        ln.a_rd = (wm * WM + (lane & 31)) * ROW;
+        ln.b_rd = A_BYTES + (wn * WN + (lane & 31)) * ROW;
+        return ln;
+    }
+
+    // byte offset inside a row of slab i of this tile's cyclic walk: slab (i + rot) mod k_steps of K
+    static __device__ __forceinline__ size_t slab_off(int i, int rot, int k_steps) {
+        const int k = min(i, k_steps - 1) + rot;
+        return (size_t)(k >= k_steps ? k - k_steps : k) * ROW;
+    }
+
+    // Issue the fills of the tile's first two slabs.  Needs nothing but free stages, so the caller
+    // runs it ahead of the previous tile's epilogue.
+    static __device__ __forceinline__ void prologue(const unsigned char* a_slab, const unsigned char* b_slab,
+                                                    size_t row_bytes, int K, int k_rot, int lane, int wave) {
+        const Lane ln = make_lane(row_bytes, lane, wave);
+        const int k_steps = K / BK, rot = k_rot % k_steps;
+        fill(stage<0>(), a_slab, b_slab, slab_off(0, rot, k_steps), ln, row_bytes, wave);
+        fill(stage<1>(), a_slab, b_slab, slab_off(1, rot, k_steps), ln, row_bytes, wave);
+    }
+
+    // The K loop of a tile whose prologue has been issued.  On return every fill has landed and
+    // every wavefront has passed a barrier: the stages are free.
+    static __device__ __forceinline__ void main(f32x16_t (&acc)[TM][TN], const unsigned char* a_slab,
+                                                const unsigned char* b_slab, size_t row_bytes, int K,
+                                                int k_rot, int lane, int wave) {
+        unsigned char* const stage0 = stage<0>();
+        unsigned char* const stage1 = stage<1>();
+        const Lane ln = make_lane(row_bytes, lane, wave);
+        const int k_steps = K / BK, last = k_steps - 1;
         const int rot = k_rot % k_steps;
-        // slab i of this tile's walk is slab (i + rot) mod k_steps of K
-        auto at = [&](int i) -> size_t { const int k = i + rot; return (size_t)(k >= k_steps ? k - k_steps : k) * ROW; };
 
-        dma_slab<BM, ROW, NW>(stage0, a_slab + at(0), lane_off, row_bytes, wave);
-        dma_slab<BN, ROW, NW>(stage0 + A_BYTES, b_slab + at(0), lane_off, row_bytes, wave);
-        __syncthreads();                 // waits for the fills (vmcnt) and for every wavefront
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(FILLS, true));       // slab 0 landed; slab 1 may fly on
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        frag_t fa0[TM], fb0[TN];
+        load_frags<T, TM, TN, ROW>(fa0, fb0, stage0, ln.a_rd, ln.b_rd, ((0 + ln.half) ^ ln.swz) << 4);
 
-        // two slabs per trip: fill the idle stage with slab ks+1 while slab ks is multiplied
-        // out of the other; the barrier ending a slab also drains the fill.  The fill after the
-        // last slab re-fetches that slab (no branch in the loop body; nothing reads it).
         const int pairs = k_steps >> 1;
         for (int pr = 0; pr < pairs; ++pr) {
-            const size_t k_odd = at(2 * pr + 1);
-            const size_t k_even = at(min(2 * pr + 2, k_steps - 1));
-            dma_slab<BM, ROW, NW>(stage1, a_slab + k_odd, lane_off, row_bytes, wave);
-            dma_slab<BN, ROW, NW>(stage1 + A_BYTES, b_slab + k_odd, lane_off, row_bytes, wave);
-            slab(acc, stage0, a_rd, b_rd, half, swz);
-            __syncthreads();
-            dma_slab<BM, ROW, NW>(stage0, a_slab + k_even, lane_off, row_bytes, wave);
-            dma_slab<BN, ROW, NW>(stage0 + A_BYTES, b_slab + k_even, lane_off, row_bytes, wave);
-            slab(acc, stage1, a_rd, b_rd, half, swz);
-            __syncthreads();
+            slab(acc, fa0, fb0, stage0, stage1, a_slab, b_slab, slab_off(2 * pr + 2, rot, k_steps), ln, row_bytes, wave);
+            slab(acc, fa0, fb0, stage1, stage0, a_slab, b_slab, slab_off(2 * pr + 3, rot, k_steps), ln, row_bytes, wave);
         }
-        if (k_steps & 1) {
-            slab(acc, stage0, a_rd, b_rd, half, swz);
-            __syncthreads();
-        }
+        if (k_steps & 1)
+            slab(acc, fa0, fb0, stage0, stage1, a_slab, b_slab, slab_off(last, rot, k_steps), ln, row_bytes, wave);
+        // drain the re-fetches of the last slab before anything refills the stages
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, true));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
     }
 };
 
@@ -289,13 +389,13 @@ struct RingPipe {
         __builtin_amdgcn_sched_barrier(0);
     }
 
-    static __device__ __forceinline__ void run(f32x16_t (&acc)[TM][TN], const unsigned char* a_slab,
-                                               const unsigned char* b_slab, size_t row_bytes, int K,
-                                               int k_rot, int lane, int wave) {
-        __shared__ __attribute__((aligned(1024))) unsigned char st0[STAGE];
-        __shared__ __attribute__((aligned(1024))) unsigned char st1[STAGE];
-        __shared__ __attribute__((aligned(1024))) unsigned char st2[STAGE];
-        __shared__ __attribute__((aligned(1024))) unsigned char st3[STAGE];
+    template <int I>
+    static __device__ __forceinline__ unsigned char* stage() {
+        __shared__ __attribute__((aligned(1024))) unsigned char st[STAGE];
+        return st;
+    }
+
+    static __device__ __forceinline__ Lane make_lane(size_t row_bytes, int lane, int wave) {
         const int wm = wave / WGN, wn = wave % WGN;
         Lane ln;
         // 16 rows of 64 bytes per 1 KB block: lane l fills row l / 4, physical chunk l % 4
@@ -305,14 +405,35 @@ struct RingPipe {
         const int half = lane >> 5, swz = (lane >> 2) & 3;
         ln.chunk0 = ((0 + half) ^ swz) << 4;
         ln.chunk1 = ((2 + half) ^ swz) << 4;
+        return ln;
+    }
+
+    // slab i of this tile's cyclic walk is slab (i + rot) mod k_steps of K
+    static __device__ __forceinline__ int slab_at(int i, int rot, int k_steps) {
+        const int k = min(i, k_steps - 1) + rot;
+        return k >= k_steps ? k - k_steps : k;
+    }
+
+    static __device__ __forceinline__ void prologue(const unsigned char* a_slab, const unsigned char* b_slab,
+                                                    size_t row_bytes, int K, int k_rot, int lane, int wave) {
+        const Lane ln = make_lane(row_bytes, lane, wave);
+        const int k_steps = K / BK, rot = k_rot % k_steps;
+        fill(stage<0>(), a_slab, b_slab, slab_at(0, rot, k_steps), ln, row_bytes, wave);
+        fill(stage<1>(), a_slab, b_slab, slab_at(1, rot, k_steps), ln, row_bytes, wave);
+        fill(stage<2>(), a_slab, b_slab, slab_at(2, rot, k_steps), ln, row_bytes, wave);
+    }
+
+    static __device__ __forceinline__ void main(f32x16_t (&acc)[TM][TN], const unsigned char* a_slab,
+                                                const unsigned char* b_slab, size_t row_bytes, int K,
+                                                int k_rot, int lane, int wave) {
+        unsigned char* const st0 = stage<0>();
+        unsigned char* const st1 = stage<1>();
+        unsigned char* const st2 = stage<2>();
+        unsigned char* const st3 = stage<3>();
+        const Lane ln = make_lane(row_bytes, lane, wave);
         const int k_steps = K / BK, last = k_steps - 1;
         const int rot = k_rot % k_steps;
-        // slab i of this tile's walk is slab (i + rot) mod k_steps of K
-        auto at = [&](int i) -> int { const int k = min(i, last) + rot; return k >= k_steps ? k - k_steps : k; };
 
-        fill(st0, a_slab, b_slab, at(0), ln, row_bytes, wave);
-        fill(st1, a_slab, b_slab, at(1), ln, row_bytes, wave);
-        fill(st2, a_slab, b_slab, at(2), ln, row_bytes, wave);
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(2 * FILLS, true));
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
@@ -320,10 +441,10 @@ struct RingPipe {
         load_frags<T, TM, TN, ROW>(fa0, fb0, st0, ln.a_rd, ln.b_rd, ln.chunk0);
 
         for (int s = 0; s <= last; s += 4) {
-            step(acc, fa0, fb0, st0, st1, st3, a_slab, b_slab, at(s + 3), ln, row_bytes, wave);
-            step(acc, fa0, fb0, st1, st2, st0, a_slab, b_slab, at(s + 4), ln, row_bytes, wave);
-            step(acc, fa0, fb0, st2, st3, st1, a_slab, b_slab, at(s + 5), ln, row_bytes, wave);
-            step(acc, fa0, fb0, st3, st0, st2, a_slab, b_slab, at(s + 6), ln, row_bytes, wave);
+            step(acc, fa0, fb0, st0, st1, st3, a_slab, b_slab, slab_at(s + 3, rot, k_steps), ln, row_bytes, wave);
+            step(acc, fa0, fb0, st1, st2, st0, a_slab, b_slab, slab_at(s + 4, rot, k_steps), ln, row_bytes, wave);
+            step(acc, fa0, fb0, st2, st3, st1, a_slab, b_slab, slab_at(s + 5, rot, k_steps), ln, row_bytes, wave);
+            step(acc, fa0, fb0, st3, st0, st2, a_slab, b_slab, slab_at(s + 6, rot, k_steps), ln, row_bytes, wave);
         }
         // drain the re-fetches of the last slab before anything refills the stages
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, true));
@@ -354,18 +475,40 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
     const int K = p.K, N = p.N;
     const size_t row_bytes = (size_t)K * sizeof(T);
 
-    // --- wave walk state (uniform across the workgroup) ---
-    int cur_wave = 0;
-    int past_tiles = 0;
-    int cur_m = p.wave_sizes[0] / BM;
-    int cur_n = p.wave_sizes[1] / BN;
-    int off_m = p.wave_offsets[0] / BM;
-    int off_n = p.wave_offsets[1] / BN;
-    int cur_tiles = cur_m * cur_n;
-    int cur_sig = p.signal_offsets[0];
-
+    // --- wave table: the first kLdsWaves rows live in LDS, the walk reads them from there ---
+    constexpr int kLdsWaves = 128;
+    __shared__ int s_waves[kLdsWaves][5];
+    for (int w = tid; w < min(p.num_waves, kLdsWaves); w += 64 * WGM * WGN) {
+        s_waves[w][0] = p.wave_sizes[2 * w] / BM;
+        s_waves[w][1] = p.wave_sizes[2 * w + 1] / BN;
+        s_waves[w][2] = p.wave_offsets[2 * w] / BM;
+        s_waves[w][3] = p.wave_offsets[2 * w + 1] / BN;
+        s_waves[w][4] = p.signal_offsets[w];
+    }
     if (tid == 0) s_abort = 0;
     __syncthreads();
+
+    // --- wave walk state (uniform across the workgroup) ---
+    int cur_wave = -1, past_tiles = 0, cur_tiles = 0;
+    int cur_m = 0, cur_n = 0, off_m = 0, off_n = 0, cur_sig = -1;
+    auto enter_wave = [&](int w) {
+        cur_wave = w;
+        if (w < kLdsWaves) {
+            cur_m = s_waves[w][0];
+            cur_n = s_waves[w][1];
+            off_m = s_waves[w][2];
+            off_n = s_waves[w][3];
+            cur_sig = s_waves[w][4];
+        } else {
+            cur_m = p.wave_sizes[w * 2] / BM;
+            cur_n = p.wave_sizes[w * 2 + 1] / BN;
+            off_m = p.wave_offsets[w * 2] / BM;
+            off_n = p.wave_offsets[w * 2 + 1] / BN;
+            cur_sig = p.signal_offsets[w];
+        }
+        cur_tiles = cur_m * cur_n;
+    };
+    enter_wave(0);
 
     auto wait_flag = [&](int sig) -> bool {
         if (tid == 0) {
@@ -380,6 +523,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
         return s_abort == 0;
     };
 
+    // the reference's consumer waits for wave 0 before it looks at its first tile (template.py:92-97)
     if (!PRODUCER) {
         if (cur_sig >= 0) {
             if (!wait_flag(cur_sig)) return;
@@ -390,29 +534,28 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
     const T* __restrict__ B = reinterpret_cast<const T*>(p.b);
     T* __restrict__ C = reinterpret_cast<T*>(p.c);
 
-    for (int it = 0; it < tiles_here; ++it) {
-        const int tile_id = pid + it * num_sms;
-
+    // Move the walk to `tile_id`; true if that entered a wave whose flag has to be waited for.
+    // -1 wave index afterwards: the table is shorter than the grid (host check failed).
+    auto advance = [&](int tile_id) -> bool {
         bool new_wave = false;
         while (tile_id >= past_tiles + cur_tiles) {
             past_tiles += cur_tiles;
-            ++cur_wave;
-            if (cur_wave >= p.num_waves) return;      // table shorter than the grid: host check failed
-            cur_m = p.wave_sizes[cur_wave * 2] / BM;
-            cur_n = p.wave_sizes[cur_wave * 2 + 1] / BN;
-            off_m = p.wave_offsets[cur_wave * 2] / BM;
-            off_n = p.wave_offsets[cur_wave * 2 + 1] / BN;
-            cur_tiles = cur_m * cur_n;
-            cur_sig = p.signal_offsets[cur_wave];
+            if (cur_wave + 1 >= p.num_waves) {
+                cur_wave = -1;
+                return false;
+            }
+            enter_wave(cur_wave + 1);
             new_wave = true;
         }
-        if (!PRODUCER) {
-            if (new_wave && cur_sig >= 0) {
-                if (!wait_flag(cur_sig)) return;
-            }
-        }
+        return !PRODUCER && new_wave && cur_sig >= 0;
+    };
 
-        // get_pid_mn (template.py:10-18) on the wave-local tile id
+    struct Tile {
+        size_t m0, n0;
+        int k_rot, wave, sig, wave_tiles;
+    };
+    // get_pid_mn (template.py:10-18) on the wave-local tile id, and the tile's K phase
+    auto locate = [&](int tile_id) -> Tile {
         const int local = tile_id - past_tiles;
         const int in_group = p.group_m * cur_n;
         const int group_id = local / in_group;
@@ -420,15 +563,35 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
         const int gsz = min(cur_m - first_m, p.group_m);
         const int pid_m = first_m + (local % gsz) + off_m;
         const int pid_n = (local % in_group) / gsz + off_n;
-
         if (p.visit_log != nullptr && tid == 0) {
             int4 rec = make_int4(pid, cur_wave, pid_m, pid_n);
             reinterpret_cast<int4*>(p.visit_log)[tile_id] = rec;
         }
+        Tile t;
+        t.m0 = (size_t)pid_m * BM;
+        t.n0 = (size_t)pid_n * BN;
+        // Tiles walk K cyclically, neighbouring tiles starting 128 elements apart.  With a
+        // power-of-two row pitch, programs that all sweep K from 0 in lockstep keep hitting the
+        // same few memory channels; four phases spread them while tiles that share a panel of A
+        // or B still stay within 512 elements of each other (L2 reuse).
+        t.k_rot = p.k_stagger ? ((pid_m + pid_n) & 3) * (128 / Pipe::BK) : 0;
+        t.wave = cur_wave;
+        t.sig = cur_sig;
+        t.wave_tiles = cur_tiles;
+        return t;
+    };
+    auto panel_a = [&](const Tile& t) { return reinterpret_cast<const unsigned char*>(A + t.m0 * (size_t)K); };
+    auto panel_b = [&](const Tile& t) { return reinterpret_cast<const unsigned char*>(B + t.n0 * (size_t)K); };
 
-        const size_t m0 = (size_t)pid_m * BM;
-        const size_t n0 = (size_t)pid_n * BN;
+    if (tiles_here == 0) return;
+    if (advance(pid)) {
+        if (!wait_flag(cur_sig)) return;
+    }
+    if (cur_wave < 0) return;
+    Tile tile = locate(pid);
+    Pipe::prologue(panel_a(tile), panel_b(tile), row_bytes, K, tile.k_rot, lane, wave);
 
+    for (int it = 0; it < tiles_here; ++it) {
         f32x16_t acc[TM][TN];
 #pragma unroll
         for (int i = 0; i < TM; ++i)
@@ -437,19 +600,29 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
 #pragma unroll
                 for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-        // Tiles walk K cyclically, neighbouring tiles starting 128 elements apart.  With a
-        // power-of-two row pitch, programs that all sweep K from 0 in lockstep keep hitting the
-        // same few memory channels; four phases spread them while tiles that share a panel of A
-        // or B still stay within 512 elements of each other (L2 reuse).
-        const int k_rot = p.k_stagger ? ((pid_m + pid_n) & 3) * (128 / Pipe::BK) : 0;
-        Pipe::run(acc, reinterpret_cast<const unsigned char*>(A + m0 * (size_t)K),
-                  reinterpret_cast<const unsigned char*>(B + n0 * (size_t)K), row_bytes, K, k_rot, lane, wave);
+        Pipe::main(acc, panel_a(tile), panel_b(tile), row_bytes, K, tile.k_rot, lane, wave);
+
+        // The stages are free: start the next tile's fills before this tile's C is stored, unless
+        // the next tile opens a wave whose flag is still to be waited for (nothing of a chunk may
+        // be read before its flag).
+        const bool has_next = it + 1 < tiles_here;
+        const int next_id = pid + (it + 1) * num_sms;
+        bool gated = false;
+        Tile next = tile;
+        if (has_next) {
+            gated = advance(next_id);
+            if (cur_wave < 0) return;
+            if (!gated) {
+                next = locate(next_id);
+                Pipe::prologue(panel_a(next), panel_b(next), row_bytes, K, next.k_rot, lane, wave);
+            }
+        }
 
         // Epilogue.  With B as the first MFMA operand a lane holds, for column m = lane % 32 of
         // D', rows n = 8g + 4*(lane/32) + 0..3: four consecutive elements of one row of C -> one
         // 8-byte store.
         {
-            T* c_row = C + (m0 + wm * WM + (lane & 31)) * (size_t)N + n0 + wn * WN + 4 * (lane >> 5);
+            T* c_row = C + (tile.m0 + wm * WM + (lane & 31)) * (size_t)N + tile.n0 + wn * WN + 4 * (lane >> 5);
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -463,18 +636,25 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
         }
 
         if (PRODUCER) {
-            if (cur_sig >= 0) {
+            if (tile.sig >= 0) {
                 __threadfence();             // every lane's C stores are visible device-wide
                 __syncthreads();
                 if (tid == 0) {
-                    const int done = __hip_atomic_fetch_add(p.counters + cur_wave, 1, __ATOMIC_RELEASE,
+                    const int done = __hip_atomic_fetch_add(p.counters + tile.wave, 1, __ATOMIC_RELEASE,
                                                             __HIP_MEMORY_SCOPE_AGENT);
-                    if (done == cur_tiles - 1)
-                        __hip_atomic_store(p.flags + cur_sig, 1ull, __ATOMIC_RELEASE,
+                    if (done == tile.wave_tiles - 1)
+                        __hip_atomic_store(p.flags + tile.sig, 1ull, __ATOMIC_RELEASE,
                                            __HIP_MEMORY_SCOPE_SYSTEM);
                 }
             }
         }
+
+        if (has_next && gated) {
+            if (!wait_flag(cur_sig)) return;
+            next = locate(next_id);
+            Pipe::prologue(panel_a(next), panel_b(next), row_bytes, K, next.k_rot, lane, wave);
+        }
+        tile = next;
     }
 }
 
@@ -562,7 +742,7 @@ static int gemm_entry(const syn_gemm_desc* d, hipStream_t stream, bool producer)
     p.k_stagger = (d->options & SYN_GEMM_NO_K_STAGGER) ? 0 : 1;
     const bool eight = (d->options & SYN_GEMM_EIGHT_WAVES) != 0;
     // the ring needs whole groups of four 32-deep slabs
-    const bool ring = !(d->options & SYN_GEMM_PAIR_PIPE) && d->K % 128 == 0;
+    const bool ring = (d->options & SYN_GEMM_RING_PIPE) && d->K % 128 == 0;
 
     if (d->dtype == SYN_DTYPE_BF16) {
         return producer ? dispatch_pipe<__bf16, true>(p, d->block_m, d->block_n, eight, ring, grid, stream)

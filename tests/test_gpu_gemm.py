@@ -56,16 +56,16 @@ def test_consumer_resident_matches_fp32_and_visit_order(hip, dtype, BM, BN):
     c = torch.zeros(M, N, dtype=dtype, device="cuda")
     flags = torch.ones(world, dtype=torch.int64, device="cuda")
     tiles = (M // BM) * (N // BN)
-    # (programs, XCD remap, 8 wavefronts, two-stage pipeline instead of the ring)
+    # (programs, XCD remap, 8 wavefronts, four-stage ring instead of the two-stage pipeline)
     variants = [(256, True, False, False), (24, False, False, True), (7, True, False, False)]
     if (BM, BN) != (128, 128):
         variants += [(256, True, True, False), (13, False, True, True)]
     outputs = []
-    for num_sms, remap, eight, pair in variants:
+    for num_sms, remap, eight, ring in variants:
         c.zero_()
         log = torch.full((tiles, 4), -1, dtype=torch.int32, device="cuda")
         gemm_consumer(ad, bd, c, flags, sizes, offsets, signals, world, num_sms, BM, BN, 64, 8,
-                      cum_tiles=M * N, visit_log=log, xcd_remap=remap, eight_waves=eight, pair_pipe=pair)
+                      cum_tiles=M * N, visit_log=log, xcd_remap=remap, eight_waves=eight, ring_pipe=ring)
         check_status()
         assert _max_rel_err(c, ref) <= REL_TOL
         _check_visits(log, sizes, offsets, signals, M, N, BM, BN, 8, num_sms, M * N, remap)
@@ -75,7 +75,8 @@ def test_consumer_resident_matches_fp32_and_visit_order(hip, dtype, BM, BN):
         assert torch.equal(outputs[0], other)
 
 
-def test_consumer_k_not_multiple_of_128_uses_the_two_stage_pipeline(hip):
+def test_consumer_k_not_multiple_of_128(hip):
+    """Odd slab counts in the two-stage pipeline; a ring request falls back to it."""
     from syncopate_amd.computation.gemm import gemm_consumer
     from syncopate_amd.computation._launch import check_status
 
@@ -87,7 +88,7 @@ def test_consumer_k_not_multiple_of_128_uses_the_two_stage_pipeline(hip):
         for BM, BN, eight in [(256, 256, False), (128, 256, True), (128, 128, False)]:
             c = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
             gemm_consumer(a.cuda(), b.cuda(), c, flags, sizes, offsets, signals, 2, 256, BM, BN,
-                          cum_tiles=M * N, eight_waves=eight)
+                          cum_tiles=M * N, eight_waves=eight, ring_pipe=(K == 192))
             check_status()
             assert _max_rel_err(c, numerics.gemm_fp32(a, b)) <= REL_TOL
 
