@@ -10,13 +10,19 @@
 // increasing order, so an early (already arrived) wave is never queued behind a
 // later one.
 //
-// Data path per 128-wide kv block, 4 wavefronts x 32 q rows each:
+// Data path per 128-row kv block, 4 wavefronts x 32 q rows each:
 //   S^T[kv, q] = K[kv, :] . Q[q, :]      K from LDS (A operand), Q fragments in registers
 //   P^T        = exp2(S^T * scale - m)   per-q statistics are lane-local: lane % 32 == q
-//   O^T[d, q] += V^T[d, kv] . P^T[kv, q] V^T from LDS (transposed while staging)
+//   O^T[d, q] += V^T[d, kv] . P^T[kv, q] V row-major in LDS, read with transposing LDS loads
 // Computing the transposed products keeps each q column in one lane pair, so
 // the softmax needs one cross-lane exchange per block, and the accumulator
 // layout of S^T is already the B-operand layout of the second product.
+//
+// K and V blocks go from HBM straight into LDS (global_load_lds_dwordx4, no register
+// staging): the fill of the next K block is issued as soon as S^T is done and overlaps the
+// softmax and the second product, the fill of the next V block overlaps the next S^T.
+// The kernel stays under 256 registers and 80 KB of LDS, so two workgroups share a compute
+// unit and one's exponentials overlap the other's matrix work.
 #include "common.h"
 
 namespace syn {
@@ -50,11 +56,9 @@ constexpr int kAttnThreads = 256;
 constexpr int kHeadDim = 128;
 constexpr int kBlockM = 128;
 constexpr int kBlockN = 128;
-constexpr int kKRowBytes = kHeadDim * 2;            // 256
-constexpr int kVtPitch = kBlockN * 2 + 8;           // 264: rows of V^T, padded against bank conflicts
-constexpr int kKBytes = kBlockN * kKRowBytes;       // 32768
-constexpr int kVtBytes = kHeadDim * kVtPitch;       // 33792
-constexpr int kAttnLdsBytes = kKBytes + kVtBytes;
+constexpr int kRowBytes = kHeadDim * 2;             // 256: one row of K or V
+constexpr int kBlockBytes = kBlockN * kRowBytes;    // 32768: one kv block of K or of V
+constexpr int kFills = kBlockBytes / 1024 / 4;      // 8 fills of 1 KB per wavefront and block
 
 template <typename T>
 struct AttnMfma;
@@ -78,56 +82,78 @@ struct AttnMfma<_Float16> {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
-// low/high 16-bit halves of two dwords -> one dword
-__device__ __forceinline__ uint32_t pack_lo(uint32_t a, uint32_t b) { return (a & 0xffffu) | (b << 16); }
-__device__ __forceinline__ uint32_t pack_hi(uint32_t a, uint32_t b) { return (a >> 16) | (b & 0xffff0000u); }
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+typedef const __attribute__((address_space(1))) void* global_void_ptr;
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) s16x4_t* lds_s16x4_ptr;
 
+// s_waitcnt immediate (gfx9 encoding): at most `vm` vector-memory operations outstanding
+constexpr int attn_vmcnt(int vm) { return (vm & 0xF) | ((vm >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
 
-// One kv block into registers: K as 8 row-chunks of 16 bytes, V as two 4x8 units.
-template <typename T>
-__device__ __forceinline__ void load_kv_block(u32x4_t (&rk)[8], u32x4_t (&rv)[8], const T* k_src,
-                                              const T* v_src, int n) {
-    const size_t blk = (size_t)n * kBlockN * kHeadDim;
+// One kv block (128 rows of 256 bytes, contiguous in HBM) into LDS.  Wavefront `wave` issues
+// 1 KB fills number wave, wave + 4, ...; lane l lands at byte 16*l of the fill, i.e. row l/16,
+// physical 16-byte chunk l%16, and `lane_off` makes it fetch the logical chunk that lives there.
+__device__ __forceinline__ void dma_kv_block(unsigned char* lds, const unsigned char* src,
+                                             unsigned lane_off, int wave) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
-        rk[i] = *reinterpret_cast<const u32x4_t*>(k_src + blk + (size_t)(16 * i) * kHeadDim);
-#pragma unroll
-    for (int u = 0; u < 2; ++u)
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            rv[4 * u + i] = *reinterpret_cast<const u32x4_t*>(v_src + blk + (size_t)i * kHeadDim + 64 * u);
+    for (int i = 0; i < kFills; ++i) {
+        const int blk = i * 4 + wave;
+        __builtin_amdgcn_global_load_lds((global_void_ptr)(src + blk * 1024 + lane_off),
+                                         (lds_void_ptr)(lds + blk * 1024), 16, 0, 0);
+    }
 }
 
+// LDS layouts (row = kv position in the block, 16 chunks of 16 bytes per row):
+//   K: logical chunk c of row r at physical chunk c ^ (r & 15)        (128-bit row reads of
+//      32 consecutive rows at one logical chunk hit 16 distinct chunks twice: conflict free)
+//   V: logical chunk c of row r at physical chunk c ^ ((r & 3) << 2)  (a transposing read
+//      touches 4 consecutive rows x 64 bytes: the 4 rows land in 4 distinct 64-byte granules)
+//
+// ds_read_b64_tr_b16: in every group of 16 lanes, lane i supplies the address of 4 consecutive
+// 16-bit elements M[i][0..3] and receives M[4e + i/4][i%4] for e = 0..3.  With lane i pointing
+// at V[kv + i/4][d0 + 4*(i%4) ...] it gets V[kv + 0..3][d0 + i]: four kv values of its own
+// column - half of an MFMA A-operand fragment of V^T.
+
 template <typename T>
-__global__ void __launch_bounds__(kAttnThreads) attn_fwd_kernel(const AttnParams p) {
+__global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnParams p) {
     typedef typename AttnMfma<T>::frag_t frag_t;
     typedef T vec4_t __attribute__((ext_vector_type(4)));
 
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    __shared__ __attribute__((aligned(1024))) unsigned char k_lds[kBlockBytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char v_lds[kBlockBytes];
     __shared__ int s_abort;
-    unsigned char* k_lds = smem;
-    unsigned char* vt_lds = smem + kKBytes;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 31;
     const int half = lane >> 5;
 
     if (tid == 0) s_abort = 0;
     __syncthreads();
 
-    // K staging: 16-byte chunk c of row (tid/16 + 16*i)
-    const int k_c = tid & 15;
-    const int k_row = tid >> 4;
-    const int k_st = k_row * kKRowBytes + ((k_c ^ (k_row & 15)) << 4);
-    // V staging: unit (a, b) = 4 kv rows x 8 d columns, two units per thread
-    const int v_a = tid & 31;
-    const int v_b = tid >> 5;          // 0..7, second unit at +8
+    // fills: lane l covers row l/16 of its 4-row group; rows of fill `blk` are 4*blk + l/16 and
+    // blk % 4 == wave, so (row & 15) == 4*wave + l/16 and (row & 3) == l/16
+    const int f_row = lane >> 4, f_c = lane & 15;
+    const unsigned k_fill_off = (unsigned)(f_row * kRowBytes + ((f_c ^ (4 * wave + f_row)) << 4));
+    const unsigned v_fill_off = (unsigned)(f_row * kRowBytes + ((f_c ^ (f_row << 2)) << 4));
+    // K fragment reads: row 32*j + r, logical chunk 2*ks + half
+    const int k_rd = r * kRowBytes;
+    // V^T fragment reads: 16-lane group g = lane/16: d0 = 16*(g & 1), kv offset 4*half (+8 for
+    // the upper half of the fragment); lane i of the group: row +i/4, columns d0 + 4*(i%4)
+    const int i16 = lane & 15;
+    const int v_row = 4 * half + (i16 >> 2);                       // & 3 == i16 >> 2
+    const int v_col_bytes = (16 * ((lane >> 4) & 1) + 4 * (i16 & 3)) * 2;    // 0..63
+    // physical offset of (row v_row + 16*t2 [+8], d tile i): chunk (4*i + v_col_bytes/16) ^ ((row&3)<<2)
+    const int v_swz = (i16 >> 2) << 2;
+    int v_rd[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        v_rd[i] = v_row * kRowBytes + ((((4 * i + (v_col_bytes >> 4)) ^ v_swz) << 4) | (v_col_bytes & 15));
 
     const T* __restrict__ Q = reinterpret_cast<const T*>(p.q);
-    const T* __restrict__ K = reinterpret_cast<const T*>(p.k);
-    const T* __restrict__ V = reinterpret_cast<const T*>(p.v);
+    const unsigned char* __restrict__ K = reinterpret_cast<const unsigned char*>(p.k);
+    const unsigned char* __restrict__ V = reinterpret_cast<const unsigned char*>(p.v);
     T* __restrict__ O = reinterpret_cast<T*>(p.o);
 
     for (int tile_id = blockIdx.x; tile_id < p.num_tiles; tile_id += gridDim.x) {
@@ -173,8 +199,12 @@ __global__ void __launch_bounds__(kAttnThreads) attn_fwd_kernel(const AttnParams
         const size_t head = (size_t)z * p.H + h;
         const int q_row = qb * kBlockM + wave * 32 + r;              // this lane's q position
         const T* q_src = Q + (head * p.Sq + q_row) * kHeadDim + 8 * half;
-        const T* k_base = K + head * (size_t)p.Skv * kHeadDim;
-        const T* v_base = V + head * (size_t)p.Skv * kHeadDim;
+        const unsigned char* k_base = K + head * (size_t)p.Skv * kRowBytes;
+        const unsigned char* v_base = V + head * (size_t)p.Skv * kRowBytes;
+
+        // both stages are free here: every wavefront has passed the barrier that ends a tile
+        dma_kv_block(k_lds, k_base + (size_t)kv_lo * kBlockBytes, k_fill_off, wave);
+        dma_kv_block(v_lds, v_base + (size_t)kv_lo * kBlockBytes, v_fill_off, wave);
 
         frag_t qf[8];
 #pragma unroll
@@ -187,36 +217,16 @@ __global__ void __launch_bounds__(kAttnThreads) attn_fwd_kernel(const AttnParams
             for (int e = 0; e < 16; ++e) o_acc[i][e] = 0.f;
         float m_i = -INFINITY;
         float l_i = 0.f;     // this lane's share of the row sum (its 64 of every 128 kv columns)
-
-        u32x4_t rk[8], rv[8];
-        const T* k_src = k_base + (size_t)k_row * kHeadDim + k_c * 8;
-        const T* v_src = v_base + (size_t)(4 * v_a) * kHeadDim + v_b * 8;
-        load_kv_block<T>(rk, rv, k_src, v_src, kv_lo);
+        // the Q loads must not be counted among the fills below
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("" ::"v"(qf[0]), "v"(qf[1]), "v"(qf[2]), "v"(qf[3]), "v"(qf[4]), "v"(qf[5]), "v"(qf[6]), "v"(qf[7]));
 
         for (int n = kv_lo; n < kv_end; ++n) {
-            __syncthreads();                 // LDS of the previous block has been consumed
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-                *reinterpret_cast<u32x4_t*>(k_lds + k_st + i * 16 * kKRowBytes) = rk[i];
-#pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                // transpose 4 kv x 8 d: for each d, the 4 kv values become one 8-byte word
-                const u32x4_t x0 = rv[4 * u + 0], x1 = rv[4 * u + 1], x2 = rv[4 * u + 2], x3 = rv[4 * u + 3];
-                unsigned char* dst = vt_lds + ((v_b + 8 * u) * 8) * kVtPitch + v_a * 8;
-#pragma unroll
-                for (int dw = 0; dw < 4; ++dw) {
-                    uint2 even, odd;
-                    even.x = pack_lo(x0[dw], x1[dw]);
-                    even.y = pack_lo(x2[dw], x3[dw]);
-                    odd.x = pack_hi(x0[dw], x1[dw]);
-                    odd.y = pack_hi(x2[dw], x3[dw]);
-                    *reinterpret_cast<uint2*>(dst + (2 * dw) * kVtPitch) = even;
-                    *reinterpret_cast<uint2*>(dst + (2 * dw + 1) * kVtPitch) = odd;
-                }
-            }
-            __syncthreads();
-            // prefetch the next block (the last iteration re-reads its own block: no branch)
-            load_kv_block<T>(rk, rv, k_src, v_src, min(n + 1, kv_end - 1));
+            // ---- K block n has landed (its fills are older than V's) ----
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_waitcnt(attn_vmcnt(kFills));
+            __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_sched_barrier(0);
 
             // ---- S^T = K . Q^T : 4 tiles of [32 kv, 32 q] ----
             f32x16_t s[4];
@@ -230,10 +240,17 @@ __global__ void __launch_bounds__(kAttnThreads) attn_fwd_kernel(const AttnParams
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const frag_t kf = *reinterpret_cast<const frag_t*>(
-                        k_lds + (32 * j + r) * kKRowBytes + chunk);
+                        k_lds + 32 * j * kRowBytes + k_rd + chunk);
                     s[j] = AttnMfma<T>::run(kf, qf[ks], s[j]);
                 }
             }
+
+            // ---- every wavefront is done with K: fetch the next K block behind the softmax ----
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_waitcnt(0xc07f);          // lgkmcnt(0): own LDS reads have returned
+            __builtin_amdgcn_s_barrier();
+            dma_kv_block(k_lds, k_base + (size_t)min(n + 1, kv_end - 1) * kBlockBytes, k_fill_off, wave);
+            __builtin_amdgcn_sched_barrier(0);
 
             // ---- online softmax in base 2 ----
             if (p.causal && n == qb) {
@@ -266,26 +283,47 @@ __global__ void __launch_bounds__(kAttnThreads) attn_fwd_kernel(const AttnParams
                     pf[2 * j + (e >> 3)][e & 7] = (T)pe;
                 }
             l_i = l_i * alpha + row_sum;
+            // rescale O only when some row's maximum moved (wavefront-uniform test)
+            if (__builtin_amdgcn_ballot_w64(m_new != m_i) != 0) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) o_acc[i][e] *= alpha;
+            }
             m_i = m_new;
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) o_acc[i][e] *= alpha;
+
+            // ---- V block n has landed (only the next K block's fills are newer) ----
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_waitcnt(attn_vmcnt(kFills));
+            __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_sched_barrier(0);
 
             // ---- O^T += V^T . P^T ----
 #pragma unroll
             for (int t2 = 0; t2 < 8; ++t2) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const unsigned char* src = vt_lds + (32 * i + r) * kVtPitch + (16 * t2 + 4 * half) * 2;
-                    const uint2 lo = *reinterpret_cast<const uint2*>(src);
-                    const uint2 hi = *reinterpret_cast<const uint2*>(src + 16);
-                    const u32x4_t both = {lo.x, lo.y, hi.x, hi.y};
+                    const unsigned char* src = v_lds + 16 * t2 * kRowBytes + v_rd[i];
+                    const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)src);
+                    const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(src + 8 * kRowBytes));
+                    typedef short s16x8_t __attribute__((ext_vector_type(8)));
+                    const s16x8_t both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                     const frag_t vf = __builtin_bit_cast(frag_t, both);
                     o_acc[i] = AttnMfma<T>::run(vf, pf[t2], o_acc[i]);
                 }
             }
+
+            // ---- every wavefront is done with V: fetch the next V block behind the next S^T ----
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_waitcnt(0xc07f);
+            __builtin_amdgcn_s_barrier();
+            dma_kv_block(v_lds, v_base + (size_t)min(n + 1, kv_end - 1) * kBlockBytes, v_fill_off, wave);
+            __builtin_amdgcn_sched_barrier(0);
         }
+        // the re-fetches of the last block land before anything refills the stages or exits
+        __builtin_amdgcn_s_waitcnt(attn_vmcnt(0));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
 
         // ---- epilogue: lse2 = m + log2(l), O = acc / l (template.py:307-309) ----
         const float l_tot = l_i + __shfl_xor(l_i, 32);
@@ -354,17 +392,7 @@ __global__ void __launch_bounds__(kAttnThreads) attn_fwd_kernel(const AttnParams
 
 template <typename T>
 static int launch_attn(const AttnParams& p, int grid, hipStream_t stream) {
-    static bool attr_done[64] = {};
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return (int)e;
-    if (dev >= 0 && dev < 64 && !attr_done[dev]) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_fwd_kernel<T>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, kAttnLdsBytes);
-        if (e != hipSuccess) return (int)e;
-        attr_done[dev] = true;
-    }
-    hipLaunchKernelGGL((attn_fwd_kernel<T>), dim3(grid), dim3(kAttnThreads), kAttnLdsBytes, stream, p);
+    hipLaunchKernelGGL((attn_fwd_kernel<T>), dim3(grid), dim3(kAttnThreads), 0, stream, p);
     return (int)hipGetLastError();
 }
 
