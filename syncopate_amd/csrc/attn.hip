@@ -23,6 +23,8 @@
 // softmax and the second product, the fill of the next V block overlaps the next S^T.
 // The kernel stays under 256 registers and 80 KB of LDS, so two workgroups share a compute
 // unit and one's exponentials overlap the other's matrix work.
+#include <type_traits>
+
 #include "common.h"
 
 namespace syn {
@@ -151,6 +153,10 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
     for (int i = 0; i < 4; ++i)
         v_rd[i] = v_row * kRowBytes + ((((4 * i + (v_col_bytes >> 4)) ^ v_swz) << 4) | (v_col_bytes & 15));
 
+    int k_chunk[8];
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) k_chunk[ks] = ((2 * ks + half) ^ (r & 15)) << 4;
+
     const T* __restrict__ Q = reinterpret_cast<const T*>(p.q);
     const unsigned char* __restrict__ K = reinterpret_cast<const unsigned char*>(p.k);
     const unsigned char* __restrict__ V = reinterpret_cast<const unsigned char*>(p.v);
@@ -221,27 +227,46 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
         __builtin_amdgcn_sched_barrier(0);
         asm volatile("" ::"v"(qf[0]), "v"(qf[1]), "v"(qf[2]), "v"(qf[3]), "v"(qf[4]), "v"(qf[5]), "v"(qf[6]), "v"(qf[7]));
 
-        for (int n = kv_lo; n < kv_end; ++n) {
+        // one kv block; MASK: the causal diagonal block (kv positions beyond a q row are masked)
+        auto kv_block = [&](const int n, auto mask_tag) {
+            constexpr bool MASK = decltype(mask_tag)::value;
             // ---- K block n has landed (its fills are older than V's) ----
             __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_waitcnt(attn_vmcnt(kFills));
             __builtin_amdgcn_s_barrier();
             __builtin_amdgcn_sched_barrier(0);
 
-            // ---- S^T = K . Q^T : 4 tiles of [32 kv, 32 q] ----
+            // ---- S^T = K . Q^T : 4 tiles of [32 kv, 32 q]; fragments of step ks+1 are read
+            //      while step ks is multiplied ----
             f32x16_t s[4];
+            {
+                const f32x16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                frag_t kf[2][4];
+                const unsigned char* k_row = k_lds + k_rd;
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+                for (int j = 0; j < 4; ++j)
+                    kf[0][j] = *reinterpret_cast<const frag_t*>(k_row + 32 * j * kRowBytes + k_chunk[0]);
+                __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);     // the four reads of step 0 go first
 #pragma unroll
-                for (int e = 0; e < 16; ++e) s[j][e] = 0.f;
+                for (int ks = 0; ks < 8; ++ks) {
+                    if (ks < 7) {
 #pragma unroll
-            for (int ks = 0; ks < 8; ++ks) {
-                const int chunk = ((2 * ks + half) ^ (r & 15)) << 4;
+                        for (int j = 0; j < 4; ++j)
+                            kf[(ks + 1) & 1][j] = *reinterpret_cast<const frag_t*>(
+                                k_row + 32 * j * kRowBytes + k_chunk[ks + 1]);
+                    }
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const frag_t kf = *reinterpret_cast<const frag_t*>(
-                        k_lds + 32 * j * kRowBytes + k_rd + chunk);
-                    s[j] = AttnMfma<T>::run(kf, qf[ks], s[j]);
+                    for (int j = 0; j < 4; ++j)
+                        s[j] = AttnMfma<T>::run(kf[ks & 1][j], qf[ks], ks == 0 ? zero : s[j]);
+                    if (ks < 7) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                        }
+                    } else {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+                    }
                 }
             }
 
@@ -253,14 +278,13 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
             __builtin_amdgcn_sched_barrier(0);
 
             // ---- online softmax in base 2 ----
-            if (p.causal && n == qb) {
+            if constexpr (MASK) {
+                const int lim = q_row - n * kBlockN - 4 * half;     // mask where 32j + 8(e/4) + e%4 > lim
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
 #pragma unroll
-                    for (int e = 0; e < 16; ++e) {
-                        const int kv_pos = n * kBlockN + 32 * j + 8 * (e >> 2) + 4 * half + (e & 3);
-                        if (kv_pos > q_row) s[j][e] = -INFINITY;
-                    }
+                    for (int e = 0; e < 16; ++e)
+                        if (32 * j + 8 * (e >> 2) + (e & 3) > lim) s[j][e] = -INFINITY;
             }
             float mx = -INFINITY;
 #pragma unroll
@@ -298,18 +322,41 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
             __builtin_amdgcn_s_barrier();
             __builtin_amdgcn_sched_barrier(0);
 
-            // ---- O^T += V^T . P^T ----
-#pragma unroll
-            for (int t2 = 0; t2 < 8; ++t2) {
+            // ---- O^T += V^T . P^T; the fragments of step t2+1 are read while step t2 is multiplied ----
+            {
+                typedef short s16x8_t __attribute__((ext_vector_type(8)));
+                s16x4_t vlo[2][4], vhi[2][4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const unsigned char* src = v_lds + 16 * t2 * kRowBytes + v_rd[i];
-                    const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)src);
-                    const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(src + 8 * kRowBytes));
-                    typedef short s16x8_t __attribute__((ext_vector_type(8)));
-                    const s16x8_t both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                    const frag_t vf = __builtin_bit_cast(frag_t, both);
-                    o_acc[i] = AttnMfma<T>::run(vf, pf[t2], o_acc[i]);
+                    vlo[0][i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(v_lds + v_rd[i]));
+                    vhi[0][i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(v_lds + v_rd[i] + 8 * kRowBytes));
+                }
+                __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);     // the eight reads of step 0 go first
+#pragma unroll
+                for (int t2 = 0; t2 < 8; ++t2) {
+                    if (t2 < 7) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const unsigned char* src = v_lds + 16 * (t2 + 1) * kRowBytes + v_rd[i];
+                            vlo[(t2 + 1) & 1][i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)src);
+                            vhi[(t2 + 1) & 1][i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(src + 8 * kRowBytes));
+                        }
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const s16x4_t lo = vlo[t2 & 1][i], hi = vhi[t2 & 1][i];
+                        const s16x8_t both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                        o_acc[i] = AttnMfma<T>::run(__builtin_bit_cast(frag_t, both), pf[t2], o_acc[i]);
+                    }
+                    if (t2 < 7) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                        }
+                    } else {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+                    }
                 }
             }
 
@@ -319,7 +366,12 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
             __builtin_amdgcn_s_barrier();
             dma_kv_block(v_lds, v_base + (size_t)min(n + 1, kv_end - 1) * kBlockBytes, v_fill_off, wave);
             __builtin_amdgcn_sched_barrier(0);
-        }
+        };
+        // under a causal mask the diagonal block, if this tile reaches it, is the last one
+        const bool diagonal = p.causal && kv_end - 1 == qb;
+        const int plain_end = diagonal ? kv_end - 1 : kv_end;
+        for (int n = kv_lo; n < plain_end; ++n) kv_block(n, std::false_type{});
+        if (diagonal) kv_block(qb, std::true_type{});
         // the re-fetches of the last block land before anything refills the stages or exits
         __builtin_amdgcn_s_waitcnt(attn_vmcnt(0));
         __builtin_amdgcn_s_barrier();
