@@ -1,8 +1,8 @@
 // Chunked ring reduce of GEMM+RS for gfx950 (tests/test_gemm_rs.py:22-72 of the reference):
 //   out[e] = local[rank*chunk + e] + sum_{i=1..W-1} recv[((rank+i) % W)*chunk + e]
-// A pure HBM stream: W reads and one write of 16 bytes per lane, all W loads of
-// an element group issued before the first add so that each lane keeps W
-// 128-bit requests in flight.
+// A pure HBM stream: W reads and one write of 16 bytes per lane and element group,
+// four groups per lane and pass, all 4 W loads issued before the first add so that
+// each lane keeps 4 W 128-bit requests in flight.
 #include "common.h"
 
 namespace syn {
@@ -41,36 +41,63 @@ __device__ __forceinline__ u32x4_t add8(const u32x4_t* parts, int count) {
     return __builtin_bit_cast(u32x4_t, r);
 }
 
+constexpr int kVecsPerThread = 4;      // 16-byte groups per lane and pass: 4 x W loads in flight
+
 template <typename T, bool ROUND_EACH, int W>
 __global__ void __launch_bounds__(kReduceThreads)
 ring_reduce_kernel(const u32x4_t* __restrict__ recv, const u32x4_t* __restrict__ local,
                    u32x4_t* __restrict__ out, int world, int rank, int64_t chunk_vecs) {
     // W > 0: world known at compile time (fully unrolled loads); W == 0: generic
+    constexpr int kParts = W > 0 ? W : kMaxWorld;
+    constexpr int64_t kGroup = (int64_t)kReduceThreads * kVecsPerThread;
     const int w = W > 0 ? W : world;
-    const int64_t stride = (int64_t)gridDim.x * kReduceThreads;
-    for (int64_t v = (int64_t)blockIdx.x * kReduceThreads + threadIdx.x; v < chunk_vecs; v += stride) {
-        u32x4_t parts[W > 0 ? W : kMaxWorld];
-        parts[0] = __builtin_nontemporal_load(local + (int64_t)rank * chunk_vecs + v);
+    const u32x4_t* own = local + (int64_t)rank * chunk_vecs;
+    for (int64_t g0 = (int64_t)blockIdx.x * kGroup; g0 < chunk_vecs; g0 += (int64_t)gridDim.x * kGroup) {
+        const int64_t v0 = g0 + threadIdx.x;
+        if (W > 0 && g0 + kGroup <= chunk_vecs) {
+            // a full group (world known at compile time): every load of the pass is issued before the first add
+            u32x4_t parts[kVecsPerThread][kParts];
 #pragma unroll
-        for (int i = 1; i < (W > 0 ? W : kMaxWorld); ++i) {
-            if (i < w) {
-                int src = rank + i;
-                if (src >= w) src -= w;
-                parts[i] = __builtin_nontemporal_load(recv + (int64_t)src * chunk_vecs + v);
+            for (int u = 0; u < kVecsPerThread; ++u) {
+                const int64_t v = v0 + u * kReduceThreads;
+                parts[u][0] = __builtin_nontemporal_load(own + v);
+#pragma unroll
+                for (int i = 1; i < kParts; ++i) {
+                    if (i < w) {
+                        int src = rank + i;
+                        if (src >= w) src -= w;
+                        parts[u][i] = __builtin_nontemporal_load(recv + (int64_t)src * chunk_vecs + v);
+                    }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kVecsPerThread; ++u)
+                __builtin_nontemporal_store(add8<T, ROUND_EACH>(parts[u], w), out + v0 + u * kReduceThreads);
+        } else {
+            for (int64_t v = v0; v < chunk_vecs; v += kReduceThreads) {
+                u32x4_t parts[kParts];
+                parts[0] = __builtin_nontemporal_load(own + v);
+#pragma unroll
+                for (int i = 1; i < kParts; ++i) {
+                    if (i < w) {
+                        int src = rank + i;
+                        if (src >= w) src -= w;
+                        parts[i] = __builtin_nontemporal_load(recv + (int64_t)src * chunk_vecs + v);
+                    }
+                }
+                __builtin_nontemporal_store(add8<T, ROUND_EACH>(parts, w), out + v);
             }
         }
-        const u32x4_t r = add8<T, ROUND_EACH>(parts, w);
-        __builtin_nontemporal_store(r, out + v);
     }
 }
 
 template <typename T, bool ROUND_EACH>
 static int launch_reduce(const void* recv, const void* local, void* out, int world, int rank,
                          int64_t chunk_vecs, hipStream_t stream) {
-    // one 16-byte group per lane and pass; enough workgroups to cover the chunk
-    // up to 16 per CU, beyond that lanes loop
-    int64_t blocks = (chunk_vecs + kReduceThreads - 1) / kReduceThreads;
-    const int64_t cap = 256 * 16;
+    // a workgroup takes 1024 16-byte groups per pass; two workgroups per CU, beyond that they loop
+    const int64_t group = (int64_t)kReduceThreads * kVecsPerThread;
+    int64_t blocks = (chunk_vecs + group - 1) / group;
+    const int64_t cap = 256 * 2;
     if (blocks > cap) blocks = cap;
     if (blocks < 1) blocks = 1;
     const dim3 grid((unsigned)blocks), block(kReduceThreads);

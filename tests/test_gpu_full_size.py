@@ -1,0 +1,171 @@
+"""The headline configurations at their full sizes, checked through properties that do not need a
+CPU pass over the whole problem: the tile-visit log against the oracle (integer work, cheap at
+any size), sampled rows against torch's fp32 matmul / attention on the GPU (library routines),
+bitwise agreement between launch configurations, counters and flags, invariance of attention
+under the arrival order of the kv chunks."""
+
+import pytest
+import torch
+
+from oracle import visit_order
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-2
+
+
+def _rel(out, ref):
+    return ((out.float() - ref.float()).abs().max() / ref.float().abs().max()).item()
+
+
+def _check_visit_log(log, sizes, offsets, signals, M, N, BM, BN, num_sms):
+    want = visit_order.gemm_tile_visits(sizes, offsets, signals, M=M, N=N, BM=BM, BN=BN, group_m=8,
+                                        num_sms=num_sms, cum_tiles=M * N)
+    got = log.cpu().view(-1, 4).tolist()
+    assert len(want) == (M // BM) * (N // BN)
+    for v in want:
+        assert got[v["tile_id"]] == [v["pid"], v["wave"], v["pid_m"], v["pid_n"]], v
+
+
+def test_ag_gemm_8192x8192x3584(hip):
+    """AG+GEMM of rank 0 of 8 (chunks of 1024 rows in swizzled order), every chunk resident."""
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.gemm import gemm_consumer
+
+    M, K, N, world, rank = 8192, 8192, 3584, 8, 0
+    g = torch.Generator(device="cuda").manual_seed(0)
+    a = (0.02 * torch.randn(M, K, device="cuda", generator=g)).bfloat16()
+    b = (0.02 * torch.randn(N, K, device="cuda", generator=g)).bfloat16()
+    rows = M // world
+    sizes = [[rows, N]] * world
+    offsets = [[((rank + k) % world) * rows, 0] for k in range(world)]
+    signals = [-1] + list(range(world - 1))
+    flags = torch.ones(world - 1, dtype=torch.int64, device="cuda")
+    sample = torch.arange(5, M, 389, device="cuda")
+    ref = a[sample].float() @ b.float().t()
+
+    outputs = []
+    # (BM, BN, programs, 8 wavefronts, ring pipeline)
+    for BM, BN, num_sms, eight, ring in [(256, 256, 224, False, False), (256, 256, 256, True, False),
+                                         (256, 256, 131, True, True), (128, 256, 224, False, False)]:
+        c = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
+        log = torch.full(((M // BM) * (N // BN), 4), -1, dtype=torch.int32, device="cuda")
+        gemm_consumer(a, b, c, flags, sizes, offsets, signals, world, num_sms, BM, BN, 64, 8,
+                      cum_tiles=M * N, visit_log=log, xcd_remap=False, eight_waves=eight, ring_pipe=ring)
+        check_status()
+        assert _rel(c[sample], ref) <= REL_TOL
+        _check_visit_log(log, sizes, offsets, signals, M, N, BM, BN, num_sms)
+        outputs.append((BM, BN, c))
+    # one tile shape -> one order of the fp32 sums, whatever the grid, workgroup shape or pipeline
+    same_tile = [c for BM, BN, c in outputs if (BM, BN) == (256, 256)]
+    for other in same_tile[1:]:
+        assert torch.equal(same_tile[0], other)
+    # other tile shapes rotate the K walk differently: equal to rounding
+    assert _rel(outputs[-1][2], outputs[0][2]) <= 2e-2
+
+
+def test_gemm_rs_producer_8192x8192x3584(hip):
+    """GEMM+RS producer of rank 0 of 8: partial C (8192, 8192) written in wave order
+    1, 2, ..., 7, 0; counters and flags complete; then the chunked reduce over 8 partials."""
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.gemm import gemm_producer
+    from syncopate_amd.computation.reduce import ring_reduce
+
+    M, K, N, world, rank, BM, BN = 8192, 3584, 8192, 8, 0, 256, 256
+    g = torch.Generator(device="cuda").manual_seed(0)
+    a = (0.02 * torch.randn(M, K, device="cuda", generator=g)).bfloat16()
+    b = (0.02 * torch.randn(N, K, device="cuda", generator=g)).bfloat16()
+    rows = M // world
+    order = [(rank + k + 1) % world for k in range(world)]
+    sizes = [[rows, N]] * world
+    offsets = [[ch * rows, 0] for ch in order]
+    signals = list(range(world))
+    flags = torch.zeros(world, dtype=torch.int64, device="cuda")
+    counters = torch.zeros(world, dtype=torch.int32, device="cuda")
+    c = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    log = torch.full(((M // BM) * (N // BN), 4), -1, dtype=torch.int32, device="cuda")
+    gemm_producer(a, b, c, flags, sizes, offsets, signals, 224, BM, BN, 64, 8, cum_tiles=M * N,
+                  counter_buffer=counters, visit_log=log, xcd_remap=False)
+    check_status()
+    assert counters.tolist() == [(rows // BM) * (N // BN)] * world
+    assert flags.tolist() == [1] * world
+    assert not torch.isnan(c).any()
+    sample = torch.arange(3, M, 411, device="cuda")
+    assert _rel(c[sample], a[sample].float() @ b.float().t()) <= REL_TOL
+    _check_visit_log(log, sizes, offsets, signals, M, N, BM, BN, 224)
+
+    # the reduce at its full size: own block of the partial plus 7 received partials
+    recv = torch.randn(world, rows, N, device="cuda", generator=g).bfloat16()
+    out = torch.empty(rows, N, dtype=torch.bfloat16, device="cuda")
+    ring_reduce(recv, out, c, rank)
+    acc = c[rank * rows:(rank + 1) * rows].clone()
+    for i in range(1, world):
+        acc = acc + recv[(rank + i) % world]          # torch adds bf16 tensors with one rounding per add
+    assert torch.equal(out, acc)
+
+
+def _attn_tables(B, H, Sq, chunk, order, signals):
+    offsets = [[0, 0, 0, o * chunk] for o in order]
+    sizes = [[B, H, Sq, chunk]] * len(order)
+    cums = [(i + 1) * B * H * Sq for i in range(len(order))]
+    return dict(wave_offsets=offsets, wave_sizes=sizes, cum_wave_sizes=cums, signal_offsets=signals,
+                cum_tiles=cums[-1])
+
+
+def test_allgather_attention_4096x32768_double_ring_order(hip):
+    """AG attention of rank 0 of 8: the local 4096 q rows against 32768 kv rows arriving as 8
+    chunks in double-ring order; sampled heads against torch's attention in fp32 on the GPU, and
+    the same result (to rounding) for a different arrival order."""
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.attn import attention_forward
+
+    B, H, Sq, Skv, D, chunks = 1, 32, 4096, 32768, 128, 8
+    g = torch.Generator(device="cuda").manual_seed(0)
+    q = torch.randn(B, H, Sq, D, device="cuda", generator=g).bfloat16()
+    k = torch.randn(B, H, Skv, D, device="cuda", generator=g).bfloat16()
+    v = torch.randn(B, H, Skv, D, device="cuda", generator=g).bfloat16()
+    flags = torch.ones(chunks, dtype=torch.int64, device="cuda")
+    scale = D ** -0.5
+    ring = _attn_tables(B, H, Sq, Skv // chunks, [0, 1, 7, 6, 4, 5, 3, 2], [-1, 0, 4, 1, 5, 2, 6, 3])
+    o, lse = attention_forward(q, k, v, scale, signal_ptr=flags, return_lse=True, **ring)
+    check_status()
+    for h in (0, 13, 31):
+        s = (q[0, h].float() @ k[0, h].float().t()) * scale
+        ref = torch.softmax(s, dim=-1) @ v[0, h].float()
+        assert _rel(o[0, h], ref) <= REL_TOL
+        assert (lse[0, h] - torch.logsumexp(s, dim=-1) / 0.6931471805599453).abs().max().item() <= 2e-2
+    plain = _attn_tables(B, H, Sq, Skv // chunks, list(range(chunks)), [-1] + list(range(chunks - 1)))
+    o2 = attention_forward(q, k, v, scale, signal_ptr=flags, num_programs=512, **plain)
+    check_status()
+    # two results that are each within REL_TOL of the fp32 value (the partial O is rounded to bf16 at
+    # every merge, as in the reference) are within twice that of each other
+    assert _rel(o2, o) <= 2 * REL_TOL
+    for h in (5, 22):
+        s = (q[0, h].float() @ k[0, h].float().t()) * scale
+        assert _rel(o2[0, h], torch.softmax(s, dim=-1) @ v[0, h].float()) <= REL_TOL
+
+
+def test_all2all_attention_16384_causal(hip):
+    """Ulysses-style attention over the whole sequence (S = 16384, 4 local heads), kv in 8 chunks
+    of 2048, causal; against torch's causal attention on sampled heads."""
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.attn import attention_forward
+
+    B, H, S, D, chunks = 1, 4, 16384, 128, 8
+    g = torch.Generator(device="cuda").manual_seed(0)
+    q = torch.randn(B, H, S, D, device="cuda", generator=g).bfloat16()
+    k = torch.randn(B, H, S, D, device="cuda", generator=g).bfloat16()
+    v = torch.randn(B, H, S, D, device="cuda", generator=g).bfloat16()
+    flags = torch.ones(chunks, dtype=torch.int64, device="cuda")
+    scale = D ** -0.5
+    tables = _attn_tables(B, H, S, S // chunks, list(range(chunks)), list(range(chunks)))
+    for causal in (True, False):
+        o = attention_forward(q, k, v, scale, signal_ptr=flags, causal=causal, **tables)
+        check_status()
+        for h in (0, 3):
+            s = (q[0, h].float() @ k[0, h].float().t()) * scale
+            if causal:
+                s = s.masked_fill(torch.ones(S, S, dtype=torch.bool, device="cuda").triu(1), float("-inf"))
+            ref = torch.softmax(s, dim=-1) @ v[0, h].float()
+            assert _rel(o[0, h], ref) <= REL_TOL
+            del s, ref
