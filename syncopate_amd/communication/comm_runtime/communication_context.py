@@ -12,6 +12,10 @@ the word.  Only the ops of `rank` are executed, in exactly the order the op
 list prescribes, so a consumer kernel launched on the compute stream really
 overlaps with data arriving chunk by chunk.
 
+`execute_mesh` replays the op lists of ALL ranks on one stream, in an order that
+honours every flag wait, for plans whose data reaches this rank through its
+neighbours' forwarding (ring, double ring).
+
 On a multi-GPU node the same op list would be replayed with the peers'
 buffers mapped through IPC and one stream per peer link; that path is not
 built here.
@@ -87,10 +91,12 @@ class CommContext:
 
     # ---- flags and stream ordering -------------------------------------------
 
-    def reset_signals(self) -> None:
+    def reset_signals(self, whole_mesh: bool = False) -> None:
+        """Zero this rank's flag words (every simulated rank's with `whole_mesh`)."""
         for group in (self.recv_signal_bufs, self.transit_signal_bufs, self.compute_signal_bufs):
             if group:
-                group[self.local_rank].fill_(0)
+                for r in (range(len(group)) if whole_mesh else (self.local_rank,)):
+                    group[r].fill_(0)
 
     def start_after(self, stream: Optional[torch.cuda.Stream] = None) -> None:
         """Communication streams start once `stream` has reached this point."""
@@ -115,65 +121,106 @@ class CommContext:
 
     def execute(self, neglect_local: bool = False) -> None:
         """Enqueue this rank's ops, stream by stream, in list order."""
-        lib = self._lib
-        world = self.info.local_world_size
         for stream, ops in zip(self.streams, self.info.operations[self.rank]):
             handle = int(stream.cuda_stream)
             for op in ops:
-                if isinstance(op, CopyEngineOp):
-                    assert op.src_rank == self.rank or op.dst_rank == self.rank
-                    if op.src_rank == op.dst_rank and neglect_local:
-                        continue
-                    src = self.comm_buffers[op.src][op.src_rank % world]
-                    dst = self.comm_buffers[op.dst][op.dst_rank % world]
-                    assert src.is_contiguous() and dst.is_contiguous()
-                    nbytes_src = src.numel() * src.element_size()
-                    nbytes_dst = dst.numel() * dst.element_size()
-                    if op.src_offset + op.size > nbytes_src or op.dst_offset + op.size > nbytes_dst:
-                        raise ValueError(f"{op} runs past the end of its buffer")
-                    if self.link_delay_us and op.src_rank != op.dst_rank:
-                        _lib.check("syn_delay_us", lib.syn_delay_us(self.link_delay_us, handle))
-                    dst_ptr, src_ptr = dst.data_ptr() + op.dst_offset, src.data_ptr() + op.src_offset
-                    kernel_ok = self.copy_blocks > 0 and not (op.size % 16 or dst_ptr % 16 or src_ptr % 16)
-                    if kernel_ok:
-                        _lib.check("syn_copy_kernel_async",
-                                   lib.syn_copy_kernel_async(dst_ptr, src_ptr, op.size, self.copy_blocks, handle))
-                    else:
-                        _lib.check("syn_copy_async", lib.syn_copy_async(dst_ptr, src_ptr, op.size, handle))
-                elif isinstance(op, IntraNodeSignal):
-                    assert op.signal_type == SignalType.RECEIVE_DATA
-                    flags = self.recv_signal_bufs[op.rank % world]
-                    if not 0 <= op.offset < flags.numel():
-                        raise ValueError(f"{op} is outside the flag array")
-                    _lib.check("syn_flag_set", lib.syn_flag_set(flags.data_ptr() + 8 * op.offset, 1, handle))
-                elif isinstance(op, WaitIntraNodeSignal):
-                    flags = self._flags(op.signal_type, op.rank % world)
-                    if not 0 <= op.offset < flags.numel():
-                        raise ValueError(f"{op} is outside the flag array")
-                    _lib.check("syn_flag_wait",
-                               lib.syn_flag_wait(flags.data_ptr() + 8 * op.offset, 1, self.wait_timeout_us,
-                                                 self.status.data_ptr(), handle))
-                elif isinstance(op, SMCopyOp):
-                    assert op.src_rank == self.rank or op.dst_rank == self.rank
-                    if op.src_rank == op.dst_rank and neglect_local:
-                        continue
-                    src = self.comm_buffers[op.src][op.src_rank % world]
-                    dst = self.comm_buffers[op.dst][op.dst_rank % world]
-                    src_box = src[tuple(slice(ax.start, ax.end) for ax in op.src_slice)]
-                    dst_box = dst[tuple(slice(ax.start, ax.end) for ax in op.dst_slice)]
-                    with torch.cuda.stream(stream):
-                        if op.reduce_op is None:
-                            dst_box.copy_(src_box.reshape(dst_box.shape))
-                        elif op.reduce_op == ReduceOp.SUM:
-                            dst_box.add_(src_box.reshape(dst_box.shape))
-                        else:
-                            raise NotImplementedError(f"reduce op {op.reduce_op} in a box copy")
-                elif isinstance(op, CollectiveComm):
-                    raise NotImplementedError(
-                        "library collectives need the other ranks to be real processes; "
-                        "the single-GPU executor replays copy/flag op lists only")
+                self._issue(op, self.rank, stream, handle, neglect_local)
+
+    def execute_mesh(self, neglect_local: bool = False) -> None:
+        """Enqueue EVERY rank's ops on this rank's first communication stream, in an order that
+        respects each list and every flag wait (an op that waits for a flag is issued only after
+        the op that writes it).  Plans in which a neighbour forwards what it has received itself
+        (ring, double ring) only deliver this rank's data when the whole mesh is replayed; on one
+        GPU that is one stream doing all the mesh's copies in turn.  Waits for another rank's
+        COMPUTE_DONE flags are taken as satisfied (only this rank's compute kernel runs); this
+        rank's own are real waits on the flags its kernel writes."""
+        if not self.streams:
+            return
+        stream = self.streams[0]
+        handle = int(stream.cuda_stream)
+        world = self.info.local_world_size
+        lists = [(r, ops) for r in range(world) for ops in self.info.operations[r]]
+        cursor = [0] * len(lists)
+        written = set()                  # (signal type, rank, offset) already enqueued as a write
+        for r in range(world):
+            if r != self.rank and self.compute_signal_bufs:
+                self.compute_signal_bufs[r].fill_(1)
+        remaining = sum(len(ops) for _, ops in lists)
+        while remaining:
+            progressed = False
+            for idx, (owner, ops) in enumerate(lists):
+                while cursor[idx] < len(ops):
+                    op = ops[cursor[idx]]
+                    if isinstance(op, WaitIntraNodeSignal) and op.signal_type != SignalType.COMPUTE_DONE:
+                        if (op.signal_type, op.rank % world, op.offset) not in written:
+                            break            # its writer has not been enqueued yet
+                    self._issue(op, owner, stream, handle, neglect_local)
+                    if isinstance(op, IntraNodeSignal):
+                        written.add((op.signal_type, op.rank % world, op.offset))
+                    cursor[idx] += 1
+                    remaining -= 1
+                    progressed = True
+            if not progressed:
+                raise RuntimeError("the op lists wait for flags nobody writes: the plan cannot be replayed")
+
+    def _issue(self, op, owner: int, stream: torch.cuda.Stream, handle: int, neglect_local: bool) -> None:
+        """Enqueue one op of rank `owner`'s list on `stream`."""
+        lib = self._lib
+        world = self.info.local_world_size
+        if isinstance(op, CopyEngineOp):
+            assert op.src_rank == owner or op.dst_rank == owner
+            if op.src_rank == op.dst_rank and neglect_local:
+                return
+            src = self.comm_buffers[op.src][op.src_rank % world]
+            dst = self.comm_buffers[op.dst][op.dst_rank % world]
+            assert src.is_contiguous() and dst.is_contiguous()
+            nbytes_src = src.numel() * src.element_size()
+            nbytes_dst = dst.numel() * dst.element_size()
+            if op.src_offset + op.size > nbytes_src or op.dst_offset + op.size > nbytes_dst:
+                raise ValueError(f"{op} runs past the end of its buffer")
+            if self.link_delay_us and op.src_rank != op.dst_rank:
+                _lib.check("syn_delay_us", lib.syn_delay_us(self.link_delay_us, handle))
+            dst_ptr, src_ptr = dst.data_ptr() + op.dst_offset, src.data_ptr() + op.src_offset
+            kernel_ok = self.copy_blocks > 0 and not (op.size % 16 or dst_ptr % 16 or src_ptr % 16)
+            if kernel_ok:
+                _lib.check("syn_copy_kernel_async",
+                           lib.syn_copy_kernel_async(dst_ptr, src_ptr, op.size, self.copy_blocks, handle))
+            else:
+                _lib.check("syn_copy_async", lib.syn_copy_async(dst_ptr, src_ptr, op.size, handle))
+        elif isinstance(op, IntraNodeSignal):
+            assert op.signal_type == SignalType.RECEIVE_DATA
+            flags = self.recv_signal_bufs[op.rank % world]
+            if not 0 <= op.offset < flags.numel():
+                raise ValueError(f"{op} is outside the flag array")
+            _lib.check("syn_flag_set", lib.syn_flag_set(flags.data_ptr() + 8 * op.offset, 1, handle))
+        elif isinstance(op, WaitIntraNodeSignal):
+            flags = self._flags(op.signal_type, op.rank % world)
+            if not 0 <= op.offset < flags.numel():
+                raise ValueError(f"{op} is outside the flag array")
+            _lib.check("syn_flag_wait",
+                       lib.syn_flag_wait(flags.data_ptr() + 8 * op.offset, 1, self.wait_timeout_us,
+                                         self.status.data_ptr(), handle))
+        elif isinstance(op, SMCopyOp):
+            assert op.src_rank == owner or op.dst_rank == owner
+            if op.src_rank == op.dst_rank and neglect_local:
+                return
+            src = self.comm_buffers[op.src][op.src_rank % world]
+            dst = self.comm_buffers[op.dst][op.dst_rank % world]
+            src_box = src[tuple(slice(ax.start, ax.end) for ax in op.src_slice)]
+            dst_box = dst[tuple(slice(ax.start, ax.end) for ax in op.dst_slice)]
+            with torch.cuda.stream(stream):
+                if op.reduce_op is None:
+                    dst_box.copy_(src_box.reshape(dst_box.shape))
+                elif op.reduce_op == ReduceOp.SUM:
+                    dst_box.add_(src_box.reshape(dst_box.shape))
                 else:
-                    raise TypeError(f"unknown op record {type(op).__name__}")
+                    raise NotImplementedError(f"reduce op {op.reduce_op} in a box copy")
+        elif isinstance(op, CollectiveComm):
+            raise NotImplementedError(
+                "library collectives need the other ranks to be real processes; "
+                "the single-GPU executor replays copy/flag op lists only")
+        else:
+            raise TypeError(f"unknown op record {type(op).__name__}")
 
     def check_status(self) -> None:
         """Synchronise and raise if a stream-side flag wait gave up."""

@@ -260,3 +260,65 @@ def test_copy_kernel_rejects_misaligned(hip):
     assert hip.syn_copy_kernel_async(buf.data_ptr(), buf.data_ptr() + 128, 60, 4, s) == _lib.SYN_EALIGN
     assert hip.syn_copy_kernel_async(buf.data_ptr(), buf.data_ptr() + 128, 64, 0, s) == _lib.SYN_EINVAL
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("kind", ["ring", "double_ring"])
+def test_ring_allgather_gemm_whole_mesh(hip, kind):
+    """Ring forms of the all-gather: a rank only receives what its neighbours forward, so the op
+    lists of the whole mesh are replayed (on one stream, in an order that honours every flag
+    wait) while the consumer GEMM of one rank walks its own schedule."""
+    from oracle import visit_order
+    from syncopate_amd.communication.comm_runtime.communication_context import CommContext
+    from syncopate_amd.communication.common_descriptors import (
+        build_double_ring_all_gather_plan,
+        build_ring_all_gather_plan,
+    )
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.gemm import gemm
+    from syncopate_amd.interface.wave_tables import gemm_consumer_tables
+
+    world, rank, M, K, N, BM, BN = 4, 2, 1024, 256, 512, 128, 128
+    if kind == "ring":
+        plans = {r: build_ring_all_gather_plan((M, K), torch.bfloat16, 0, world, r, "a") for r in range(world)}
+    else:
+        plans = {r: build_double_ring_all_gather_plan((M, K), torch.bfloat16, 0, world, 2, r, "a")
+                 for r in range(world)}
+    schedules, info = _compile(plans)
+    tables = gemm_consumer_tables(schedules[rank]["a"], N)
+    rows = M // world
+    arrival = [off[0] // rows for off in tables.block_offsets]
+    assert sorted(arrival) == list(range(world)) and arrival[0] == rank
+    if kind == "ring":
+        assert arrival == [(rank - k) % world for k in range(world)]
+
+    g = torch.Generator().manual_seed(21)
+    a = (0.05 * torch.randn(M, K, generator=g)).bfloat16()
+    b = (0.05 * torch.randn(N, K, generator=g)).bfloat16()
+    ctx = CommContext(rank, info, link_delay_us=10)
+    for r in range(world):
+        ctx.comm_buffers["a"][r][r * rows:(r + 1) * rows].copy_(a[r * rows:(r + 1) * rows])
+    c = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
+    tiles = (M // BM) * (N // BN)
+    log = torch.full((tiles, 4), -1, dtype=torch.int32, device="cuda")
+    main = torch.cuda.current_stream()
+
+    ctx.reset_signals(whole_mesh=True)
+    ctx.start_after(main)
+    ctx.execute_mesh()
+    gemm(ctx.comm_buffers["a"][rank], b.cuda(), c, world, 24, BM, BN, 64, 8,
+         cur_wave_sizes=tables.block_shapes, wave_offsets=tables.block_offsets,
+         signal_ptr=ctx.recv_signal_bufs[rank], signal_offsets=tables.signal_offsets,
+         cum_tiles=tables.cum_tiles, visit_log=log)
+    ctx.end_before(main)
+    check_status()
+    ctx.check_status()
+
+    for r in range(world):                           # the gather completed on every simulated rank
+        assert torch.equal(ctx.comm_buffers["a"][r].cpu(), a), f"rank {r}"
+    assert _rel(c, numerics.gemm_fp32(a, b)) <= REL_TOL
+    want = visit_order.gemm_tile_visits(tables.block_shapes, tables.block_offsets, tables.signal_offsets,
+                                        M=M, N=N, BM=BM, BN=BN, group_m=8, num_sms=24,
+                                        cum_tiles=tables.cum_tiles)
+    got = log.cpu().tolist()
+    for v in want:
+        assert got[v["tile_id"]] == [v["pid"], v["wave"], v["pid_m"], v["pid_n"]], v
