@@ -150,10 +150,10 @@ int syn_ring_reduce(const void* recv, const void* local, void* out,
  * int32 [Z, H, Sq / block_m] scratch owned by the caller.
  */
 typedef struct syn_attn_desc {
-    const void* q;                  /* [Z, H, Sq, D]                                      */
-    const void* k;                  /* [Z, H, Skv, D]                                     */
-    const void* v;                  /* [Z, H, Skv, D]                                     */
-    void* o;                        /* [Z, H, Sq, D]                                      */
+    const void* q;                  /* (z, h, q row, d), see *_strides                    */
+    const void* k;                  /* (z, h, kv row, d)                                  */
+    const void* v;                  /* (z, h, kv row, d)                                  */
+    void* o;                        /* (z, h, q row, d)                                   */
     float* lse;                     /* [Z, H, Sq]                                         */
     int32_t* lock;                  /* [Z, H, Sq/block_m], zeroed                         */
     int32_t* first;                 /* [Z, H, Sq/block_m], zeroed                         */
@@ -175,6 +175,14 @@ typedef struct syn_attn_desc {
     float sm_scale;
     int64_t cum_tiles;              /* total Z*H*Q elements over all waves                */
     int64_t spin_timeout_us;
+    /* element strides {batch, head, row} of q, k, v and o; d is contiguous.  All zero selects
+       the contiguous [Z, H, S, D] layout of the reference's bhsd kernels
+       (tests/computation/transform/examples/example_attn.py); {S*H*D, D, H*D} is its bshd
+       layout (example_attn_bshd.py).  Strides must be multiples of 8 elements.            */
+    int64_t q_strides[3];
+    int64_t k_strides[3];
+    int64_t v_strides[3];
+    int64_t o_strides[3];
 } syn_attn_desc;
 
 int syn_attn_fwd(const syn_attn_desc* desc, syn_stream_t stream);

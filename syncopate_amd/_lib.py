@@ -101,6 +101,10 @@ class AttnDesc(ctypes.Structure):
         ("sm_scale", c_float),
         ("cum_tiles", c_int64),
         ("spin_timeout_us", c_int64),
+        ("q_strides", c_int64 * 3),
+        ("k_strides", c_int64 * 3),
+        ("v_strides", c_int64 * 3),
+        ("o_strides", c_int64 * 3),
     ]
 
 

@@ -13,7 +13,9 @@ Two call forms, as in the reference:
   Table entries along Q and KV are in ELEMENTS and `cum_wave_sizes`/`cum_tiles`
   count Z*H*Q elements.
 
-Layout: q, o [Z, H, Sq, D]; k, v [Z, H, Skv, D]; D = 128; bf16 or fp16.
+Layout: q, o [Z, H, Sq, D]; k, v [Z, H, Skv, D] ("bhsd", the default), or q, o [Z, Sq, H, D];
+k, v [Z, Skv, H, D] ("bshd", the reference's example_attn_bshd.py); D = 128 contiguous; bf16 or
+fp16.  Views with other batch / head / row strides (slices of a stacked comm buffer) are fine.
 """
 
 from __future__ import annotations
@@ -55,6 +57,7 @@ def attention_forward(
     NUM_WAVES: Optional[int] = None,
     cum_tiles: Optional[int] = None,
     causal: bool = False,
+    layout: str = "bhsd",
     num_programs: int = 0,
     out: Optional[torch.Tensor] = None,
     return_lse: bool = False,
@@ -73,17 +76,24 @@ def attention_forward(
     if not (q.dtype == k.dtype == v.dtype):
         raise TypeError("q, k and v must share one element type")
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
-        raise ValueError("q, k, v must be [Z, H, S, D]")
+        raise ValueError("q, k, v must be 4-D")
+    if layout not in ("bhsd", "bshd"):
+        raise ValueError(f"Unknown layout {layout}")
     HEAD_DIM_Q, HEAD_DIM_K, HEAD_DIM_V = q.shape[-1], k.shape[-1], v.shape[-1]
     assert HEAD_DIM_Q == HEAD_DIM_K and HEAD_DIM_K == HEAD_DIM_V
     if HEAD_DIM_K != 128:
         raise ValueError("the gfx950 kernel is specialised for head_dim 128")
-    Z, H, Sq, D = q.shape
-    if k.shape[:2] != q.shape[:2] or v.shape != k.shape:
-        raise ValueError("k and v must be [Z, H, Skv, D] with q's Z and H")
-    Skv = k.shape[2]
-    if not (q.is_contiguous() and k.is_contiguous() and v.is_contiguous()):
-        raise ValueError("q, k and v must be contiguous (views of a contiguous comm buffer are fine)")
+    h_ax, s_ax = (1, 2) if layout == "bhsd" else (2, 1)
+    Z, H, Sq, D = q.shape[0], q.shape[h_ax], q.shape[s_ax], q.shape[3]
+    if (k.shape[0], k.shape[h_ax]) != (Z, H) or v.shape != k.shape:
+        raise ValueError("k and v must have q's batch and head extents and one shape")
+    Skv = k.shape[s_ax]
+
+    def strides(t: torch.Tensor):
+        if t.stride(3) != 1 or any(t.stride(ax) % 8 for ax in (0, 1, 2)):
+            raise ValueError("the head dimension must be contiguous and rows 16-byte aligned")
+        return (ctypes.c_int64 * 3)(t.stride(0), t.stride(h_ax), t.stride(s_ax))
+
     flags = flag_buffer(signal_ptr)
 
     offs = as_device_table(wave_offsets, dev, 4)
@@ -111,8 +121,8 @@ def attention_forward(
         if caller_owned:
             remember_checked(tables, (num_waves, Z, H, Sq, Skv, cum_tiles, flags.numel()))
 
-    o = torch.empty_like(q) if out is None else out
-    if o.shape != q.shape or o.dtype != q.dtype or not o.is_contiguous():
+    o = torch.empty(q.shape, dtype=q.dtype, device=dev) if out is None else out
+    if o.shape != q.shape or o.dtype != q.dtype:
         raise ValueError("out must match q")
     # lse (base 2), lock and first-writer marker: the reference's M / guard / first
     # (template.py:382-384), one lock per 128-row q block
@@ -133,6 +143,7 @@ def attention_forward(
         num_waves=num_waves, Z=Z, H=H, Sq=Sq, Skv=Skv, D=D, dtype=_lib.dtype_code(q.dtype),
         block_m=BLOCK_M, block_n=BLOCK_N, causal=1 if causal else 0, num_programs=int(num_programs),
         sm_scale=float(sm_scale), cum_tiles=int(cum_tiles), spin_timeout_us=int(spin_timeout_us),
+        q_strides=strides(q), k_strides=strides(k), v_strides=strides(v), o_strides=strides(o),
     )
     with torch.cuda.device(dev):
         _lib.check("syn_attn_fwd", lib.syn_attn_fwd(ctypes.byref(desc), _lib.stream_handle(stream)))

@@ -52,6 +52,8 @@ struct AttnParams {
     int32_t causal;
     int32_t num_tiles;
     float qk_scale;       // sm_scale * 1.44269504 (template.py:178-179)
+    // element strides {batch, head, row}
+    int64_t q_st[3], k_st[3], v_st[3], o_st[3];
 };
 
 constexpr int kAttnThreads = 256;
@@ -92,15 +94,16 @@ typedef __attribute__((address_space(3))) s16x4_t* lds_s16x4_ptr;
 // s_waitcnt immediate (gfx9 encoding): at most `vm` vector-memory operations outstanding
 constexpr int attn_vmcnt(int vm) { return (vm & 0xF) | ((vm >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
 
-// One kv block (128 rows of 256 bytes, contiguous in HBM) into LDS.  Wavefront `wave` issues
-// 1 KB fills number wave, wave + 4, ...; lane l lands at byte 16*l of the fill, i.e. row l/16,
-// physical 16-byte chunk l%16, and `lane_off` makes it fetch the logical chunk that lives there.
-__device__ __forceinline__ void dma_kv_block(unsigned char* lds, const unsigned char* src,
+// One kv block (128 rows of 256 bytes, `pitch` bytes apart in HBM) into LDS.  Wavefront `wave`
+// issues 1 KB fills number wave, wave + 4, ... (4 rows each); lane l lands at byte 16*l of the
+// fill, i.e. row l/16, physical 16-byte chunk l%16, and `lane_off` (row l/16 at the pitch, plus
+// the logical chunk that lives there) makes it fetch the right 16 bytes.
+__device__ __forceinline__ void dma_kv_block(unsigned char* lds, const unsigned char* src, size_t pitch,
                                              unsigned lane_off, int wave) {
 #pragma unroll
     for (int i = 0; i < kFills; ++i) {
         const int blk = i * 4 + wave;
-        __builtin_amdgcn_global_load_lds((global_void_ptr)(src + blk * 1024 + lane_off),
+        __builtin_amdgcn_global_load_lds((global_void_ptr)(src + (size_t)(blk * 4) * pitch + lane_off),
                                          (lds_void_ptr)(lds + blk * 1024), 16, 0, 0);
     }
 }
@@ -137,8 +140,9 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
     // fills: lane l covers row l/16 of its 4-row group; rows of fill `blk` are 4*blk + l/16 and
     // blk % 4 == wave, so (row & 15) == 4*wave + l/16 and (row & 3) == l/16
     const int f_row = lane >> 4, f_c = lane & 15;
-    const unsigned k_fill_off = (unsigned)(f_row * kRowBytes + ((f_c ^ (4 * wave + f_row)) << 4));
-    const unsigned v_fill_off = (unsigned)(f_row * kRowBytes + ((f_c ^ (f_row << 2)) << 4));
+    const size_t k_pitch = (size_t)p.k_st[2] * sizeof(T), v_pitch = (size_t)p.v_st[2] * sizeof(T);
+    const unsigned k_fill_off = (unsigned)(f_row * k_pitch + ((f_c ^ (4 * wave + f_row)) << 4));
+    const unsigned v_fill_off = (unsigned)(f_row * v_pitch + ((f_c ^ (f_row << 2)) << 4));
     // K fragment reads: row 32*j + r, logical chunk 2*ks + half
     const int k_rd = r * kRowBytes;
     // V^T fragment reads: 16-lane group g = lane/16: d0 = 16*(g & 1), kv offset 4*half (+8 for
@@ -204,13 +208,13 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
 
         const size_t head = (size_t)z * p.H + h;
         const int q_row = qb * kBlockM + wave * 32 + r;              // this lane's q position
-        const T* q_src = Q + (head * p.Sq + q_row) * kHeadDim + 8 * half;
-        const unsigned char* k_base = K + head * (size_t)p.Skv * kRowBytes;
-        const unsigned char* v_base = V + head * (size_t)p.Skv * kRowBytes;
+        const T* q_src = Q + z * p.q_st[0] + h * p.q_st[1] + q_row * p.q_st[2] + 8 * half;
+        const unsigned char* k_base = K + (z * p.k_st[0] + h * p.k_st[1]) * (int64_t)sizeof(T);
+        const unsigned char* v_base = V + (z * p.v_st[0] + h * p.v_st[1]) * (int64_t)sizeof(T);
 
         // both stages are free here: every wavefront has passed the barrier that ends a tile
-        dma_kv_block(k_lds, k_base + (size_t)kv_lo * kBlockBytes, k_fill_off, wave);
-        dma_kv_block(v_lds, v_base + (size_t)kv_lo * kBlockBytes, v_fill_off, wave);
+        dma_kv_block(k_lds, k_base + (size_t)kv_lo * kBlockN * k_pitch, k_pitch, k_fill_off, wave);
+        dma_kv_block(v_lds, v_base + (size_t)kv_lo * kBlockN * v_pitch, v_pitch, v_fill_off, wave);
 
         frag_t qf[8];
 #pragma unroll
@@ -274,7 +278,7 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
             __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_waitcnt(0xc07f);          // lgkmcnt(0): own LDS reads have returned
             __builtin_amdgcn_s_barrier();
-            dma_kv_block(k_lds, k_base + (size_t)min(n + 1, kv_end - 1) * kBlockBytes, k_fill_off, wave);
+            dma_kv_block(k_lds, k_base + (size_t)min(n + 1, kv_end - 1) * kBlockN * k_pitch, k_pitch, k_fill_off, wave);
             __builtin_amdgcn_sched_barrier(0);
 
             // ---- online softmax in base 2 ----
@@ -364,7 +368,7 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
             __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_waitcnt(0xc07f);
             __builtin_amdgcn_s_barrier();
-            dma_kv_block(v_lds, v_base + (size_t)min(n + 1, kv_end - 1) * kBlockBytes, v_fill_off, wave);
+            dma_kv_block(v_lds, v_base + (size_t)min(n + 1, kv_end - 1) * kBlockN * v_pitch, v_pitch, v_fill_off, wave);
             __builtin_amdgcn_sched_barrier(0);
         };
         // under a causal mask the diagonal block, if this tile reaches it, is the last one
@@ -412,7 +416,7 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
             w_old = fast_exp2(m_old - lse_out);
             w_new = fast_exp2(lse2 - lse_out);
         }
-        T* o_row = O + (head * p.Sq + q_row) * kHeadDim + 4 * half;
+        T* o_row = O + z * p.o_st[0] + h * p.o_st[1] + q_row * p.o_st[2] + 4 * half;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -526,6 +530,23 @@ int syn_attn_fwd(const syn_attn_desc* d, syn_stream_t stream) {
     p.causal = d->causal ? 1 : 0;
     p.num_tiles = (int)tiles;
     p.qk_scale = d->sm_scale * 1.44269504f;
+    {
+        // all-zero strides: contiguous [Z, H, S, D]
+        const int64_t dq[3] = {(int64_t)d->H * d->Sq * kHeadDim, (int64_t)d->Sq * kHeadDim, kHeadDim};
+        const int64_t dk[3] = {(int64_t)d->H * d->Skv * kHeadDim, (int64_t)d->Skv * kHeadDim, kHeadDim};
+        struct { const int64_t* in; const int64_t* dflt; int64_t* out; } sets[4] = {
+            {d->q_strides, dq, p.q_st}, {d->k_strides, dk, p.k_st}, {d->v_strides, dk, p.v_st}, {d->o_strides, dq, p.o_st}};
+        for (auto& s : sets) {
+            const bool unset = s.in[0] == 0 && s.in[1] == 0 && s.in[2] == 0;
+            for (int i = 0; i < 3; ++i) {
+                s.out[i] = unset ? s.dflt[i] : s.in[i];
+                if (s.out[i] < 0 || s.out[i] % 8) return SYN_EALIGN;     // 16-byte rows
+            }
+            if (s.out[2] < kHeadDim) return SYN_EINVAL;
+            // the lane offset of a fill is 32 bits: 4 rows at the pitch must fit
+            if (s.out[2] * 2 * 4 > (int64_t)UINT32_MAX) return SYN_EINVAL;
+        }
+    }
 
     int grid = d->num_programs > 0 ? d->num_programs : (int)tiles;
     if (grid > tiles) grid = (int)tiles;

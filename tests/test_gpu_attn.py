@@ -102,3 +102,38 @@ def test_hand_template_form_resident(hip):
     ref = p @ v.float()
     torch.testing.assert_close(o.float().cpu(), ref, atol=5e-2, rtol=0)   # the reference's bound (:486)
     assert _rel(o, ref) <= REL_TOL
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_bshd_layout_and_strided_views(hip, causal):
+    """The reference's second layout, q/k/v as [Z, S, H, D] (example_attn_bshd.py), and views of
+    a stacked comm buffer whose batch/head/row strides are not those of a contiguous tensor."""
+    from syncopate_amd.computation.attn import attention_forward
+    from syncopate_amd.computation._launch import check_status
+
+    Z, H, S = 2, 3, 512
+    q, k, v = _qkv(Z, H, S, S, torch.bfloat16, seed=4)
+    sm_scale = 128 ** -0.5
+    ref = numerics.sdpa_fp32(q, k, v, sm_scale, causal=causal)
+    chunks = [(0, 256), (256, 512)]
+    offsets, sizes, cums, signals, total = _kv_waves(Z, H, S, chunks, [-1, 0])
+    flags = torch.ones(1, dtype=torch.int64, device="cuda")
+    tables = dict(wave_offsets=offsets, wave_sizes=sizes, cum_wave_sizes=cums, signal_ptr=flags,
+                  signal_offsets=signals, cum_tiles=total, causal=causal)
+
+    # [Z, S, H, D] tensors
+    qs, ks, vs = (t.permute(0, 2, 1, 3).contiguous().cuda() for t in (q, k, v))
+    o = attention_forward(qs, ks, vs, sm_scale, layout="bshd", **tables)
+    check_status()
+    assert o.shape == qs.shape
+    assert _rel(o.permute(0, 2, 1, 3), ref) <= REL_TOL
+
+    # k and v as slices of one stacked [2, Z, H, S + 128, D] buffer, q a slice of a wider tensor
+    kv = torch.zeros(2, Z, H, S + 128, 128, dtype=torch.bfloat16, device="cuda")
+    kv[0, :, :, 64:64 + S].copy_(k)
+    kv[1, :, :, 64:64 + S].copy_(v)
+    wide = torch.zeros(Z, H + 1, S, 128, dtype=torch.bfloat16, device="cuda")
+    wide[:, 1:].copy_(q)
+    o2 = attention_forward(wide[:, 1:], kv[0, :, :, 64:64 + S], kv[1, :, :, 64:64 + S], sm_scale, **tables)
+    check_status()
+    assert _rel(o2, ref) <= REL_TOL

@@ -103,8 +103,8 @@ def test_gemm_rs_iteration(hip, rank):
     assert _rel(out, total) <= 2e-2
 
 
-@pytest.mark.parametrize("rank", [1, 3])
-def test_allgather_attention_iteration(hip, rank):
+@pytest.mark.parametrize("rank,layout", [(1, "bhsd"), (3, "bhsd"), (2, "bshd")])
+def test_allgather_attention_iteration(hip, rank, layout):
     """K/V chunks pulled from their owners on a side stream (copy, then flag) while the
     attention kernel walks the waves of the lowered schedule; the local Q attends to the whole
     sequence."""
@@ -116,7 +116,7 @@ def test_allgather_attention_iteration(hip, rank):
 
     world, B, H, SEQ, D = 4, 1, 2, 1024, 128
     per_rank = SEQ // world
-    shape, seq_axis, axes = plan_layout_spec("bhsd", B, H, SEQ, D)
+    shape, seq_axis, axes = plan_layout_spec(layout, B, H, SEQ, D)
     plans = {r: build_all_gather_plan_1d_swizzle(shape, torch.bfloat16, seq_axis, world, r, "kv", "pull")
              for r in range(world)}
     schedules, info = _compile(plans)
@@ -126,13 +126,14 @@ def test_allgather_attention_iteration(hip, rank):
 
     g = torch.Generator().manual_seed(5)
     kv = torch.randn(*shape, generator=g).bfloat16()
-    q = torch.randn(B, H, per_rank, D, generator=g).bfloat16()
+    q = torch.randn(B, H, per_rank, D, generator=g).bfloat16()       # [B, H, S, D] whatever the layout
     ctx = CommContext(rank, info, link_delay_us=30)
     for r in range(world):                           # every simulated rank holds its own slice
-        ctx.comm_buffers["kv"][r][:, :, :, r * per_rank:(r + 1) * per_rank].copy_(
-            kv[:, :, :, r * per_rank:(r + 1) * per_rank])
+        own = [slice(None)] * 5
+        own[seq_axis] = slice(r * per_rank, (r + 1) * per_rank)
+        ctx.comm_buffers["kv"][r][tuple(own)].copy_(kv[tuple(own)])
     buf = ctx.comm_buffers["kv"][rank]
-    qd = q.cuda()
+    qd = q.cuda() if layout == "bhsd" else q.permute(0, 2, 1, 3).contiguous().cuda()
     tiles = tables.cum_tiles // 128
     log = torch.full((tiles, 8), -1, dtype=torch.int32, device="cuda")
     main = torch.cuda.current_stream()
@@ -143,14 +144,16 @@ def test_allgather_attention_iteration(hip, rank):
     out = attention_forward(qd, buf[0], buf[1], D ** -0.5, wave_offsets=tables.wave_offsets,
                             wave_sizes=tables.wave_sizes, cum_wave_sizes=tables.cum_wave_sizes,
                             signal_ptr=ctx.recv_signal_bufs[rank], signal_offsets=tables.signal_offsets,
-                            NUM_WAVES=len(tables.signal_offsets), cum_tiles=tables.cum_tiles, visit_log=log)
+                            NUM_WAVES=len(tables.signal_offsets), cum_tiles=tables.cum_tiles, visit_log=log,
+                            layout=layout)
     ctx.end_before(main)
     check_status()
     ctx.check_status()
 
     assert torch.equal(buf.cpu(), kv)                # the gather itself
-    want = numerics.sdpa_fp32(q, kv[0], kv[1], D ** -0.5)
-    assert _rel(out, want) <= REL_TOL
+    to_bhsd = (lambda t: t) if layout == "bhsd" else (lambda t: t.permute(0, 2, 1, 3))
+    want = numerics.sdpa_fp32(q, to_bhsd(kv[0]), to_bhsd(kv[1]), D ** -0.5)
+    assert _rel(to_bhsd(out), want) <= REL_TOL
     assert (log[:, 0] >= 0).all()                    # every tile of every wave ran
 
 
