@@ -19,8 +19,9 @@
 // layout of S^T is already the B-operand layout of the second product.
 //
 // K and V blocks go from HBM straight into LDS (global_load_lds_dwordx4, no register
-// staging): the fill of the next K block is issued as soon as S^T is done and overlaps the
-// softmax and the second product, the fill of the next V block overlaps the next S^T.
+// staging): the fills of V block n are issued between the MFMAs of S^T of block n, those of
+// K block n+1 between the exponentials of block n, one at a time so that the in-order
+// wavefront is never held at the vector-memory queue.
 // The kernel stays under 256 registers and 80 KB of LDS, so two workgroups share a compute
 // unit and one's exponentials overlap the other's matrix work.
 #include <type_traits>
@@ -214,7 +215,6 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
 
         // both stages are free here: every wavefront has passed the barrier that ends a tile
         dma_kv_block(k_lds, k_base + (size_t)kv_lo * kBlockN * k_pitch, k_pitch, k_fill_off, wave);
-        dma_kv_block(v_lds, v_base + (size_t)kv_lo * kBlockN * v_pitch, v_pitch, v_fill_off, wave);
 
         frag_t qf[8];
 #pragma unroll
@@ -234,16 +234,19 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
         // one kv block; MASK: the causal diagonal block (kv positions beyond a q row are masked)
         auto kv_block = [&](const int n, auto mask_tag) {
             constexpr bool MASK = decltype(mask_tag)::value;
-            // ---- K block n has landed (its fills are older than V's) ----
+            // ---- K block n has landed (nothing newer is in flight: V block n is fetched below) ----
             __builtin_amdgcn_sched_barrier(0);
-            __builtin_amdgcn_s_waitcnt(attn_vmcnt(kFills));
+            __builtin_amdgcn_s_waitcnt(attn_vmcnt(0));
             __builtin_amdgcn_s_barrier();
             __builtin_amdgcn_sched_barrier(0);
 
             // ---- S^T = K . Q^T : 4 tiles of [32 kv, 32 q]; fragments of step ks+1 are read
             //      while step ks is multiplied ----
+            // The fills of V block n are issued one per k16 step between the MFMAs: a wavefront issues in
+            // order, and eight 1 KB fills in a row would hold it at the vector-memory queue.
             f32x16_t s[4];
             {
+                dma_kv_block(v_lds, v_base + (size_t)n * kBlockN * v_pitch, v_pitch, v_fill_off, wave);
                 const f32x16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
                 frag_t kf[2][4];
                 const unsigned char* k_row = k_lds + k_rd;
@@ -271,14 +274,14 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
                     } else {
                         __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
                     }
+                    __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
                 }
             }
 
-            // ---- every wavefront is done with K: fetch the next K block behind the softmax ----
+            // ---- every wavefront is done with K: the next K block is fetched inside the softmax ----
             __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_waitcnt(0xc07f);          // lgkmcnt(0): own LDS reads have returned
             __builtin_amdgcn_s_barrier();
-            dma_kv_block(k_lds, k_base + (size_t)min(n + 1, kv_end - 1) * kBlockN * k_pitch, k_pitch, k_fill_off, wave);
             __builtin_amdgcn_sched_barrier(0);
 
             // ---- online softmax in base 2 ----
@@ -298,6 +301,16 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
             mx = fmaxf(mx, __shfl_xor(mx, 32));
             const float m_new = fmaxf(m_i, mx * p.qk_scale);
             const float alpha = fast_exp2(m_i - m_new);
+            // rescale O only when some row's maximum moved (wavefront-uniform test)
+            if (__builtin_amdgcn_ballot_w64(m_new != m_i) != 0) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) o_acc[i][e] *= alpha;
+            }
+            // the exponentials, with the eight fills of K block n+1 spread between them
+            __builtin_amdgcn_sched_barrier(0);
+            dma_kv_block(k_lds, k_base + (size_t)min(n + 1, kv_end - 1) * kBlockN * k_pitch, k_pitch, k_fill_off, wave);
             float row_sum = 0.f;
             frag_t pf[8];
 #pragma unroll
@@ -310,14 +323,12 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
                     // the kv indices 16t + 8*(i/4) + 4*half + i%4 that step t contracts over
                     pf[2 * j + (e >> 3)][e & 7] = (T)pe;
                 }
-            l_i = l_i * alpha + row_sum;
-            // rescale O only when some row's maximum moved (wavefront-uniform test)
-            if (__builtin_amdgcn_ballot_w64(m_new != m_i) != 0) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) o_acc[i][e] *= alpha;
+            for (int f = 0; f < kFills; ++f) {
+                __builtin_amdgcn_sched_group_barrier(0x400, 8, 0);      // 8 of the 64 exponentials
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
             }
+            l_i = l_i * alpha + row_sum;
             m_i = m_new;
 
             // ---- V block n has landed (only the next K block's fills are newer) ----
@@ -364,11 +375,10 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
                 }
             }
 
-            // ---- every wavefront is done with V: fetch the next V block behind the next S^T ----
+            // ---- every wavefront is done with V: the next V block is fetched inside the next S^T ----
             __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_waitcnt(0xc07f);
             __builtin_amdgcn_s_barrier();
-            dma_kv_block(v_lds, v_base + (size_t)min(n + 1, kv_end - 1) * kBlockN * v_pitch, v_pitch, v_fill_off, wave);
             __builtin_amdgcn_sched_barrier(0);
         };
         // under a causal mask the diagonal block, if this tile reaches it, is the last one
