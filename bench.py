@@ -212,6 +212,77 @@ def run_reduce(device, steps, warmup):
     return ms, nbytes
 
 
+def run_attention(device, steps, warmup):
+    """All-gather attention at BASELINE configuration 5: 4096 local q rows, 32 heads, against 32768
+    kv rows as 8 chunks of 4096 in double-ring arrival order (every chunk resident), head dim 128."""
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.attn import attention_forward
+
+    B, H, Sq, Skv, D, chunks = 1, 32, 4096, 32768, 128, 8
+    torch.manual_seed(2)
+    q = torch.randn(B, H, Sq, D, device=device).bfloat16()
+    k = torch.randn(B, H, Skv, D, device=device).bfloat16()
+    v = torch.randn(B, H, Skv, D, device=device).bfloat16()
+    chunk = Skv // chunks
+    as_table = lambda rows: torch.tensor(rows, dtype=torch.int32, device=device)
+    cums = [(i + 1) * B * H * Sq for i in range(chunks)]
+    tables = dict(wave_offsets=as_table([[0, 0, 0, o * chunk] for o in (0, 1, 7, 6, 4, 5, 3, 2)]),
+                  wave_sizes=as_table([[B, H, Sq, chunk]] * chunks), cum_wave_sizes=as_table(cums),
+                  signal_offsets=as_table([-1, 0, 4, 1, 5, 2, 6, 3]), cum_tiles=cums[-1],
+                  signal_ptr=torch.ones(chunks, dtype=torch.int64, device=device))
+    out = torch.empty_like(q)
+    for _ in range(warmup):
+        attention_forward(q, k, v, D ** -0.5, out=out, **tables)
+    torch.cuda.synchronize()
+    begin, end = _events(1)[0], _events(1)[0]
+    begin.record()
+    for _ in range(steps):
+        attention_forward(q, k, v, D ** -0.5, out=out, **tables)
+    end.record()
+    torch.cuda.synchronize()
+    check_status()
+    s = (q[0, 7].float() @ k[0, 7].float().t()) * D ** -0.5
+    ref = torch.softmax(s, dim=-1) @ v[0, 7].float()
+    err = ((out[0, 7].float() - ref).abs().max() / ref.abs().max()).item()
+    return begin.elapsed_time(end) / steps, 4.0 * B * H * Sq * Skv * D, err
+
+
+def run_producer(device, steps, warmup):
+    """GEMM+RS producer at BASELINE configuration 3: partial C (8192, 8192) = A (8192, 3584) B^T in
+    wave order 1..7, 0 with per-wave counters and flags."""
+    from syncopate_amd.computation.gemm import gemm_producer
+
+    m, k, n, world = 8192, 3584, 8192, 8
+    torch.manual_seed(3)
+    a = (0.02 * torch.randn(m, k, device=device)).bfloat16()
+    b = (0.02 * torch.randn(n, k, device=device)).bfloat16()
+    c = torch.empty(m, n, dtype=torch.bfloat16, device=device)
+    rows = m // world
+    as_table = lambda rows_: torch.tensor(rows_, dtype=torch.int32, device=device)
+    sizes = as_table([[rows, n]] * world)
+    offsets = as_table([[((RANK + i + 1) % world) * rows, 0] for i in range(world)])
+    signals = as_table(list(range(world)))
+    flags = torch.zeros(world, dtype=torch.int64, device=device)
+    counters = torch.zeros(world, dtype=torch.int32, device=device)
+
+    def launch():
+        counters.zero_()
+        gemm_producer(a, b, c, flags, sizes, offsets, signals, NUM_SMS, BM, BN, BK, GROUP_M, cum_tiles=m * n,
+                      counter_buffer=counters, xcd_remap=False, eight_waves=EIGHT_WAVES)
+
+    for _ in range(warmup):
+        launch()
+    torch.cuda.synchronize()
+    begin, end = _events(1)[0], _events(1)[0]
+    begin.record()
+    for _ in range(steps):
+        launch()
+    end.record()
+    torch.cuda.synchronize()
+    assert flags.tolist() == [1] * world
+    return begin.elapsed_time(end) / steps, 2.0 * m * n * k
+
+
 def cpu_baseline(state):
     """torch CPU matmul over the gathered operands (fp32 values of the same bf16 inputs):
     a bounded sample of the same GEMM — a band of rows of A against all of B."""
@@ -269,6 +340,8 @@ def main():
     traffic_calibration(device)
     err, gathered = check_ag_gemm(state)
     reduce_ms, reduce_bytes = run_reduce(device, max(args.steps, 30), args.warmup)
+    attn_ms, attn_flop, attn_err = run_attention(device, 5, 2)
+    prod_ms, prod_flop = run_producer(device, args.steps, args.warmup)
 
     flop = 2.0 * M * N * K
     value = flop / (wall_ms * 1e-3) / 1e12
@@ -304,6 +377,12 @@ def main():
         "rs_reduce_GBps": reduce_bytes / (reduce_ms * 1e-3) / 1e9,
         "rs_reduce_us": reduce_ms * 1e3,
         "rs_reduce_pct_hbm_peak": 100.0 * reduce_bytes / (reduce_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+        "rs_producer_tflops": prod_flop / (prod_ms * 1e-3) / 1e12,
+        "rs_producer_pct_bf16_mfma_peak": 100.0 * prod_flop / (prod_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+        "attn_tflops": attn_flop / (attn_ms * 1e-3) / 1e12,
+        "attn_pct_bf16_mfma_peak": 100.0 * attn_flop / (attn_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+        "attn_ms": attn_ms,
+        "attn_max_rel_err_vs_fp32": attn_err,
         "host_compile_ms": state["compile_ms"],
         "max_rel_err_vs_fp32": err,
         "gathered_a_matches": gathered,

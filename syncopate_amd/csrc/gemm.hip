@@ -631,13 +631,23 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
                     for (int g = 0; g < 4; ++g) {
                         const uint2 v = pack4<T>(acc[i][j][4 * g], acc[i][j][4 * g + 1],
                                                  acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
-                        *reinterpret_cast<uint2*>(c_row + (size_t)(32 * i) * N + 32 * j + 8 * g) = v;
+                        T* dst = c_row + (size_t)(32 * i) * N + 32 * j + 8 * g;
+                        if (PRODUCER) {
+                            // written through the XCD's L2: the release below then has nothing
+                            // of this tile left to write back
+                            __hip_atomic_store(reinterpret_cast<uint64_t*>(dst), __builtin_bit_cast(uint64_t, v),
+                                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        } else {
+                            *reinterpret_cast<uint2*>(dst) = v;
+                        }
                     }
         }
 
         if (PRODUCER) {
             if (tile.sig >= 0) {
-                __threadfence();             // every lane's C stores are visible device-wide
+                // every lane's C stores are visible device-wide before the count moves (release only:
+                // an acquire here would also throw away the L2 contents the next tile reuses)
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
                 __syncthreads();
                 if (tid == 0) {
                     const int done = __hip_atomic_fetch_add(p.counters + tile.wave, 1, __ATOMIC_RELEASE,
