@@ -267,7 +267,8 @@ def run_producer(device, steps, warmup):
 
     def launch():
         counters.zero_()
-        gemm_producer(a, b, c, flags, sizes, offsets, signals, NUM_SMS, BM, BN, BK, GROUP_M, cum_tiles=m * n,
+        # 1024 tiles of 256 x 256: four full rounds of 256 programs
+        gemm_producer(a, b, c, flags, sizes, offsets, signals, 256, BM, BN, BK, GROUP_M, cum_tiles=m * n,
                       counter_buffer=counters, xcd_remap=False, eight_waves=EIGHT_WAVES)
 
     for _ in range(warmup):

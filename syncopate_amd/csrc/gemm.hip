@@ -645,9 +645,10 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
 
         if (PRODUCER) {
             if (tile.sig >= 0) {
-                // every lane's C stores are visible device-wide before the count moves (release only:
-                // an acquire here would also throw away the L2 contents the next tile reuses)
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+                // Every lane's C stores were agent-scope write-through stores; the barrier's wait for
+                // their acknowledgements makes them visible device-wide before thread 0 moves the
+                // count (a release).  No L2 write-back or invalidate: the next tile reuses that L2.
+                __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, true));
                 __syncthreads();
                 if (tid == 0) {
                     const int done = __hip_atomic_fetch_add(p.counters + tile.wave, 1, __ATOMIC_RELEASE,

@@ -32,8 +32,9 @@ def _compile(plans):
     return schedules, info
 
 
-@pytest.mark.parametrize("rank", [0, 2])
-def test_gemm_rs_iteration(hip, rank):
+@pytest.mark.parametrize("rank,shape", [(0, (4, 1024, 512, 256, 128, 128, 13)), (2, (4, 1024, 512, 256, 128, 128, 13)),
+                                        (5, (8, 8192, 4096, 512, 256, 256, 224))])
+def test_gemm_rs_iteration(hip, rank, shape):
     """Producer GEMM -> comm stream waits on each wave's COMPUTE_DONE flag and pushes the chunk
     to its owner -> ring reduce of the received partials."""
     from syncopate_amd.communication.comm_runtime.communication_context import CommContext
@@ -43,7 +44,7 @@ def test_gemm_rs_iteration(hip, rank):
     from syncopate_amd.computation.reduce import ring_reduce_tma
     from syncopate_amd.interface.wave_tables import gemm_producer_tables
 
-    world, M, N, K, BM, BN = 4, 1024, 512, 256, 128, 128
+    world, M, N, K, BM, BN, programs = shape
     rows = M // world
     g = torch.Generator().manual_seed(11 + rank)
     a = (0.1 * torch.randn(M, K, generator=g)).bfloat16()
@@ -71,7 +72,7 @@ def test_gemm_rs_iteration(hip, rank):
     ctx.reset_signals()
     comm_stream.wait_stream(main)
     gemm_producer(ad, bd, src, ctx.compute_signal_bufs[rank], tables.block_shapes, tables.block_offsets,
-                  tables.signal_offsets, 13, BM, BN, 64, 8, cum_tiles=tables.cum_tiles)
+                  tables.signal_offsets, programs, BM, BN, 64, 8, cum_tiles=tables.cum_tiles)
     ctx.start_after(comm_stream)
     ctx.execute(neglect_local=True)
     ctx.end_before(comm_stream)
