@@ -103,6 +103,37 @@ int syn_gemm_consumer(const syn_gemm_desc* desc, syn_stream_t stream);
 int syn_gemm_producer(const syn_gemm_desc* desc, syn_stream_t stream);
 
 /*
+ * Remote bindings of a GEMM launch: per wave, A is read from a peer's shard and / or the C
+ * tile goes into a peer's buffer instead of the local one.  Counterpart of the reference's
+ * dl.symm_at(ptr, target_rank) rebinding: kernel_gemm_ag_read_remote
+ * (syncopate/computation/gemm/template_ag.py:43-187: A rows of wave w come from
+ * a_peers[a_target_rank[w]] at the wave-local row, C is written at the global row),
+ * kernel_gemm_rs_producer_persistent (template_rs.py:37-209: the C tile is atomically added
+ * into c_peers[c_target_rank[w]] at the wave-local row) and the generated form with
+ * target_rank / dst_offsets arguments (transform/transformer.py:1158-1178,
+ * tests/test_gemm_rs_direct_reduce.py:166-189).  On one GPU the peers are buffers of the same
+ * process; on a node they are peer-mapped allocations.
+ */
+typedef struct syn_gemm_remote {
+    const void* const* a_peers;     /* device array of pointers to [rows, K] shards, or NULL   */
+    const int32_t* a_target_rank;   /* device int32[num_waves]: index into a_peers             */
+    void* const* c_peers;           /* device array of pointers to peer C buffers, or NULL     */
+    const int32_t* c_target_rank;   /* device int32[num_waves]: index into c_peers             */
+    const int32_t* c_dst_offsets;   /* device int32[num_waves, 2]: {row, col} of the wave's
+                                       region inside the peer C, in elements                   */
+    int32_t c_ld;                   /* row length of a peer C buffer (multiple of 4)           */
+    int32_t c_atomic_add;           /* 1: add into the peer C (packed 16-bit float atomics),
+                                       0: store                                                */
+} syn_gemm_remote;
+
+/*
+ * The consumer walk (flags honoured where a wave has one) with the bindings above.  desc->a
+ * may be NULL when a_peers is given, desc->c when c_peers is.  Default pipeline only.
+ */
+int syn_gemm_remote_binding(const syn_gemm_desc* desc, const syn_gemm_remote* remote,
+                            syn_stream_t stream);
+
+/*
  * Host-only check of a GEMM wave table against the operand shapes, block
  * sizes and flag-array length; the launch entry points cannot do it because
  * the tables they get live in device memory.  All pointers are HOST pointers.

@@ -71,6 +71,18 @@ class GemmDesc(ctypes.Structure):
     ]
 
 
+class GemmRemote(ctypes.Structure):
+    _fields_ = [
+        ("a_peers", c_void_p),
+        ("a_target_rank", c_void_p),
+        ("c_peers", c_void_p),
+        ("c_target_rank", c_void_p),
+        ("c_dst_offsets", c_void_p),
+        ("c_ld", c_int32),
+        ("c_atomic_add", c_int32),
+    ]
+
+
 class AttnDesc(ctypes.Structure):
     _fields_ = [
         ("q", c_void_p),
@@ -112,6 +124,7 @@ class AttnDesc(ctypes.Structure):
 _SIGNATURES = {
     "syn_gemm_consumer": (c_int32, [POINTER(GemmDesc), c_void_p]),
     "syn_gemm_producer": (c_int32, [POINTER(GemmDesc), c_void_p]),
+    "syn_gemm_remote_binding": (c_int32, [POINTER(GemmDesc), POINTER(GemmRemote), c_void_p]),
     "syn_gemm_check_waves": (
         c_int32,
         [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,

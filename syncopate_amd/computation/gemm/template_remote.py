@@ -1,0 +1,255 @@
+"""Launchers of the GEMM forms that bind an operand to a peer per wave (MI355X HIP, C ABI).
+
+* ``gemm_ag_direct_read`` — the GEMM reads the A rows of every wave straight from the shard of
+  the rank that owns them instead of from a gathered buffer
+  (syncopate/computation/gemm/template_ag.py:43-187, launcher :190-260).
+* ``gemm_rs_producer_persistent`` — the C tile of every wave is atomically added into the
+  [M / W, N] result of the rank that owns those rows
+  (syncopate/computation/gemm/template_rs.py:37-209, launcher :212-290).
+* ``gemm_remote`` — the call form the transform pass generates for a descriptor with a
+  RemoteBinding: ``target_rank`` and ``dst_offsets`` per wave, store or atomic add
+  (syncopate/computation/transform/transformer.py:1158-1178; use in
+  tests/test_gemm_rs_direct_reduce.py:166-189).
+
+The reference resolves a peer's buffer with ``dl.symm_at(ptr, rank)`` on an NVSHMEM heap.  Here
+the caller passes the peers' buffers themselves (``a`` / ``c`` as a list with one tensor per
+rank): on one MI355X they are tensors of the same process, on a node they would be peer-mapped
+allocations.  Everything else (tables in elements, B stored [N, K]) is as in ``template.py``.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Optional, Sequence
+
+import torch
+
+from ... import _lib
+from .._launch import TableLike, as_device_table, host_copy, host_ptr, require_cuda, status_words
+
+_pointer_tables: dict = {}
+
+
+def _pointer_table(tensors: Sequence[torch.Tensor], dev: torch.device) -> torch.Tensor:
+    """Device array of the tensors' addresses (kept per set of addresses: a launch must not
+    allocate in steady state)."""
+    key = (dev.index, tuple(t.data_ptr() for t in tensors))
+    table = _pointer_tables.get(key)
+    if table is None:
+        if len(_pointer_tables) > 64:
+            _pointer_tables.clear()
+        table = torch.tensor(list(key[1]), dtype=torch.int64, device=dev)
+        _pointer_tables[key] = table
+    return table
+
+
+def _check_ranks(name: str, ranks: torch.Tensor, count: int, num_waves: int) -> None:
+    host = host_copy(ranks)
+    if host.numel() < num_waves:
+        raise ValueError(f"{name} is shorter than the wave tables")
+    if int(host[:num_waves].min()) < 0 or int(host[:num_waves].max()) >= count:
+        raise ValueError(f"{name} names a rank outside 0..{count - 1}")
+
+
+def gemm_remote(
+    a,
+    b: torch.Tensor,
+    c,
+    num_gemm_sms: int,
+    BLOCK_SIZE_M: int = 128,
+    BLOCK_SIZE_N: int = 256,
+    BLOCK_SIZE_K: int = 64,
+    GROUP_SIZE_M: int = 8,
+    STAGES: int = 3,
+    *,
+    cur_wave_sizes: TableLike,
+    wave_offsets: TableLike,
+    M: int,
+    a_target_rank: Optional[TableLike] = None,
+    target_rank: Optional[TableLike] = None,
+    dst_offsets: Optional[TableLike] = None,
+    atomic_add: bool = False,
+    signal_ptr: Optional[torch.Tensor] = None,
+    signal_offsets: Optional[TableLike] = None,
+    cum_tiles: int = 0,
+    visit_log: Optional[torch.Tensor] = None,
+    xcd_remap: bool = True,
+    eight_waves: bool = False,
+    stream: Optional[torch.cuda.Stream] = None,
+) -> None:
+    """C = A @ B.T over an [M, N] tile space walked in wave order, with per-wave peer bindings.
+
+    `a` is a tensor [M, K], or a list of per-rank shards [rows, K] together with
+    `a_target_rank` (then the A rows of wave w are rows `tile row inside the wave` of shard
+    a_target_rank[w]).  `c` is a tensor [M, N], or a list of per-rank buffers [rows, ldc]
+    together with `target_rank` and `dst_offsets` ([num_waves, 2] element offsets of the wave's
+    region in the peer buffer); `atomic_add` adds instead of storing.
+    """
+    a_list = list(a) if isinstance(a, (list, tuple)) else None
+    c_list = list(c) if isinstance(c, (list, tuple)) else None
+    if a_list is None and c_list is None:
+        raise ValueError("neither a nor c is bound to peers: use gemm / gemm_consumer")
+    first_a = a_list[0] if a_list is not None else a
+    first_c = c_list[0] if c_list is not None else c
+    dev = require_cuda(first_a, b, first_c)
+    K, N = b.shape[1], b.shape[0]
+    for t in (a_list or [a]):
+        if t.dim() != 2 or t.shape[1] != K or t.dtype != b.dtype or not t.is_contiguous() or t.device != dev:
+            raise ValueError("every A operand must be a contiguous [rows, K] tensor of b's type and device")
+    for t in (c_list or [c]):
+        if t.dim() != 2 or t.dtype != b.dtype or not t.is_contiguous() or t.device != dev:
+            raise ValueError("every C operand must be a contiguous 2-D tensor of b's type and device")
+    if not b.is_contiguous():
+        raise ValueError("b must be contiguous [N, K]")
+    if a_list is None and tuple(a.shape) != (M, K):
+        raise ValueError(f"a must be ({M}, {K})")
+    if c_list is None and tuple(c.shape) != (M, N):
+        raise ValueError(f"c must be ({M}, {N})")
+
+    sizes = as_device_table(cur_wave_sizes, dev, 2)
+    offsets = as_device_table(wave_offsets, dev, 2)
+    num_waves = sizes.shape[0]
+    if offsets.shape[0] != num_waves:
+        raise ValueError("wave size and offset tables disagree on the number of waves")
+    if signal_offsets is None:
+        signals = torch.full((num_waves,), -1, dtype=torch.int32, device=dev)
+        flags = torch.zeros((1,), dtype=torch.int64, device=dev) if signal_ptr is None else signal_ptr
+    else:
+        if signal_ptr is None:
+            raise ValueError("signal_offsets without signal_ptr")
+        signals = as_device_table(signal_offsets, dev, None)
+        flags = signal_ptr
+
+    lib = _lib.load()
+    hs, ho, hg = host_copy(sizes), host_copy(offsets), host_copy(signals)
+    _lib.check("syn_gemm_check_waves",
+               lib.syn_gemm_check_waves(host_ptr(hs), host_ptr(ho), host_ptr(hg), num_waves, M, N, K,
+                                        BLOCK_SIZE_M, BLOCK_SIZE_N, BLOCK_SIZE_K, int(cum_tiles), flags.numel()))
+
+    remote = _lib.GemmRemote()
+    keep = []
+    if a_list is not None:
+        if a_target_rank is None:
+            raise ValueError("a list of A shards needs a_target_rank")
+        a_ranks = as_device_table(a_target_rank, dev, None)
+        _check_ranks("a_target_rank", a_ranks, len(a_list), num_waves)
+        shard_rows = min(t.shape[0] for t in a_list)
+        if int(hs[:, 0].max()) > shard_rows:
+            raise ValueError("a wave has more rows than an A shard")
+        table = _pointer_table(a_list, dev)
+        keep += [a_ranks, table]
+        remote.a_peers, remote.a_target_rank = table.data_ptr(), a_ranks.data_ptr()
+    if c_list is not None:
+        if target_rank is None or dst_offsets is None:
+            raise ValueError("a list of C buffers needs target_rank and dst_offsets")
+        c_ranks = as_device_table(target_rank, dev, None)
+        dst = as_device_table(dst_offsets, dev, 2)
+        _check_ranks("target_rank", c_ranks, len(c_list), num_waves)
+        ldc = c_list[0].shape[1]
+        rows = min(t.shape[0] for t in c_list)
+        if any(t.shape[1] != ldc for t in c_list) or ldc % 4:
+            raise ValueError("peer C buffers must share one row length, a multiple of 4")
+        hd = host_copy(dst)
+        if dst.shape[0] < num_waves or int(hd.min()) < 0:
+            raise ValueError("dst_offsets must hold one non-negative (row, col) pair per wave")
+        if int((hd[:num_waves, 0] + hs[:, 0]).max()) > rows or int((hd[:num_waves, 1] + hs[:, 1]).max()) > ldc:
+            raise ValueError("a wave's destination region does not fit the peer C buffer")
+        if int(hd[:num_waves, 1].max()) % 4:
+            raise ValueError("dst column offsets must be multiples of 4 elements")
+        table = _pointer_table(c_list, dev)
+        keep += [c_ranks, dst, table]
+        remote.c_peers, remote.c_target_rank = table.data_ptr(), c_ranks.data_ptr()
+        remote.c_dst_offsets, remote.c_ld = dst.data_ptr(), ldc
+        remote.c_atomic_add = 1 if atomic_add else 0
+    elif atomic_add:
+        raise ValueError("atomic_add needs c bound to peers")
+
+    if visit_log is not None:
+        tiles = (int(cum_tiles) if cum_tiles else M * N) // (BLOCK_SIZE_M * BLOCK_SIZE_N)
+        if visit_log.dtype != torch.int32 or visit_log.numel() < 4 * tiles or not visit_log.is_contiguous():
+            raise ValueError(f"visit_log must be a contiguous int32 tensor of at least {4 * tiles} words")
+    desc = _lib.GemmDesc(
+        a=None if a_list is not None else a.data_ptr(), b=b.data_ptr(),
+        c=None if c_list is not None else c.data_ptr(), flags=flags.data_ptr(),
+        wave_sizes=sizes.data_ptr(), wave_offsets=offsets.data_ptr(), signal_offsets=signals.data_ptr(),
+        counters=None, visit_log=None if visit_log is None else visit_log.data_ptr(),
+        status=status_words(dev).data_ptr(), num_waves=num_waves, M=M, N=N, K=K,
+        dtype=_lib.dtype_code(b.dtype), block_m=BLOCK_SIZE_M, block_n=BLOCK_SIZE_N, block_k=BLOCK_SIZE_K,
+        group_m=GROUP_SIZE_M, num_sms=num_gemm_sms, cum_tiles=int(cum_tiles), spin_timeout_us=0,
+        options=(_lib.SYN_GEMM_XCD_REMAP if xcd_remap else 0) | (_lib.SYN_GEMM_EIGHT_WAVES if eight_waves else 0),
+    )
+    with torch.cuda.device(dev):
+        _lib.check("syn_gemm_remote_binding",
+                   lib.syn_gemm_remote_binding(ctypes.byref(desc), ctypes.byref(remote), _lib.stream_handle(stream)))
+    del keep
+
+
+def gemm_ag_direct_read(
+    a,
+    b,
+    c,
+    cur_wave_size,
+    wave_offset,
+    target_rank,
+    world_size,
+    local_world_size,
+    num_gemm_sms,
+    use_a_tma: bool = True,
+    BLOCK_SIZE_M=128,
+    BLOCK_SIZE_N=256,
+    BLOCK_SIZE_K=64,
+    GROUP_SIZE_M=8,
+    STAGES=3,
+    **kwargs,
+):
+    """AG+GEMM without a gathered buffer: `a` is the list of the ranks' [M / W, K] shards
+    (index = rank); wave w reads shard target_rank[w]; c is the local [M, N] result
+    (reference: template_ag.py:190-260).  `use_a_tma` is accepted and ignored."""
+    shards = list(a)
+    if len(shards) != world_size:
+        raise ValueError("a must list one shard per rank")
+    local_m = shards[0].shape[0]
+    assert local_m * world_size == c.shape[0], (
+        f"c must hold gathered rows (expected {local_m * world_size}, got {c.shape[0]})")
+    assert c.shape[1] == b.shape[0]
+    gemm_remote(shards, b, c, num_gemm_sms, BLOCK_SIZE_M, BLOCK_SIZE_N, BLOCK_SIZE_K, GROUP_SIZE_M, STAGES,
+                cur_wave_sizes=cur_wave_size, wave_offsets=wave_offset, M=local_m * world_size,
+                a_target_rank=target_rank, cum_tiles=c.shape[0] * c.shape[1], **kwargs)
+
+
+def gemm_rs_producer_persistent(
+    a,
+    b,
+    c,
+    cur_wave_size,
+    wave_offset,
+    target_rank,
+    world_size,
+    local_world_size,
+    num_gemm_sms,
+    BLOCK_SIZE_M=128,
+    BLOCK_SIZE_N=256,
+    BLOCK_SIZE_K=64,
+    GROUP_SIZE_M=8,
+    STAGES=3,
+    use_c_tma: bool = True,
+    **kwargs,
+):
+    """GEMM+RS by remote atomics: a [M, K_local], b [N, K_local]; `c` is the list of the ranks'
+    [M / W, N] results (index = rank), zeroed by the caller's side of the collective; the tile of
+    wave w is added into c[target_rank[w]] at its wave-local row (reference:
+    template_rs.py:212-290; unlike it this launcher neither zeroes c nor barriers: on one GPU
+    the caller launches every rank's kernel in turn on one stream)."""
+    bufs = list(c)
+    if len(bufs) != world_size:
+        raise ValueError("c must list one buffer per rank")
+    m = a.shape[0]
+    m_per_rank = m // world_size
+    assert m_per_rank % BLOCK_SIZE_M == 0
+    # rows are wave-local in the owner's buffer, columns keep their global position
+    # (template_rs.py:157-166: offs_cm from the wave-local pid_m, offs_bn from the global pid_n)
+    dst = host_copy(as_device_table(wave_offset, a.device, 2)).clone()
+    dst[:, 0] = 0
+    gemm_remote(a, b, bufs, num_gemm_sms, BLOCK_SIZE_M, BLOCK_SIZE_N, BLOCK_SIZE_K, GROUP_SIZE_M, STAGES,
+                cur_wave_sizes=cur_wave_size, wave_offsets=wave_offset, M=m, target_rank=target_rank,
+                dst_offsets=dst, atomic_add=True, cum_tiles=m * b.shape[0], **kwargs)

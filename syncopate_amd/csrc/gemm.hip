@@ -43,7 +43,18 @@ struct GemmParams {
     int32_t num_tiles;
     int32_t xcd_remap;
     int32_t k_stagger;
+    // remote bindings (kernel mode 2): per-wave peer tables for A and / or C
+    const void* const* a_peers;
+    const int32_t* a_target;
+    void* const* c_peers;
+    const int32_t* c_target;
+    const int32_t* c_dst_offsets;
+    int32_t c_ld;
+    int32_t c_atomic;
 };
+
+// kernel modes
+constexpr int kConsumer = 0, kProducer = 1, kRemote = 2;
 
 template <typename T>
 struct Mfma32;
@@ -455,8 +466,30 @@ struct RingPipe {
 
 // ------------------------------------------------------------------ kernel
 
-template <typename T, typename Pipe, int BM, int BN, int WGM, int WGN, bool PRODUCER>
+// C += v (four consecutive elements) with two packed 16-bit atomic adds
+template <typename T>
+__device__ __forceinline__ void atomic_add4(T* dst, uint2 v);
+
+template <>
+__device__ __forceinline__ void atomic_add4<__bf16>(__bf16* dst, uint2 v) {
+    typedef __bf16 v2 __attribute__((ext_vector_type(2)));
+    typedef __attribute__((address_space(1))) v2* gptr;
+    __builtin_amdgcn_global_atomic_fadd_v2bf16((gptr)dst, __builtin_bit_cast(v2, v.x));
+    __builtin_amdgcn_global_atomic_fadd_v2bf16((gptr)(dst + 2), __builtin_bit_cast(v2, v.y));
+}
+
+template <>
+__device__ __forceinline__ void atomic_add4<_Float16>(_Float16* dst, uint2 v) {
+    typedef _Float16 v2 __attribute__((ext_vector_type(2)));
+    typedef __attribute__((address_space(1))) v2* gptr;
+    __builtin_amdgcn_global_atomic_fadd_v2f16((gptr)dst, __builtin_bit_cast(v2, v.x));
+    __builtin_amdgcn_global_atomic_fadd_v2f16((gptr)(dst + 2), __builtin_bit_cast(v2, v.y));
+}
+
+template <typename T, typename Pipe, int BM, int BN, int WGM, int WGN, int MODE>
 __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmParams p) {
+    constexpr bool PRODUCER = MODE == kProducer;
+    constexpr bool REMOTE = MODE == kRemote;
     constexpr int WM = BM / WGM, WN = BN / WGN;   // wavefront tile
     constexpr int TM = WM / 32, TN = WN / 32;     // 32x32 MFMA tiles per wavefront
 
@@ -491,6 +524,9 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
     // --- wave walk state (uniform across the workgroup) ---
     int cur_wave = -1, past_tiles = 0, cur_tiles = 0;
     int cur_m = 0, cur_n = 0, off_m = 0, off_n = 0, cur_sig = -1;
+    const T* a_base = nullptr;
+    T* c_base = nullptr;
+    int dst_m = 0, dst_n = 0;
     auto enter_wave = [&](int w) {
         cur_wave = w;
         if (w < kLdsWaves) {
@@ -507,6 +543,16 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
             cur_sig = p.signal_offsets[w];
         }
         cur_tiles = cur_m * cur_n;
+        if (REMOTE) {
+            // the wave's peer: A rows are read from its shard and / or C tiles go into its buffer,
+            // both addressed by wave-local rows (template_ag.py:151-161, template_rs.py:140-166)
+            a_base = p.a_peers ? reinterpret_cast<const T*>(p.a_peers[p.a_target[w]]) : nullptr;
+            if (p.c_peers) {
+                c_base = reinterpret_cast<T*>(p.c_peers[p.c_target[w]]);
+                dst_m = p.c_dst_offsets[2 * w];
+                dst_n = p.c_dst_offsets[2 * w + 1];
+            }
+        }
     };
     enter_wave(0);
 
@@ -551,7 +597,10 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
     };
 
     struct Tile {
-        size_t m0, n0;
+        const unsigned char* a_panel;    // first row of the tile's 'BM' rows of A
+        const unsigned char* b_panel;    // first row of the tile's 'BN' rows of B
+        T* c_tile;                       // element (0, 0) of the tile in its C buffer
+        size_t ldc;
         int k_rot, wave, sig, wave_tiles;
     };
     // get_pid_mn (template.py:10-18) on the wave-local tile id, and the tile's K phase
@@ -561,15 +610,26 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
         const int group_id = local / in_group;
         const int first_m = group_id * p.group_m;
         const int gsz = min(cur_m - first_m, p.group_m);
-        const int pid_m = first_m + (local % gsz) + off_m;
-        const int pid_n = (local % in_group) / gsz + off_n;
+        const int pid_m_local = first_m + (local % gsz);
+        const int pid_n_local = (local % in_group) / gsz;
+        const int pid_m = pid_m_local + off_m;
+        const int pid_n = pid_n_local + off_n;
         if (p.visit_log != nullptr && tid == 0) {
             int4 rec = make_int4(pid, cur_wave, pid_m, pid_n);
             reinterpret_cast<int4*>(p.visit_log)[tile_id] = rec;
         }
         Tile t;
-        t.m0 = (size_t)pid_m * BM;
-        t.n0 = (size_t)pid_n * BN;
+        t.a_panel = reinterpret_cast<const unsigned char*>(A + (size_t)pid_m * BM * K);
+        t.b_panel = reinterpret_cast<const unsigned char*>(B + (size_t)pid_n * BN * K);
+        t.c_tile = C + (size_t)pid_m * BM * N + (size_t)pid_n * BN;
+        t.ldc = (size_t)N;
+        if (REMOTE) {
+            if (a_base) t.a_panel = reinterpret_cast<const unsigned char*>(a_base + (size_t)pid_m_local * BM * K);
+            if (c_base) {
+                t.ldc = (size_t)p.c_ld;
+                t.c_tile = c_base + ((size_t)dst_m + (size_t)pid_m_local * BM) * t.ldc + dst_n + (size_t)pid_n_local * BN;
+            }
+        }
         // Tiles walk K cyclically, neighbouring tiles starting 128 elements apart.  With a
         // power-of-two row pitch, programs that all sweep K from 0 in lockstep keep hitting the
         // same few memory channels; four phases spread them while tiles that share a panel of A
@@ -580,8 +640,8 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
         t.wave_tiles = cur_tiles;
         return t;
     };
-    auto panel_a = [&](const Tile& t) { return reinterpret_cast<const unsigned char*>(A + t.m0 * (size_t)K); };
-    auto panel_b = [&](const Tile& t) { return reinterpret_cast<const unsigned char*>(B + t.n0 * (size_t)K); };
+    auto panel_a = [&](const Tile& t) { return t.a_panel; };
+    auto panel_b = [&](const Tile& t) { return t.b_panel; };
 
     if (tiles_here == 0) return;
     if (advance(pid)) {
@@ -622,7 +682,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
         // D', rows n = 8g + 4*(lane/32) + 0..3: four consecutive elements of one row of C -> one
         // 8-byte store.
         {
-            T* c_row = C + (tile.m0 + wm * WM + (lane & 31)) * (size_t)N + tile.n0 + wn * WN + 4 * (lane >> 5);
+            T* c_row = tile.c_tile + (size_t)(wm * WM + (lane & 31)) * tile.ldc + wn * WN + 4 * (lane >> 5);
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -631,8 +691,10 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
                     for (int g = 0; g < 4; ++g) {
                         const uint2 v = pack4<T>(acc[i][j][4 * g], acc[i][j][4 * g + 1],
                                                  acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
-                        T* dst = c_row + (size_t)(32 * i) * N + 32 * j + 8 * g;
-                        if (PRODUCER) {
+                        T* dst = c_row + (size_t)(32 * i) * tile.ldc + 32 * j + 8 * g;
+                        if (REMOTE && p.c_atomic) {
+                            atomic_add4<T>(dst, v);
+                        } else if (PRODUCER) {
                             // written through the XCD's L2: the release below then has nothing
                             // of this tile left to write back
                             __hip_atomic_store(reinterpret_cast<uint64_t*>(dst), __builtin_bit_cast(uint64_t, v),
@@ -677,48 +739,62 @@ static int64_t gemm_num_tiles(int64_t cum_tiles, int M, int N, int bm, int bn) {
 }
 
 template <typename T, template <typename, int, int, int, int> class PipeT, int BM, int BN, int WGM, int WGN,
-          bool PRODUCER>
+          int MODE>
 static int launch_gemm(const GemmParams& p, int grid, hipStream_t stream) {
     typedef PipeT<T, BM, BN, WGM, WGN> Pipe;
-    hipLaunchKernelGGL((gemm_wave_kernel<T, Pipe, BM, BN, WGM, WGN, PRODUCER>), dim3(grid),
+    hipLaunchKernelGGL((gemm_wave_kernel<T, Pipe, BM, BN, WGM, WGN, MODE>), dim3(grid),
                        dim3(64 * WGM * WGN), 0, stream, p);
     return (int)hipGetLastError();
 }
 
 // Workgroup shapes: 4 wavefronts (2x2, one per SIMD) or 8 (two per SIMD: one can issue MFMAs
 // while the other waits for LDS or a barrier).
-template <typename T, template <typename, int, int, int, int> class PipeT, bool PRODUCER>
+template <typename T, template <typename, int, int, int, int> class PipeT, int MODE>
 static int dispatch_tile(const GemmParams& p, int bm, int bn, bool eight, int grid, hipStream_t stream) {
     if (eight) {
-        if (bm == 256 && bn == 256) return launch_gemm<T, PipeT, 256, 256, 2, 4, PRODUCER>(p, grid, stream);
-        if (bm == 128 && bn == 256) return launch_gemm<T, PipeT, 128, 256, 2, 4, PRODUCER>(p, grid, stream);
-        if (bm == 256 && bn == 128) return launch_gemm<T, PipeT, 256, 128, 4, 2, PRODUCER>(p, grid, stream);
+        if (bm == 256 && bn == 256) return launch_gemm<T, PipeT, 256, 256, 2, 4, MODE>(p, grid, stream);
+        if (bm == 128 && bn == 256) return launch_gemm<T, PipeT, 128, 256, 2, 4, MODE>(p, grid, stream);
+        if (bm == 256 && bn == 128) return launch_gemm<T, PipeT, 256, 128, 4, 2, MODE>(p, grid, stream);
         return SYN_EINVAL;
     }
-    if (bm == 256 && bn == 256) return launch_gemm<T, PipeT, 256, 256, 2, 2, PRODUCER>(p, grid, stream);
-    if (bm == 128 && bn == 256) return launch_gemm<T, PipeT, 128, 256, 2, 2, PRODUCER>(p, grid, stream);
-    if (bm == 256 && bn == 128) return launch_gemm<T, PipeT, 256, 128, 2, 2, PRODUCER>(p, grid, stream);
-    if (bm == 128 && bn == 128) return launch_gemm<T, PipeT, 128, 128, 2, 2, PRODUCER>(p, grid, stream);
+    if (bm == 256 && bn == 256) return launch_gemm<T, PipeT, 256, 256, 2, 2, MODE>(p, grid, stream);
+    if (bm == 128 && bn == 256) return launch_gemm<T, PipeT, 128, 256, 2, 2, MODE>(p, grid, stream);
+    if (bm == 256 && bn == 128) return launch_gemm<T, PipeT, 256, 128, 2, 2, MODE>(p, grid, stream);
+    if (bm == 128 && bn == 128) return launch_gemm<T, PipeT, 128, 128, 2, 2, MODE>(p, grid, stream);
     return SYN_EINVAL;
 }
 
-template <typename T, bool PRODUCER>
+template <typename T, int MODE>
 static int dispatch_pipe(const GemmParams& p, int bm, int bn, bool eight, bool ring, int grid,
                          hipStream_t stream) {
-    if (ring) return dispatch_tile<T, RingPipe, PRODUCER>(p, bm, bn, eight, grid, stream);
-    return dispatch_tile<T, PairPipe, PRODUCER>(p, bm, bn, eight, grid, stream);
+    // the remote-binding form exists for the default pipeline only
+    if (MODE != kRemote) {
+        if (ring) return dispatch_tile<T, RingPipe, MODE == kRemote ? kConsumer : MODE>(p, bm, bn, eight, grid, stream);
+    }
+    return dispatch_tile<T, PairPipe, MODE>(p, bm, bn, eight, grid, stream);
 }
 
-static int gemm_entry(const syn_gemm_desc* d, hipStream_t stream, bool producer) {
+static int gemm_entry(const syn_gemm_desc* d, hipStream_t stream, int mode,
+                      const syn_gemm_remote* remote = nullptr) {
     if (d == nullptr) return SYN_EINVAL;
-    if (!d->a || !d->b || !d->c || !d->wave_sizes || !d->wave_offsets || !d->signal_offsets)
+    const bool producer = mode == kProducer;
+    const bool a_remote = remote && remote->a_peers, c_remote = remote && remote->c_peers;
+    if (mode == kRemote) {
+        if (!remote || (!a_remote && !c_remote)) return SYN_EINVAL;
+        if (a_remote && !remote->a_target_rank) return SYN_EINVAL;
+        if (c_remote && (!remote->c_target_rank || !remote->c_dst_offsets || remote->c_ld <= 0)) return SYN_EINVAL;
+        if (c_remote && remote->c_ld % 4) return SYN_EALIGN;
+        if (remote->c_atomic_add && !c_remote) return SYN_EINVAL;
+    }
+    if ((!d->a && !a_remote) || !d->b || (!d->c && !c_remote) || !d->wave_sizes || !d->wave_offsets ||
+        !d->signal_offsets)
         return SYN_EINVAL;
     if (d->num_waves <= 0 || d->M <= 0 || d->N <= 0 || d->K <= 0) return SYN_EINVAL;
     if (d->block_k != 64) return SYN_EINVAL;
     if (d->group_m <= 0 || d->num_sms <= 0) return SYN_EINVAL;
     if (d->dtype != SYN_DTYPE_BF16 && d->dtype != SYN_DTYPE_FP16) return SYN_EINVAL;
     if (d->M % d->block_m || d->N % d->block_n || d->K % 64) return SYN_EINVAL;
-    if (!aligned16(d->a) || !aligned16(d->b) || !aligned16(d->c)) return SYN_EALIGN;
+    if ((d->a && !aligned16(d->a)) || !aligned16(d->b) || (d->c && !aligned16(d->c))) return SYN_EALIGN;
     if (producer && d->counters == nullptr) return SYN_EINVAL;
     if (d->flags == nullptr) return SYN_EINVAL;
     if (d->visit_log && !aligned16(d->visit_log)) return SYN_EALIGN;
@@ -751,16 +827,26 @@ static int gemm_entry(const syn_gemm_desc* d, hipStream_t stream, bool producer)
     p.num_tiles = (int)tiles;
     p.xcd_remap = (d->options & SYN_GEMM_XCD_REMAP) ? 1 : 0;
     p.k_stagger = (d->options & SYN_GEMM_NO_K_STAGGER) ? 0 : 1;
+    p.a_peers = a_remote ? remote->a_peers : nullptr;
+    p.a_target = a_remote ? remote->a_target_rank : nullptr;
+    p.c_peers = c_remote ? remote->c_peers : nullptr;
+    p.c_target = c_remote ? remote->c_target_rank : nullptr;
+    p.c_dst_offsets = c_remote ? remote->c_dst_offsets : nullptr;
+    p.c_ld = c_remote ? remote->c_ld : 0;
+    p.c_atomic = (remote && remote->c_atomic_add) ? 1 : 0;
     const bool eight = (d->options & SYN_GEMM_EIGHT_WAVES) != 0;
     // the ring needs whole groups of four 32-deep slabs
     const bool ring = (d->options & SYN_GEMM_RING_PIPE) && d->K % 128 == 0;
 
+    const int bm = d->block_m, bn = d->block_n;
     if (d->dtype == SYN_DTYPE_BF16) {
-        return producer ? dispatch_pipe<__bf16, true>(p, d->block_m, d->block_n, eight, ring, grid, stream)
-                        : dispatch_pipe<__bf16, false>(p, d->block_m, d->block_n, eight, ring, grid, stream);
+        if (mode == kRemote) return dispatch_pipe<__bf16, kRemote>(p, bm, bn, eight, false, grid, stream);
+        return producer ? dispatch_pipe<__bf16, kProducer>(p, bm, bn, eight, ring, grid, stream)
+                        : dispatch_pipe<__bf16, kConsumer>(p, bm, bn, eight, ring, grid, stream);
     }
-    return producer ? dispatch_pipe<_Float16, true>(p, d->block_m, d->block_n, eight, ring, grid, stream)
-                    : dispatch_pipe<_Float16, false>(p, d->block_m, d->block_n, eight, ring, grid, stream);
+    if (mode == kRemote) return dispatch_pipe<_Float16, kRemote>(p, bm, bn, eight, false, grid, stream);
+    return producer ? dispatch_pipe<_Float16, kProducer>(p, bm, bn, eight, ring, grid, stream)
+                    : dispatch_pipe<_Float16, kConsumer>(p, bm, bn, eight, ring, grid, stream);
 }
 
 }  // namespace syn
@@ -768,11 +854,15 @@ static int gemm_entry(const syn_gemm_desc* d, hipStream_t stream, bool producer)
 extern "C" {
 
 int syn_gemm_consumer(const syn_gemm_desc* desc, syn_stream_t stream) {
-    return syn::gemm_entry(desc, reinterpret_cast<hipStream_t>(stream), false);
+    return syn::gemm_entry(desc, reinterpret_cast<hipStream_t>(stream), syn::kConsumer);
 }
 
 int syn_gemm_producer(const syn_gemm_desc* desc, syn_stream_t stream) {
-    return syn::gemm_entry(desc, reinterpret_cast<hipStream_t>(stream), true);
+    return syn::gemm_entry(desc, reinterpret_cast<hipStream_t>(stream), syn::kProducer);
+}
+
+int syn_gemm_remote_binding(const syn_gemm_desc* desc, const syn_gemm_remote* remote, syn_stream_t stream) {
+    return syn::gemm_entry(desc, reinterpret_cast<hipStream_t>(stream), syn::kRemote, remote);
 }
 
 int syn_gemm_grid(int64_t cum_tiles, int32_t M, int32_t N, int32_t block_m, int32_t block_n,
