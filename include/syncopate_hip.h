@@ -43,12 +43,14 @@ extern "C" {
                                        logical program ids share an XCD (and its L2)      */
 #define SYN_GEMM_EIGHT_WAVES 2u     /* 512-thread workgroups (two wavefronts per SIMD)     */
 #define SYN_GEMM_RING_PIPE 4u       /* four LDS stages of 32-deep K slabs instead of the default
-                                       two stages of 64-deep slabs; needs K % 128 == 0,
+                                       two or three stages of 64-deep slabs; needs K % 128 == 0,
                                        otherwise the default pipeline runs                 */
 #define SYN_GEMM_NO_K_STAGGER 8u    /* every tile sweeps K from 0 (default: neighbouring
                                        tiles start 128 elements apart and wrap around, which
                                        spreads lockstep programs over the memory channels;
                                        the fp32 sums are then taken in rotated order)      */
+#define SYN_GEMM_TWO_STAGE 16u      /* two LDS stages even for tiles of which three fit (every
+                                       shape but 256x256): one slab in flight instead of two */
 
 typedef void* syn_stream_t;        /* hipStream_t */
 

@@ -27,6 +27,7 @@ SYN_GEMM_XCD_REMAP = 1
 SYN_GEMM_EIGHT_WAVES = 2
 SYN_GEMM_RING_PIPE = 4
 SYN_GEMM_NO_K_STAGGER = 8
+SYN_GEMM_TWO_STAGE = 16
 
 _ERRORS = {
     SYN_EINVAL: "SYN_EINVAL (malformed argument or unsupported configuration)",

@@ -55,6 +55,7 @@ def _launch(
     eight_waves: bool,
     ring_pipe: bool,
     k_stagger: bool,
+    two_stage: bool,
     spin_timeout_us: int,
     stream: Optional[torch.cuda.Stream],
 ) -> None:
@@ -134,7 +135,8 @@ def _launch(
         cum_tiles=int(cum_tiles),
         spin_timeout_us=int(spin_timeout_us),
         options=(_lib.SYN_GEMM_XCD_REMAP if xcd_remap else 0) | (_lib.SYN_GEMM_EIGHT_WAVES if eight_waves else 0)
-        | (_lib.SYN_GEMM_RING_PIPE if ring_pipe else 0) | (0 if k_stagger else _lib.SYN_GEMM_NO_K_STAGGER),
+        | (_lib.SYN_GEMM_RING_PIPE if ring_pipe else 0) | (0 if k_stagger else _lib.SYN_GEMM_NO_K_STAGGER)
+        | (_lib.SYN_GEMM_TWO_STAGE if two_stage else 0),
     )
     with torch.cuda.device(dev):
         fn = lib.syn_gemm_producer if producer else lib.syn_gemm_consumer
@@ -164,6 +166,7 @@ def gemm_consumer(
     eight_waves=False,
     ring_pipe=False,
     k_stagger=True,
+    two_stage=False,
     spin_timeout_us=DEFAULT_SPIN_TIMEOUT_US,
     stream=None,
 ):
@@ -179,7 +182,7 @@ def gemm_consumer(
     assert M_per_rank % BLOCK_SIZE_M == 0
     _launch(False, a, b, c, signal_buffer, cur_wave_size, wave_offset, signal_offsets, num_gemm_sms,
             BLOCK_SIZE_M, BLOCK_SIZE_N, BLOCK_SIZE_K, GROUP_SIZE_M, cum_tiles, None, visit_log,
-            xcd_remap, eight_waves, ring_pipe, k_stagger, spin_timeout_us, stream)
+            xcd_remap, eight_waves, ring_pipe, k_stagger, two_stage, spin_timeout_us, stream)
 
 
 def gemm_producer(
@@ -204,6 +207,7 @@ def gemm_producer(
     eight_waves=False,
     ring_pipe=False,
     k_stagger=True,
+    two_stage=False,
     stream=None,
 ):
     """GEMM+RS producer: same GEMM; every finished tile bumps its wave's counter
@@ -213,7 +217,7 @@ def gemm_producer(
     """
     _launch(True, a, b, c, signal_buffer, cur_wave_size, wave_offset, signal_offsets, num_gemm_sms,
             BLOCK_SIZE_M, BLOCK_SIZE_N, BLOCK_SIZE_K, GROUP_SIZE_M, cum_tiles, counter_buffer,
-            visit_log, xcd_remap, eight_waves, ring_pipe, k_stagger, DEFAULT_SPIN_TIMEOUT_US, stream)
+            visit_log, xcd_remap, eight_waves, ring_pipe, k_stagger, two_stage, DEFAULT_SPIN_TIMEOUT_US, stream)
 
 
 def gemm(
@@ -239,6 +243,7 @@ def gemm(
     eight_waves=False,
     ring_pipe=False,
     k_stagger=True,
+    two_stage=False,
     spin_timeout_us=DEFAULT_SPIN_TIMEOUT_US,
     stream=None,
 ):
@@ -249,4 +254,4 @@ def gemm(
     """
     _launch(counter_ptr is not None, a, b, c, signal_ptr, cur_wave_sizes, wave_offsets, signal_offsets,
             num_gemm_sms, BLOCK_SIZE_M, BLOCK_SIZE_N, BLOCK_SIZE_K, GROUP_SIZE_M, cum_tiles,
-            counter_ptr, visit_log, xcd_remap, eight_waves, ring_pipe, k_stagger, spin_timeout_us, stream)
+            counter_ptr, visit_log, xcd_remap, eight_waves, ring_pipe, k_stagger, two_stage, spin_timeout_us, stream)

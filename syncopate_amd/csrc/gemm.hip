@@ -10,8 +10,9 @@
 //
 // Two pipelines over the same tile walk, both with one barrier per slab and MFMA work on
 // both sides of it:
-//   pair   2 stages of 64-deep slabs: rows are whole 128-byte cache lines, one slab in flight
-//          while the other is multiplied; any K % 64 == 0.  The default.
+//   slab   2 or 3 stages of 64-deep slabs: rows are whole 128-byte cache lines; one slab (two,
+//          where three stages fit the 160 KB of LDS: every tile but 256x256) in flight while
+//          another is multiplied; any K % 64 == 0.  The default.
 //   ring   4 stages of 32-deep slabs, three in flight; rows are half cache lines, which costs
 //          L1 fill bandwidth.  Needs K % 128 == 0.
 // A tile's first fills are issued before the previous tile's C is stored.
@@ -206,6 +207,30 @@ __device__ __forceinline__ void dma_part(unsigned char* stage, const unsigned ch
     }
 }
 
+#ifdef SYN_EXP_TIMING
+__device__ long long g_timing[256 * 8][8];
+struct TimingAcc { long long wait = 0, bar = 0, fillissue = 0; };
+__device__ TimingAcc* g_tacc_dummy;
+#define SYN_T() __builtin_amdgcn_s_memtime()
+#endif
+
+// The same for the slab pipelines, shaped so that a fill costs two instructions (M0, load): the
+// wavefront's fill j is 1 KB block j * NW + wave of the stage; blocks of A come first and BM / 8
+// is a multiple of NW, so whether fill j reads A or B is known at compile time.  `a_k` / `b_k`
+// are the wavefront-uniform addresses of the panels at this slab's k, voff[i] the lane's byte
+// offset for the i-th block of an operand (its row inside block i * NW + wave, and the swizzled
+// 16-byte chunk): uniform base + 32-bit lane offset is the scalar-base addressing form.
+template <int FIRST, int LAST, int BM, int NW, int NV>
+__device__ __forceinline__ void dma_blocks(unsigned char* stage_wave, const unsigned char* a_k,
+                                           const unsigned char* b_k, const unsigned (&voff)[NV]) {
+    constexpr int kAFills = BM / (8 * NW);
+#pragma unroll
+    for (int j = FIRST; j < LAST; ++j) {
+        const unsigned char* src = j < kAFills ? a_k + voff[j] : b_k + voff[j - kAFills];
+        __builtin_amdgcn_global_load_lds((global_void_ptr)src, (lds_void_ptr)(stage_wave + j * NW * 1024), 16, 0, 0);
+    }
+}
+
 // ------------------------------------------------------------------ pipelines
 //
 // Both are split in two: prologue() issues the first fills of a tile from the uniform addresses
@@ -213,7 +238,8 @@ __device__ __forceinline__ void dma_part(unsigned char* stage, const unsigned ch
 // main() returns every fill has landed and every wavefront has passed a barrier, so the stages
 // may be refilled at once - the kernel issues the next tile's prologue before it stores C.
 
-// pair: two stages of 64-deep slabs.  LDS row r (128 bytes) keeps logical chunk c at physical
+// slab: NST = two or three stages of 64-deep slabs (the description is for two; with three the
+// refill is slab s+3 and a fill has two slab times to land).  LDS row r (128 bytes) keeps logical chunk c at physical
 // chunk c ^ ((r >> 1) & 7): a row covers half of the 64 banks (even rows the low half), a
 // 128-bit read is served 16 consecutive rows per cycle, and (r >> 1) & 7 gives the 8 rows that
 // share a half 8 distinct chunks.  Rows are whole 128-byte cache lines.
@@ -225,8 +251,8 @@ __device__ __forceinline__ void dma_part(unsigned char* stage, const unsigned ch
 //                                    into the stage slab s has just been read out of
 // so a barrier costs no LDS latency and a fill has one slab time to land.  Fills past the
 // last slab re-fetch it (nothing reads them).
-template <typename T, int BM, int BN, int WGM, int WGN>
-struct PairPipe {
+template <typename T, int BM, int BN, int WGM, int WGN, int NST>
+struct SlabPipe {
     static constexpr int NW = WGM * WGN;
     static constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
     static constexpr int BK = 64, ROW = BK * 2;
@@ -235,47 +261,89 @@ struct PairPipe {
     static constexpr int K_ALIGN = 64;
     typedef typename Mfma32<T>::frag_t frag_t;
 
+    static constexpr int NV = (BM > BN ? BM : BN) / (8 * NW);    // fills per wavefront and operand
+    static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "whole fills per wavefront and operand");
     struct Lane {
-        unsigned lane_off;
+        unsigned voff[NV];
         int a_rd, b_rd, half, swz;
     };
 
     static __device__ __forceinline__ void fill(unsigned char* st, const unsigned char* a_slab,
                                                 const unsigned char* b_slab, size_t k_off, const Lane& ln,
                                                 size_t row_bytes, int wave) {
-        dma_part<0, FILLS, BM, ROW, NW>(st, a_slab + k_off, b_slab + k_off, ln.lane_off, row_bytes, wave);
+        dma_blocks<0, FILLS, BM, NW, NV>(st + wave * 1024, a_slab + k_off, b_slab + k_off, ln.voff);
     }
 
-    // f0 holds the fragments of (cur, step 0) on entry and of (nxt, step 0) on exit
+    // With three stages a slab's fills go out in four parts, one per k16 step, so that the
+    // vector-memory queue never holds more than a few of them: part 0 of slab s+3 in step 3 of
+    // slab s (into the stage slab s has left), parts 1-3 in steps 0-2 of slab s+1.
+    static constexpr int SPREAD = NST == 3;
+    static constexpr int part_begin(int q) { return SPREAD ? FILLS * q / 4 : (q == 0 ? 0 : FILLS); }
+    template <int Q>
+    static __device__ __forceinline__ void fill_part(unsigned char* st, const unsigned char* a_slab,
+                                                     const unsigned char* b_slab, size_t k_off, const Lane& ln,
+                                                     size_t row_bytes, int wave) {
+        dma_blocks<part_begin(Q), part_begin(Q + 1), BM, NW, NV>(st + wave * 1024, a_slab + k_off, b_slab + k_off,
+                                                                 ln.voff);
+    }
+    template <int Q>
+    static constexpr int part_size() { return part_begin(Q + 1) - part_begin(Q); }
+
+    // f0 holds the fragments of (cur, step 0) on entry and of (nxt, step 0) on exit.  `prv` is the
+    // stage of slab s-1 (three stages only), which takes parts 1-3 of slab s+2 (at k_prev).
     static __device__ __forceinline__ void slab(f32x16_t (&acc)[TM][TN], frag_t (&fa0)[TM], frag_t (&fb0)[TN],
-                                                unsigned char* cur, const unsigned char* nxt,
+                                                unsigned char* cur, const unsigned char* nxt, unsigned char* prv,
                                                 const unsigned char* a_slab, const unsigned char* b_slab,
-                                                size_t k_refill, const Lane& ln, size_t row_bytes, int wave) {
+                                                size_t k_refill, size_t k_prev, const Lane& ln, size_t row_bytes,
+                                                int wave
+#ifdef SYN_EXP_TIMING
+                                                , long long& tw, long long& tb, long long& t012, long long& t3
+#endif
+                                                ) {
         frag_t fa1[TM], fb1[TN];
+#ifdef SYN_EXP_TIMING
+        const long long ts = SYN_T();
+#endif
+        if constexpr (SPREAD) fill_part<1>(prv, a_slab, b_slab, k_prev, ln, row_bytes, wave);
         load_frags<T, TM, TN, ROW>(fa1, fb1, cur, ln.a_rd, ln.b_rd, ((2 + ln.half) ^ ln.swz) << 4);
         mma_step<T, TM, TN>(acc, fa0, fb0);
-        spread_hint<TM + TN, TM * TN, 0>();
+        spread_hint<TM + TN, TM * TN, SPREAD ? part_size<1>() : 0>();
         __builtin_amdgcn_sched_barrier(0);
 
+        if constexpr (SPREAD) fill_part<2>(prv, a_slab, b_slab, k_prev, ln, row_bytes, wave);
         load_frags<T, TM, TN, ROW>(fa0, fb0, cur, ln.a_rd, ln.b_rd, ((4 + ln.half) ^ ln.swz) << 4);
         mma_step<T, TM, TN>(acc, fa1, fb1);
-        spread_hint<TM + TN, TM * TN, 0>();
+        spread_hint<TM + TN, TM * TN, SPREAD ? part_size<2>() : 0>();
         __builtin_amdgcn_sched_barrier(0);
 
+        if constexpr (SPREAD) fill_part<3>(prv, a_slab, b_slab, k_prev, ln, row_bytes, wave);
         load_frags<T, TM, TN, ROW>(fa1, fb1, cur, ln.a_rd, ln.b_rd, ((6 + ln.half) ^ ln.swz) << 4);
         mma_step<T, TM, TN>(acc, fa0, fb0);
-        spread_hint<TM + TN, TM * TN, 0>();
+        spread_hint<TM + TN, TM * TN, SPREAD ? part_size<3>() : 0>();
         __builtin_amdgcn_sched_barrier(0);
 
-        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, true));
+        // own fills of slab s+1 landed (those of slab s+2, all younger, may fly on)
+#ifdef SYN_EXP_TIMING
+        const long long t0 = SYN_T();
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm((NST - 2) * FILLS, true));
+        const long long t1 = SYN_T();
         __builtin_amdgcn_s_barrier();
+        const long long t2 = SYN_T();
+        tw += t1 - t0; tb += t2 - t1; t012 += t0 - ts;
+#else
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm((NST - 2) * FILLS, true));
+        __builtin_amdgcn_s_barrier();
+#endif
         __builtin_amdgcn_sched_barrier(0);
 
-        fill(cur, a_slab, b_slab, k_refill, ln, row_bytes, wave);
+        fill_part<0>(cur, a_slab, b_slab, k_refill, ln, row_bytes, wave);
         load_frags<T, TM, TN, ROW>(fa0, fb0, nxt, ln.a_rd, ln.b_rd, ((0 + ln.half) ^ ln.swz) << 4);
         mma_step<T, TM, TN>(acc, fa1, fb1);
-        spread_hint<TM + TN, TM * TN, FILLS>();
+        spread_hint<TM + TN, TM * TN, part_size<0>()>();
         __builtin_amdgcn_sched_barrier(0);
+#ifdef SYN_EXP_TIMING
+        t3 += SYN_T() - t2;
+#endif
     }
 
     // the stages are distinct objects: LDS reads of one never wait for fills of the other
@@ -291,7 +359,9 @@ struct PairPipe {
         const int ld_row = lane >> 3;
         // blocks this wavefront fills are wave, wave + NW, ... (NW even): block parity = wave parity
         const int ld_chunk = (lane & 7) ^ ((((wave & 1) << 3 | ld_row) >> 1) & 7);
-        ln.lane_off = (unsigned)(ld_row * row_bytes) + ld_chunk * 16;
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+            ln.voff[i] = (unsigned)(((i * NW + wave) * 8 + ld_row) * row_bytes) + ld_chunk * 16;
         ln.half = lane >> 5;
         ln.swz = (lane >> 1) & 7;
         ln.a_rd = (wm * WM + (lane & 31)) * ROW;
@@ -313,6 +383,7 @@ struct PairPipe {
         const int k_steps = K / BK, rot = k_rot % k_steps;
         fill(stage<0>(), a_slab, b_slab, slab_off(0, rot, k_steps), ln, row_bytes, wave);
         fill(stage<1>(), a_slab, b_slab, slab_off(1, rot, k_steps), ln, row_bytes, wave);
+        if constexpr (NST == 3) fill_part<0>(stage<2>(), a_slab, b_slab, slab_off(2, rot, k_steps), ln, row_bytes, wave);
     }
 
     // The K loop of a tile whose prologue has been issued.  On return every fill has landed and
@@ -323,28 +394,186 @@ struct PairPipe {
         unsigned char* const stage0 = stage<0>();
         unsigned char* const stage1 = stage<1>();
         const Lane ln = make_lane(row_bytes, lane, wave);
-        const int k_steps = K / BK, last = k_steps - 1;
+        const int k_steps = K / BK;
         const int rot = k_rot % k_steps;
 
-        __builtin_amdgcn_s_waitcnt(waitcnt_imm(FILLS, true));       // slab 0 landed; slab 1 may fly on
+        // slab 0 landed; slab 1 (and part 0 of slab 2) may fly on
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(FILLS + (NST == 3 ? part_size<0>() : 0), true));
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
         frag_t fa0[TM], fb0[TN];
         load_frags<T, TM, TN, ROW>(fa0, fb0, stage0, ln.a_rd, ln.b_rd, ((0 + ln.half) ^ ln.swz) << 4);
 
-        const int pairs = k_steps >> 1;
-        for (int pr = 0; pr < pairs; ++pr) {
-            slab(acc, fa0, fb0, stage0, stage1, a_slab, b_slab, slab_off(2 * pr + 2, rot, k_steps), ln, row_bytes, wave);
-            slab(acc, fa0, fb0, stage1, stage0, a_slab, b_slab, slab_off(2 * pr + 3, rot, k_steps), ln, row_bytes, wave);
+#ifdef SYN_EXP_TIMING
+        long long tw = 0, tb = 0, t012 = 0, t3 = 0;
+        const long long tk0 = SYN_T();
+        auto run = [&](unsigned char* cur, const unsigned char* nxt, unsigned char* prv, int s) {
+            slab(acc, fa0, fb0, cur, nxt, prv, a_slab, b_slab, slab_off(s + NST, rot, k_steps),
+                 slab_off(s + 2, rot, k_steps), ln, row_bytes, wave, tw, tb, t012, t3);
+        };
+#else
+        auto run = [&](unsigned char* cur, const unsigned char* nxt, unsigned char* prv, int s) {
+            slab(acc, fa0, fb0, cur, nxt, prv, a_slab, b_slab, slab_off(s + NST, rot, k_steps),
+                 slab_off(s + 2, rot, k_steps), ln, row_bytes, wave);
+        };
+#endif
+        if constexpr (NST == 2) {
+            const int pairs = k_steps >> 1;
+            for (int pr = 0; pr < pairs; ++pr) {
+                run(stage0, stage1, stage1, 2 * pr);
+                run(stage1, stage0, stage0, 2 * pr + 1);
+            }
+            if (k_steps & 1) run(stage0, stage1, stage1, k_steps - 1);
+        } else {
+            unsigned char* const stage2 = stage<2>();
+            const int triples = k_steps / 3, rest = k_steps - 3 * triples;
+            for (int tr = 0; tr < triples; ++tr) {
+                run(stage0, stage1, stage2, 3 * tr);
+                run(stage1, stage2, stage0, 3 * tr + 1);
+                run(stage2, stage0, stage1, 3 * tr + 2);
+            }
+            if (rest >= 1) run(stage0, stage1, stage2, 3 * triples);
+            if (rest == 2) run(stage1, stage2, stage0, 3 * triples + 1);
         }
-        if (k_steps & 1)
-            slab(acc, fa0, fb0, stage0, stage1, a_slab, b_slab, slab_off(last, rot, k_steps), ln, row_bytes, wave);
+#ifdef SYN_EXP_TIMING
+        if (lane == 0) {
+            long long* g = g_timing[(blockIdx.x % 256) * 8 + wave];
+            g[0] += tw; g[1] += tb; g[2] += SYN_T() - tk0; g[3] += 1; g[4] += t012; g[5] += t3;
+        }
+#endif
         // drain the re-fetches of the last slab before anything refills the stages
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, true));
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
     }
 };
+
+template <typename T, int BM, int BN, int WGM, int WGN>
+using PairPipe = SlabPipe<T, BM, BN, WGM, WGN, 2>;
+// early: two stages again, for the tile of which only two fit (256x256), with the LDS reads of a
+// slab bunched at its start so that its stage can be refilled during three of the four k16 steps
+// instead of one.  A wavefront keeps the fragments of all four steps in registers (128 VGPRs):
+//     step 3 of slab s-1: MFMAs | read the fragments of steps 0, 1 of slab s
+//     step 0: MFMAs | read the fragments of steps 2, 3;  wait for them;  barrier: the stage is free
+//     step 1: MFMAs | first third of the fills of slab s+2 into that stage
+//     step 2: MFMAs | second third;  wait: own fills of slab s+1 landed;  barrier
+//     step 3: MFMAs | last third | read steps 0, 1 of slab s+1
+// 64 fills of 1 KB take the texture path of a compute unit about 1400 cycles, a k16 step of MFMAs
+// 512: issued in one step they hold the wavefronts (and their MFMAs) up, spread over three they
+// do not.
+template <typename T, int BM, int BN, int WGM, int WGN>
+struct EarlyPipe : SlabPipe<T, BM, BN, WGM, WGN, 2> {
+    typedef SlabPipe<T, BM, BN, WGM, WGN, 2> Base;
+    using Base::TM;
+    using Base::TN;
+    using Base::ROW;
+    using Base::FILLS;
+    using Base::NW;
+    using Base::NV;
+    using Base::BK;
+    typedef typename Base::frag_t frag_t;
+    typedef typename Base::Lane Lane;
+    static constexpr int PA = (FILLS + 2) / 3, PB = (FILLS - PA + 1) / 2, PC = FILLS - PA - PB;
+
+    template <int STEP>
+    static __device__ __forceinline__ void read_step(frag_t (&fa)[TM], frag_t (&fb)[TN], const unsigned char* st,
+                                                     const Lane& ln) {
+        load_frags<T, TM, TN, ROW>(fa, fb, st, ln.a_rd, ln.b_rd, ((2 * STEP + ln.half) ^ ln.swz) << 4);
+    }
+
+    // MFMAS MFMAs with READS LDS reads bunched two per MFMA at the front and FILLS fills spread out
+    template <int G, int MFMAS, int READS, int NFILL>
+    static __device__ __forceinline__ void hint_front() {
+        if constexpr (G < MFMAS) {
+            __builtin_amdgcn_sched_group_barrier(kSgMfma, 1, 0);
+            constexpr int r = (2 * (G + 1) < READS ? 2 * (G + 1) : READS) - (2 * G < READS ? 2 * G : READS);
+            constexpr int f = NFILL * (G + 1) / MFMAS - NFILL * G / MFMAS;
+            if constexpr (r > 0) __builtin_amdgcn_sched_group_barrier(kSgDsRead, r, 0);
+            if constexpr (f > 0) __builtin_amdgcn_sched_group_barrier(kSgVmemRead, f, 0);
+            hint_front<G + 1, MFMAS, READS, NFILL>();
+        }
+    }
+
+    static __device__ __forceinline__ void slab(f32x16_t (&acc)[TM][TN], frag_t (&fa)[4][TM], frag_t (&fb)[4][TN],
+                                                unsigned char* cur, const unsigned char* nxt,
+                                                const unsigned char* a_slab, const unsigned char* b_slab,
+                                                size_t k_refill, const Lane& ln, int wave) {
+        const unsigned char* a_k = a_slab + k_refill;
+        const unsigned char* b_k = b_slab + k_refill;
+        unsigned char* const dst = cur + wave * 1024;
+
+        read_step<2>(fa[2], fb[2], cur, ln);
+        read_step<3>(fa[3], fb[3], cur, ln);
+        mma_step<T, TM, TN>(acc, fa[0], fb[0]);
+        hint_front<0, TM * TN, 2 * (TM + TN), 0>();
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, true));     // own reads of this stage returned
+        __builtin_amdgcn_s_barrier();                          // everyone's: the stage is free
+        __builtin_amdgcn_sched_barrier(0);
+
+        dma_blocks<0, PA, BM, NW, NV>(dst, a_k, b_k, ln.voff);
+        mma_step<T, TM, TN>(acc, fa[1], fb[1]);
+        spread_hint<0, TM * TN, PA>();
+        __builtin_amdgcn_sched_barrier(0);
+
+        dma_blocks<PA, PA + PB, BM, NW, NV>(dst, a_k, b_k, ln.voff);
+        mma_step<T, TM, TN>(acc, fa[2], fb[2]);
+        spread_hint<0, TM * TN, PB>();
+        __builtin_amdgcn_sched_barrier(0);
+        // own fills of slab s+1 landed (the two thirds of slab s+2 issued since may fly on)
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(PA + PB, false));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+
+        dma_blocks<PA + PB, FILLS, BM, NW, NV>(dst, a_k, b_k, ln.voff);
+        read_step<0>(fa[0], fb[0], nxt, ln);
+        read_step<1>(fa[1], fb[1], nxt, ln);
+        mma_step<T, TM, TN>(acc, fa[3], fb[3]);
+        hint_front<0, TM * TN, 2 * (TM + TN), PC>();
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    static __device__ __forceinline__ void main(f32x16_t (&acc)[TM][TN], const unsigned char* a_slab,
+                                                const unsigned char* b_slab, size_t row_bytes, int K,
+                                                int k_rot, int lane, int wave) {
+        unsigned char* const stage0 = Base::template stage<0>();
+        unsigned char* const stage1 = Base::template stage<1>();
+        const Lane ln = Base::make_lane(row_bytes, lane, wave);
+        const int k_steps = K / BK;
+        const int rot = k_rot % k_steps;
+
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(FILLS, true));       // slab 0 landed; slab 1 may fly on
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        frag_t fa[4][TM], fb[4][TN];
+        read_step<0>(fa[0], fb[0], stage0, ln);
+        read_step<1>(fa[1], fb[1], stage0, ln);
+
+        const int pairs = k_steps >> 1;
+        for (int pr = 0; pr < pairs; ++pr) {
+            slab(acc, fa, fb, stage0, stage1, a_slab, b_slab, Base::slab_off(2 * pr + 2, rot, k_steps), ln, wave);
+            slab(acc, fa, fb, stage1, stage0, a_slab, b_slab, Base::slab_off(2 * pr + 3, rot, k_steps), ln, wave);
+        }
+        if (k_steps & 1)
+            slab(acc, fa, fb, stage0, stage1, a_slab, b_slab, Base::slab_off(k_steps + 1, rot, k_steps), ln, wave);
+        // drain the re-fetches of the last slab before anything refills the stages
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, true));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+    }
+};
+
+// the deepest arrangement that fits next to the wave table: three stages, or the early-read form
+template <typename T, int BM, int BN, int WGM, int WGN, bool THREE = (3 * (BM + BN) * 128 <= 150 * 1024)>
+struct DeepPipeSel {
+    typedef SlabPipe<T, BM, BN, WGM, WGN, 3> type;
+};
+template <typename T, int BM, int BN, int WGM, int WGN>
+struct DeepPipeSel<T, BM, BN, WGM, WGN, false> {
+    typedef EarlyPipe<T, BM, BN, WGM, WGN> type;
+};
+template <typename T, int BM, int BN, int WGM, int WGN>
+using DeepPipe = typename DeepPipeSel<T, BM, BN, WGM, WGN>::type;
 
 // ring: four stages of 32-deep slabs.  LDS row r (64 bytes) keeps logical chunk c at physical
 // chunk c ^ ((r >> 2) & 3): 16 consecutive rows then hit 16 distinct 16-byte bank groups.
@@ -765,13 +994,14 @@ static int dispatch_tile(const GemmParams& p, int bm, int bn, bool eight, int gr
 }
 
 template <typename T, int MODE>
-static int dispatch_pipe(const GemmParams& p, int bm, int bn, bool eight, bool ring, int grid,
+static int dispatch_pipe(const GemmParams& p, int bm, int bn, bool eight, bool ring, bool two_stage, int grid,
                          hipStream_t stream) {
     // the remote-binding form exists for the default pipeline only
     if (MODE != kRemote) {
         if (ring) return dispatch_tile<T, RingPipe, MODE == kRemote ? kConsumer : MODE>(p, bm, bn, eight, grid, stream);
+        if (two_stage) return dispatch_tile<T, PairPipe, MODE == kRemote ? kConsumer : MODE>(p, bm, bn, eight, grid, stream);
     }
-    return dispatch_tile<T, PairPipe, MODE>(p, bm, bn, eight, grid, stream);
+    return dispatch_tile<T, DeepPipe, MODE>(p, bm, bn, eight, grid, stream);
 }
 
 static int gemm_entry(const syn_gemm_desc* d, hipStream_t stream, int mode,
@@ -839,14 +1069,15 @@ static int gemm_entry(const syn_gemm_desc* d, hipStream_t stream, int mode,
     const bool ring = (d->options & SYN_GEMM_RING_PIPE) && d->K % 128 == 0;
 
     const int bm = d->block_m, bn = d->block_n;
+    const bool two = (d->options & SYN_GEMM_TWO_STAGE) != 0;
     if (d->dtype == SYN_DTYPE_BF16) {
-        if (mode == kRemote) return dispatch_pipe<__bf16, kRemote>(p, bm, bn, eight, false, grid, stream);
-        return producer ? dispatch_pipe<__bf16, kProducer>(p, bm, bn, eight, ring, grid, stream)
-                        : dispatch_pipe<__bf16, kConsumer>(p, bm, bn, eight, ring, grid, stream);
+        if (mode == kRemote) return dispatch_pipe<__bf16, kRemote>(p, bm, bn, eight, false, false, grid, stream);
+        return producer ? dispatch_pipe<__bf16, kProducer>(p, bm, bn, eight, ring, two, grid, stream)
+                        : dispatch_pipe<__bf16, kConsumer>(p, bm, bn, eight, ring, two, grid, stream);
     }
-    if (mode == kRemote) return dispatch_pipe<_Float16, kRemote>(p, bm, bn, eight, false, grid, stream);
-    return producer ? dispatch_pipe<_Float16, kProducer>(p, bm, bn, eight, ring, grid, stream)
-                    : dispatch_pipe<_Float16, kConsumer>(p, bm, bn, eight, ring, grid, stream);
+    if (mode == kRemote) return dispatch_pipe<_Float16, kRemote>(p, bm, bn, eight, false, false, grid, stream);
+    return producer ? dispatch_pipe<_Float16, kProducer>(p, bm, bn, eight, ring, two, grid, stream)
+                    : dispatch_pipe<_Float16, kConsumer>(p, bm, bn, eight, ring, two, grid, stream);
 }
 
 }  // namespace syn
@@ -864,6 +1095,16 @@ int syn_gemm_producer(const syn_gemm_desc* desc, syn_stream_t stream) {
 int syn_gemm_remote_binding(const syn_gemm_desc* desc, const syn_gemm_remote* remote, syn_stream_t stream) {
     return syn::gemm_entry(desc, reinterpret_cast<hipStream_t>(stream), syn::kRemote, remote);
 }
+
+#ifdef SYN_EXP_TIMING
+int syn_exp_timing(void* host_dst, int reset) {
+    if (reset) {
+        static long long zeros[256 * 8][8];
+        return (int)hipMemcpyToSymbol(HIP_SYMBOL(syn::g_timing), zeros, sizeof(zeros));
+    }
+    return (int)hipMemcpyFromSymbol(host_dst, HIP_SYMBOL(syn::g_timing), sizeof(long long) * 256 * 8 * 8);
+}
+#endif
 
 int syn_gemm_grid(int64_t cum_tiles, int32_t M, int32_t N, int32_t block_m, int32_t block_n,
                   int32_t num_sms) {
