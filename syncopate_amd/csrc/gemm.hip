@@ -257,6 +257,7 @@ struct SlabPipe {
     static constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
     static constexpr int BK = 64, ROW = BK * 2;
     static constexpr int A_BYTES = BM * ROW, STAGE = (BM + BN) * ROW;
+    static constexpr int LDS_BYTES = NST * STAGE;
     static constexpr int FILLS = (BM + BN) / (8 * NW);
     static constexpr int K_ALIGN = 64;
     typedef typename Mfma32<T>::frag_t frag_t;
@@ -497,7 +498,14 @@ struct EarlyPipe : SlabPipe<T, BM, BN, WGM, WGN, 2> {
     static __device__ __forceinline__ void slab(f32x16_t (&acc)[TM][TN], frag_t (&fa)[4][TM], frag_t (&fb)[4][TN],
                                                 unsigned char* cur, const unsigned char* nxt,
                                                 const unsigned char* a_slab, const unsigned char* b_slab,
-                                                size_t k_refill, const Lane& ln, int wave) {
+                                                size_t k_refill, const Lane& ln, int wave
+#ifdef SYN_EXP_TIMING
+                                                , long long (&tt)[6]
+#endif
+                                                ) {
+#ifdef SYN_EXP_TIMING
+        const long long q0 = SYN_T();
+#endif
         const unsigned char* a_k = a_slab + k_refill;
         const unsigned char* b_k = b_slab + k_refill;
         unsigned char* const dst = cur + wave * 1024;
@@ -507,8 +515,17 @@ struct EarlyPipe : SlabPipe<T, BM, BN, WGM, WGN, 2> {
         mma_step<T, TM, TN>(acc, fa[0], fb[0]);
         hint_front<0, TM * TN, 2 * (TM + TN), 0>();
         __builtin_amdgcn_sched_barrier(0);
+#ifdef SYN_EXP_TIMING
+        const long long q1 = SYN_T();
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, true));
+        const long long q2 = SYN_T();
+        __builtin_amdgcn_s_barrier();
+        const long long q3 = SYN_T();
+        tt[0] += q1 - q0; tt[1] += q2 - q1; tt[2] += q3 - q2;
+#else
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, true));     // own reads of this stage returned
         __builtin_amdgcn_s_barrier();                          // everyone's: the stage is free
+#endif
         __builtin_amdgcn_sched_barrier(0);
 
         dma_blocks<0, PA, BM, NW, NV>(dst, a_k, b_k, ln.voff);
@@ -521,8 +538,17 @@ struct EarlyPipe : SlabPipe<T, BM, BN, WGM, WGN, 2> {
         spread_hint<0, TM * TN, PB>();
         __builtin_amdgcn_sched_barrier(0);
         // own fills of slab s+1 landed (the two thirds of slab s+2 issued since may fly on)
+#ifdef SYN_EXP_TIMING
+        const long long q4 = SYN_T();
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(PA + PB, false));
+        const long long q5 = SYN_T();
+        __builtin_amdgcn_s_barrier();
+        const long long q6 = SYN_T();
+        tt[3] += q4 - q3; tt[4] += q5 - q4; tt[5] += q6 - q5;
+#else
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(PA + PB, false));
         __builtin_amdgcn_s_barrier();
+#endif
         __builtin_amdgcn_sched_barrier(0);
 
         dma_blocks<PA + PB, FILLS, BM, NW, NV>(dst, a_k, b_k, ln.voff);
@@ -550,12 +576,26 @@ struct EarlyPipe : SlabPipe<T, BM, BN, WGM, WGN, 2> {
         read_step<1>(fa[1], fb[1], stage0, ln);
 
         const int pairs = k_steps >> 1;
+#ifdef SYN_EXP_TIMING
+        long long tt[6] = {0, 0, 0, 0, 0, 0};
+        const long long tk0 = SYN_T();
+#define SYN_TT , tt
+#else
+#define SYN_TT
+#endif
         for (int pr = 0; pr < pairs; ++pr) {
-            slab(acc, fa, fb, stage0, stage1, a_slab, b_slab, Base::slab_off(2 * pr + 2, rot, k_steps), ln, wave);
-            slab(acc, fa, fb, stage1, stage0, a_slab, b_slab, Base::slab_off(2 * pr + 3, rot, k_steps), ln, wave);
+            slab(acc, fa, fb, stage0, stage1, a_slab, b_slab, Base::slab_off(2 * pr + 2, rot, k_steps), ln, wave SYN_TT);
+            slab(acc, fa, fb, stage1, stage0, a_slab, b_slab, Base::slab_off(2 * pr + 3, rot, k_steps), ln, wave SYN_TT);
         }
         if (k_steps & 1)
-            slab(acc, fa, fb, stage0, stage1, a_slab, b_slab, Base::slab_off(k_steps + 1, rot, k_steps), ln, wave);
+            slab(acc, fa, fb, stage0, stage1, a_slab, b_slab, Base::slab_off(k_steps + 1, rot, k_steps), ln, wave SYN_TT);
+#ifdef SYN_EXP_TIMING
+        if (lane == 0) {
+            long long* g = g_timing[(blockIdx.x % 256) * 8 + wave];
+            g[0] += tt[1] + tt[4]; g[1] += tt[2] + tt[5]; g[2] += SYN_T() - tk0; g[3] += 1;
+            g[4] += tt[0]; g[5] += tt[3]; g[6] += tt[1]; g[7] += tt[2];
+        }
+#endif
         // drain the re-fetches of the last slab before anything refills the stages
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, true));
         __builtin_amdgcn_s_barrier();
@@ -564,7 +604,9 @@ struct EarlyPipe : SlabPipe<T, BM, BN, WGM, WGN, 2> {
 };
 
 // the deepest arrangement that fits next to the wave table: three stages, or the early-read form
-template <typename T, int BM, int BN, int WGM, int WGN, bool THREE = (3 * (BM + BN) * 128 <= 150 * 1024)>
+// (the kernel's own LDS: up to 4 KB of wave table, 32 rows x 80 bytes of C staging per wavefront)
+template <typename T, int BM, int BN, int WGM, int WGN,
+          bool THREE = (3 * (BM + BN) * 128 + WGM * WGN * 32 * 80 + 4096 <= 160 * 1024)>
 struct DeepPipeSel {
     typedef SlabPipe<T, BM, BN, WGM, WGN, 3> type;
 };
@@ -591,6 +633,7 @@ struct RingPipe {
     static constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
     static constexpr int BK = 32, ROW = BK * 2;
     static constexpr int A_BYTES = BM * ROW, STAGE = (BM + BN) * ROW;
+    static constexpr int LDS_BYTES = 4 * STAGE;
     static constexpr int FILLS = (BM + BN) / (16 * NW);     // fills per wavefront and slab
     static constexpr int K_ALIGN = 128;
     typedef typename Mfma32<T>::frag_t frag_t;
@@ -723,6 +766,13 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
     constexpr int TM = WM / 32, TN = WN / 32;     // 32x32 MFMA tiles per wavefront
 
     __shared__ int s_abort;
+    // C staging of the epilogue: 32 rows x CS_COLS columns per wavefront, 64 columns where LDS allows
+    constexpr int NWAVES = WGM * WGN;
+    constexpr int CS_COLS = (!REMOTE && Pipe::LDS_BYTES + NWAVES * 32 * (64 * 2 + 16) + 4096 <= 160 * 1024) ? 64 : 32;
+    __shared__ __attribute__((aligned(16))) unsigned char s_cstage[REMOTE ? 16 : NWAVES * 32 * (CS_COLS * 2 + 16)];
+#ifdef SYN_EXP_TIMING
+    const long long t_kernel0 = SYN_T();
+#endif
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -889,7 +939,13 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
 #pragma unroll
                 for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
+#ifdef SYN_EXP_TIMING
+        if (tid == 0 && it < 2) g_timing[(blockIdx.x % 256) * 8 + 7][it * 3 + 0] = SYN_T() - t_kernel0;
+#endif
         Pipe::main(acc, panel_a(tile), panel_b(tile), row_bytes, K, tile.k_rot, lane, wave);
+#ifdef SYN_EXP_TIMING
+        if (tid == 0 && it < 2) g_timing[(blockIdx.x % 256) * 8 + 7][it * 3 + 1] = SYN_T() - t_kernel0;
+#endif
 
         // The stages are free: start the next tile's fills before this tile's C is stored, unless
         // the next tile opens a wave whose flag is still to be waited for (nothing of a chunk may
@@ -908,9 +964,9 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
         }
 
         // Epilogue.  With B as the first MFMA operand a lane holds, for column m = lane % 32 of
-        // D', rows n = 8g + 4*(lane/32) + 0..3: four consecutive elements of one row of C -> one
-        // 8-byte store.
-        {
+        // D', rows n = 8g + 4*(lane/32) + 0..3: four consecutive elements of one row of C.
+        if constexpr (REMOTE) {
+            // peer buffers are only 8-byte aligned: one 8-byte store (or two packed atomics) per group
             T* c_row = tile.c_tile + (size_t)(wm * WM + (lane & 31)) * tile.ldc + wn * WN + 4 * (lane >> 5);
 #pragma unroll
             for (int i = 0; i < TM; ++i)
@@ -921,17 +977,53 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
                         const uint2 v = pack4<T>(acc[i][j][4 * g], acc[i][j][4 * g + 1],
                                                  acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
                         T* dst = c_row + (size_t)(32 * i) * tile.ldc + 32 * j + 8 * g;
-                        if (REMOTE && p.c_atomic) {
+                        if (p.c_atomic) {
                             atomic_add4<T>(dst, v);
-                        } else if (PRODUCER) {
-                            // written through the XCD's L2: the release below then has nothing
-                            // of this tile left to write back
-                            __hip_atomic_store(reinterpret_cast<uint64_t*>(dst), __builtin_bit_cast(uint64_t, v),
-                                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                         } else {
                             *reinterpret_cast<uint2*>(dst) = v;
                         }
                     }
+        } else {
+            // A store instruction of those groups would touch 32 rows with 16 bytes each, and the
+            // texture path takes a cycle per cache line touched.  So a strip of 32 rows x CS_COLS
+            // columns goes through a private piece of LDS (rows padded by 16 bytes) and leaves as
+            // 16 bytes per lane, whole rows of the strip side by side: 8 or 16 lines per instruction.
+            constexpr int CS_ROW = CS_COLS * 2 + 16;          // bytes per staged row
+            constexpr int LPR = CS_COLS / 8;                  // lanes per row on the way out
+            constexpr int RPI = 64 / LPR;                     // rows per store instruction
+            unsigned char* const cs = s_cstage + wave * (32 * CS_ROW);
+            unsigned char* const cs_wr = cs + (lane & 31) * CS_ROW + 8 * (lane >> 5);
+            const unsigned char* const cs_rd = cs + (lane / LPR) * CS_ROW + (lane % LPR) * 16;
+            T* const c_out = tile.c_tile + (size_t)(wm * WM + lane / LPR) * tile.ldc + wn * WN + (lane % LPR) * 8;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int js = 0; js < TN; js += CS_COLS / 32) {
+#pragma unroll
+                    for (int jj = 0; jj < CS_COLS / 32; ++jj)
+#pragma unroll
+                        for (int g = 0; g < 4; ++g)
+                            *reinterpret_cast<uint2*>(cs_wr + jj * 64 + g * 16) =
+                                pack4<T>(acc[i][js + jj][4 * g], acc[i][js + jj][4 * g + 1],
+                                         acc[i][js + jj][4 * g + 2], acc[i][js + jj][4 * g + 3]);
+#pragma unroll
+                    for (int t = 0; t < 32 / RPI; ++t) {
+                        const uint4 v = *reinterpret_cast<const uint4*>(cs_rd + t * RPI * CS_ROW);
+                        T* dst = c_out + (size_t)(32 * i + t * RPI) * tile.ldc + 32 * js;
+                        if (PRODUCER) {
+                            // written through the XCD's L2: the release below then has nothing
+                            // of this tile left to write back
+                            __hip_atomic_store(reinterpret_cast<uint64_t*>(dst),
+                                               (uint64_t)v.x | ((uint64_t)v.y << 32), __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_AGENT);
+                            __hip_atomic_store(reinterpret_cast<uint64_t*>(dst) + 1,
+                                               (uint64_t)v.z | ((uint64_t)v.w << 32), __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_AGENT);
+                        } else {
+                            *reinterpret_cast<uint4*>(dst) = v;
+                        }
+                    }
+                }
         }
 
         if (PRODUCER) {
@@ -957,6 +1049,10 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
             Pipe::prologue(panel_a(next), panel_b(next), row_bytes, K, next.k_rot, lane, wave);
         }
         tile = next;
+#ifdef SYN_EXP_TIMING
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, true));
+        if (tid == 0 && it < 2) g_timing[(blockIdx.x % 256) * 8 + 7][it * 3 + 2] = SYN_T() - t_kernel0;
+#endif
     }
 }
 
