@@ -44,7 +44,7 @@ def _events(n):
     return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
 
 
-def build_ag_gemm(device):
+def build_ag_gemm(device, copy_blocks=0):
     from syncopate_amd.communication.code_gen import CommGenerator
     from syncopate_amd.communication.comm_runtime.communication_context import CommContext
     from syncopate_amd.communication.common_descriptors import build_all_gather_plan_1d_swizzle
@@ -65,7 +65,7 @@ def build_ag_gemm(device):
     torch.manual_seed(0)
     a = (0.02 * torch.randn(M, K, device=device)).bfloat16()
     b = (0.02 * torch.randn(N, K, device=device)).bfloat16()
-    ctx = CommContext(RANK, info, device=device)
+    ctx = CommContext(RANK, info, device=device, copy_blocks=copy_blocks)
     rows = M // WORLD
     for r in range(WORLD):     # every rank's symmetric buffer holds its own shard
         ctx.comm_buffers["a"][r][r * rows:(r + 1) * rows].copy_(a[r * rows:(r + 1) * rows])
@@ -323,6 +323,9 @@ def main():
     ap.add_argument("--resident-only", action="store_true",
                     help="skip the flag-gated steps (for hardware-counter runs, which serialise kernels: "
                          "a gated consumer would wait for copies that can only start after it)")
+    ap.add_argument("--copy-blocks", type=int, default=0,
+                    help="0: the producer's chunk copies are hipMemcpyAsync (default); N > 0: the library's "
+                         "streaming copy kernel with N workgroups")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one rank's share on ONE GPU: the other ranks of the mesh are "
@@ -335,7 +338,7 @@ def main():
     device = torch.device("cuda", 0)
     torch.cuda.set_device(device)
 
-    state = build_ag_gemm(device)
+    state = build_ag_gemm(device, args.copy_blocks)
     wall_ms, gated_ms, resident_ms = run_ag_gemm(state, args.steps, args.warmup, args.resident_only,
                                                  not args.no_graph)
     traffic_calibration(device)
@@ -367,7 +370,9 @@ def main():
                         "fp32 accumulate",
             "tile": [BM, BN, BK],
             "programs": NUM_SMS,
-            "producer": "side stream: hipMemcpyAsync + flag-set kernel per chunk",
+            "producer": "side stream: " + ("hipMemcpyAsync" if args.copy_blocks == 0 else
+                                           f"copy kernel of {args.copy_blocks} workgroups")
+                        + " + flag-set kernel per chunk",
             "launch": "eager" if args.no_graph else "hip graph replay of the whole step",
         },
         "pct_bf16_mfma_peak": 100.0 * value / MFMA_BF16_PEAK_TFLOPS,

@@ -207,12 +207,6 @@ __device__ __forceinline__ void dma_part(unsigned char* stage, const unsigned ch
     }
 }
 
-#ifdef SYN_EXP_TIMING
-__device__ long long g_timing[256 * 8][8];
-struct TimingAcc { long long wait = 0, bar = 0, fillissue = 0; };
-__device__ TimingAcc* g_tacc_dummy;
-#define SYN_T() __builtin_amdgcn_s_memtime()
-#endif
 
 // The same for the slab pipelines, shaped so that a fill costs two instructions (M0, load): the
 // wavefront's fill j is 1 KB block j * NW + wave of the stage; blocks of A come first and BM / 8
@@ -297,14 +291,8 @@ struct SlabPipe {
                                                 const unsigned char* a_slab, const unsigned char* b_slab,
                                                 size_t k_refill, size_t k_prev, const Lane& ln, size_t row_bytes,
                                                 int wave
-#ifdef SYN_EXP_TIMING
-                                                , long long& tw, long long& tb, long long& t012, long long& t3
-#endif
                                                 ) {
         frag_t fa1[TM], fb1[TN];
-#ifdef SYN_EXP_TIMING
-        const long long ts = SYN_T();
-#endif
         if constexpr (SPREAD) fill_part<1>(prv, a_slab, b_slab, k_prev, ln, row_bytes, wave);
         load_frags<T, TM, TN, ROW>(fa1, fb1, cur, ln.a_rd, ln.b_rd, ((2 + ln.half) ^ ln.swz) << 4);
         mma_step<T, TM, TN>(acc, fa0, fb0);
@@ -324,17 +312,8 @@ struct SlabPipe {
         __builtin_amdgcn_sched_barrier(0);
 
         // own fills of slab s+1 landed (those of slab s+2, all younger, may fly on)
-#ifdef SYN_EXP_TIMING
-        const long long t0 = SYN_T();
-        __builtin_amdgcn_s_waitcnt(waitcnt_imm((NST - 2) * FILLS, true));
-        const long long t1 = SYN_T();
-        __builtin_amdgcn_s_barrier();
-        const long long t2 = SYN_T();
-        tw += t1 - t0; tb += t2 - t1; t012 += t0 - ts;
-#else
         __builtin_amdgcn_s_waitcnt(waitcnt_imm((NST - 2) * FILLS, true));
         __builtin_amdgcn_s_barrier();
-#endif
         __builtin_amdgcn_sched_barrier(0);
 
         fill_part<0>(cur, a_slab, b_slab, k_refill, ln, row_bytes, wave);
@@ -342,9 +321,6 @@ struct SlabPipe {
         mma_step<T, TM, TN>(acc, fa1, fb1);
         spread_hint<TM + TN, TM * TN, part_size<0>()>();
         __builtin_amdgcn_sched_barrier(0);
-#ifdef SYN_EXP_TIMING
-        t3 += SYN_T() - t2;
-#endif
     }
 
     // the stages are distinct objects: LDS reads of one never wait for fills of the other
@@ -405,19 +381,10 @@ struct SlabPipe {
         frag_t fa0[TM], fb0[TN];
         load_frags<T, TM, TN, ROW>(fa0, fb0, stage0, ln.a_rd, ln.b_rd, ((0 + ln.half) ^ ln.swz) << 4);
 
-#ifdef SYN_EXP_TIMING
-        long long tw = 0, tb = 0, t012 = 0, t3 = 0;
-        const long long tk0 = SYN_T();
-        auto run = [&](unsigned char* cur, const unsigned char* nxt, unsigned char* prv, int s) {
-            slab(acc, fa0, fb0, cur, nxt, prv, a_slab, b_slab, slab_off(s + NST, rot, k_steps),
-                 slab_off(s + 2, rot, k_steps), ln, row_bytes, wave, tw, tb, t012, t3);
-        };
-#else
         auto run = [&](unsigned char* cur, const unsigned char* nxt, unsigned char* prv, int s) {
             slab(acc, fa0, fb0, cur, nxt, prv, a_slab, b_slab, slab_off(s + NST, rot, k_steps),
                  slab_off(s + 2, rot, k_steps), ln, row_bytes, wave);
         };
-#endif
         if constexpr (NST == 2) {
             const int pairs = k_steps >> 1;
             for (int pr = 0; pr < pairs; ++pr) {
@@ -436,12 +403,6 @@ struct SlabPipe {
             if (rest >= 1) run(stage0, stage1, stage2, 3 * triples);
             if (rest == 2) run(stage1, stage2, stage0, 3 * triples + 1);
         }
-#ifdef SYN_EXP_TIMING
-        if (lane == 0) {
-            long long* g = g_timing[(blockIdx.x % 256) * 8 + wave];
-            g[0] += tw; g[1] += tb; g[2] += SYN_T() - tk0; g[3] += 1; g[4] += t012; g[5] += t3;
-        }
-#endif
         // drain the re-fetches of the last slab before anything refills the stages
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, true));
         __builtin_amdgcn_s_barrier();
@@ -495,17 +456,12 @@ struct EarlyPipe : SlabPipe<T, BM, BN, WGM, WGN, 2> {
         }
     }
 
+
     static __device__ __forceinline__ void slab(f32x16_t (&acc)[TM][TN], frag_t (&fa)[4][TM], frag_t (&fb)[4][TN],
                                                 unsigned char* cur, const unsigned char* nxt,
                                                 const unsigned char* a_slab, const unsigned char* b_slab,
                                                 size_t k_refill, const Lane& ln, int wave
-#ifdef SYN_EXP_TIMING
-                                                , long long (&tt)[6]
-#endif
                                                 ) {
-#ifdef SYN_EXP_TIMING
-        const long long q0 = SYN_T();
-#endif
         const unsigned char* a_k = a_slab + k_refill;
         const unsigned char* b_k = b_slab + k_refill;
         unsigned char* const dst = cur + wave * 1024;
@@ -515,17 +471,8 @@ struct EarlyPipe : SlabPipe<T, BM, BN, WGM, WGN, 2> {
         mma_step<T, TM, TN>(acc, fa[0], fb[0]);
         hint_front<0, TM * TN, 2 * (TM + TN), 0>();
         __builtin_amdgcn_sched_barrier(0);
-#ifdef SYN_EXP_TIMING
-        const long long q1 = SYN_T();
-        __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, true));
-        const long long q2 = SYN_T();
-        __builtin_amdgcn_s_barrier();
-        const long long q3 = SYN_T();
-        tt[0] += q1 - q0; tt[1] += q2 - q1; tt[2] += q3 - q2;
-#else
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, true));     // own reads of this stage returned
         __builtin_amdgcn_s_barrier();                          // everyone's: the stage is free
-#endif
         __builtin_amdgcn_sched_barrier(0);
 
         dma_blocks<0, PA, BM, NW, NV>(dst, a_k, b_k, ln.voff);
@@ -538,17 +485,8 @@ struct EarlyPipe : SlabPipe<T, BM, BN, WGM, WGN, 2> {
         spread_hint<0, TM * TN, PB>();
         __builtin_amdgcn_sched_barrier(0);
         // own fills of slab s+1 landed (the two thirds of slab s+2 issued since may fly on)
-#ifdef SYN_EXP_TIMING
-        const long long q4 = SYN_T();
-        __builtin_amdgcn_s_waitcnt(waitcnt_imm(PA + PB, false));
-        const long long q5 = SYN_T();
-        __builtin_amdgcn_s_barrier();
-        const long long q6 = SYN_T();
-        tt[3] += q4 - q3; tt[4] += q5 - q4; tt[5] += q6 - q5;
-#else
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(PA + PB, false));
         __builtin_amdgcn_s_barrier();
-#endif
         __builtin_amdgcn_sched_barrier(0);
 
         dma_blocks<PA + PB, FILLS, BM, NW, NV>(dst, a_k, b_k, ln.voff);
@@ -576,26 +514,12 @@ struct EarlyPipe : SlabPipe<T, BM, BN, WGM, WGN, 2> {
         read_step<1>(fa[1], fb[1], stage0, ln);
 
         const int pairs = k_steps >> 1;
-#ifdef SYN_EXP_TIMING
-        long long tt[6] = {0, 0, 0, 0, 0, 0};
-        const long long tk0 = SYN_T();
-#define SYN_TT , tt
-#else
-#define SYN_TT
-#endif
         for (int pr = 0; pr < pairs; ++pr) {
-            slab(acc, fa, fb, stage0, stage1, a_slab, b_slab, Base::slab_off(2 * pr + 2, rot, k_steps), ln, wave SYN_TT);
-            slab(acc, fa, fb, stage1, stage0, a_slab, b_slab, Base::slab_off(2 * pr + 3, rot, k_steps), ln, wave SYN_TT);
+            slab(acc, fa, fb, stage0, stage1, a_slab, b_slab, Base::slab_off(2 * pr + 2, rot, k_steps), ln, wave);
+            slab(acc, fa, fb, stage1, stage0, a_slab, b_slab, Base::slab_off(2 * pr + 3, rot, k_steps), ln, wave);
         }
         if (k_steps & 1)
-            slab(acc, fa, fb, stage0, stage1, a_slab, b_slab, Base::slab_off(k_steps + 1, rot, k_steps), ln, wave SYN_TT);
-#ifdef SYN_EXP_TIMING
-        if (lane == 0) {
-            long long* g = g_timing[(blockIdx.x % 256) * 8 + wave];
-            g[0] += tt[1] + tt[4]; g[1] += tt[2] + tt[5]; g[2] += SYN_T() - tk0; g[3] += 1;
-            g[4] += tt[0]; g[5] += tt[3]; g[6] += tt[1]; g[7] += tt[2];
-        }
-#endif
+            slab(acc, fa, fb, stage0, stage1, a_slab, b_slab, Base::slab_off(k_steps + 1, rot, k_steps), ln, wave);
         // drain the re-fetches of the last slab before anything refills the stages
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, true));
         __builtin_amdgcn_s_barrier();
@@ -770,9 +694,6 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
     constexpr int NWAVES = WGM * WGN;
     constexpr int CS_COLS = (!REMOTE && Pipe::LDS_BYTES + NWAVES * 32 * (64 * 2 + 16) + 4096 <= 160 * 1024) ? 64 : 32;
     __shared__ __attribute__((aligned(16))) unsigned char s_cstage[REMOTE ? 16 : NWAVES * 32 * (CS_COLS * 2 + 16)];
-#ifdef SYN_EXP_TIMING
-    const long long t_kernel0 = SYN_T();
-#endif
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -939,13 +860,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
 #pragma unroll
                 for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-#ifdef SYN_EXP_TIMING
-        if (tid == 0 && it < 2) g_timing[(blockIdx.x % 256) * 8 + 7][it * 3 + 0] = SYN_T() - t_kernel0;
-#endif
         Pipe::main(acc, panel_a(tile), panel_b(tile), row_bytes, K, tile.k_rot, lane, wave);
-#ifdef SYN_EXP_TIMING
-        if (tid == 0 && it < 2) g_timing[(blockIdx.x % 256) * 8 + 7][it * 3 + 1] = SYN_T() - t_kernel0;
-#endif
 
         // The stages are free: start the next tile's fills before this tile's C is stored, unless
         // the next tile opens a wave whose flag is still to be waited for (nothing of a chunk may
@@ -1049,10 +964,6 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
             Pipe::prologue(panel_a(next), panel_b(next), row_bytes, K, next.k_rot, lane, wave);
         }
         tile = next;
-#ifdef SYN_EXP_TIMING
-        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, true));
-        if (tid == 0 && it < 2) g_timing[(blockIdx.x % 256) * 8 + 7][it * 3 + 2] = SYN_T() - t_kernel0;
-#endif
     }
 }
 
@@ -1192,15 +1103,6 @@ int syn_gemm_remote_binding(const syn_gemm_desc* desc, const syn_gemm_remote* re
     return syn::gemm_entry(desc, reinterpret_cast<hipStream_t>(stream), syn::kRemote, remote);
 }
 
-#ifdef SYN_EXP_TIMING
-int syn_exp_timing(void* host_dst, int reset) {
-    if (reset) {
-        static long long zeros[256 * 8][8];
-        return (int)hipMemcpyToSymbol(HIP_SYMBOL(syn::g_timing), zeros, sizeof(zeros));
-    }
-    return (int)hipMemcpyFromSymbol(host_dst, HIP_SYMBOL(syn::g_timing), sizeof(long long) * 256 * 8 * 8);
-}
-#endif
 
 int syn_gemm_grid(int64_t cum_tiles, int32_t M, int32_t N, int32_t block_m, int32_t block_n,
                   int32_t num_sms) {
