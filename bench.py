@@ -65,7 +65,8 @@ def build_ag_gemm(device, copy_blocks=0):
     torch.manual_seed(0)
     a = (0.02 * torch.randn(M, K, device=device)).bfloat16()
     b = (0.02 * torch.randn(N, K, device=device)).bfloat16()
-    ctx = CommContext(RANK, info, device=device, copy_blocks=copy_blocks)
+    # two flag sets: the reset of one iteration's flags happens behind the next one's copies
+    ctx = CommContext(RANK, info, device=device, copy_blocks=copy_blocks, flag_sets=2)
     rows = M // WORLD
     for r in range(WORLD):     # every rank's symmetric buffer holds its own shard
         ctx.comm_buffers["a"][r][r * rows:(r + 1) * rows].copy_(a[r * rows:(r + 1) * rows])
@@ -85,9 +86,7 @@ def run_ag_gemm(state, steps, warmup, resident_only=False, use_graph=True):
 
     ctx, b, c, tables = state["ctx"], state["b"], state["c"], state["tables"]
     symm = ctx.comm_buffers["a"][RANK]
-    flags = ctx.recv_signal_bufs[RANK]
     stream = torch.cuda.current_stream()
-    rows = M // WORLD
 
     def consumer(flag_words):
         gemm(symm, b, c, WORLD, NUM_SMS, BM, BN, BK, GROUP_M, signal_ptr=flag_words, xcd_remap=False,
@@ -95,36 +94,49 @@ def run_ag_gemm(state, steps, warmup, resident_only=False, use_graph=True):
 
     def fused_step():
         cur = torch.cuda.current_stream()
-        ctx.reset_signals()
+        ctx.reset_signals()               # switches to the zeroed flag set
         ctx.start_after(cur)
         ctx.execute()
-        consumer(flags)
+        consumer(ctx.recv_signal_bufs[RANK])
         ctx.end_before(cur)
 
-    # One step is ~25 launches (flag reset, 7 copies, 7 flag writes, stream joins, the GEMM):
-    # replayed as a HIP graph so that the host's launch rate is not what gets measured.  The graph
-    # holds kernels and memcpy nodes only.
-    step = fused_step
-    if use_graph:
-        fused_step()
-        torch.cuda.synchronize()
+    # One step is ~25 launches (7 copies, 7 flag writes, flag reset, stream joins, the GEMM):
+    # replayed as HIP graphs so that the host's launch rate is not what gets measured (kernels
+    # and memcpy nodes only).  A graph holds an even number of steps, since consecutive steps
+    # use alternate flag sets: two for the warm-up, all timed steps in one; an odd step count
+    # ends with one step launched from the host.
+    def capture(n):
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            fused_step()
-        step = graph.replay
+            for _ in range(n):
+                fused_step()
+        return graph
+
+    fused_step()
+    fused_step()
+    torch.cuda.synchronize()
+    timed_in_graph = steps - steps % 2
+    warm_graph = capture(2) if use_graph else None
+    timed_graph = capture(timed_in_graph) if use_graph and timed_in_graph else None
 
     # ---- gated run: the step the metric is quoted on ----
     wall_ms = gated_kernel_ms = None
-    if resident_only:
-        fused_step()                      # once, so that the gathered buffer is complete
-        torch.cuda.synchronize()
-    else:
-        for _ in range(warmup):
-            step()
+    if not resident_only:
+        for _ in range((warmup + 1) // 2):
+            if use_graph:
+                warm_graph.replay()
+            else:
+                fused_step()
+                fused_step()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(steps):            # EXACTLY `steps` fused steps, nothing else on the streams
-            step()
+        if timed_graph is not None:          # EXACTLY `steps` fused steps, nothing else on the streams
+            timed_graph.replay()
+            if steps % 2:
+                fused_step()
+        else:
+            for _ in range(steps):
+                fused_step()
         torch.cuda.synchronize()
         wall_ms = (time.perf_counter() - t0) * 1e3 / steps
         # the same steps once more with HIP events around the consumer launch (event markers
@@ -135,7 +147,7 @@ def run_ag_gemm(state, steps, warmup, resident_only=False, use_graph=True):
             ctx.start_after(stream)
             ctx.execute()
             begin[i].record(stream)
-            consumer(flags)
+            consumer(ctx.recv_signal_bufs[RANK])
             end[i].record(stream)
             ctx.end_before(stream)
         torch.cuda.synchronize()
@@ -144,7 +156,7 @@ def run_ag_gemm(state, steps, warmup, resident_only=False, use_graph=True):
     ctx.check_status()
 
     # ---- same kernel, every chunk resident and every flag already set ----
-    resident_flags = torch.ones_like(flags)
+    resident_flags = torch.ones_like(ctx.recv_signal_bufs[RANK])
     for _ in range(warmup):
         consumer(resident_flags)
     torch.cuda.synchronize()
@@ -373,7 +385,7 @@ def main():
             "producer": "side stream: " + ("hipMemcpyAsync" if args.copy_blocks == 0 else
                                            f"copy kernel of {args.copy_blocks} workgroups")
                         + " + flag-set kernel per chunk",
-            "launch": "eager" if args.no_graph else "hip graph replay of the whole step",
+            "launch": "eager" if args.no_graph else "one hip graph replay of all timed steps",
         },
         "pct_bf16_mfma_peak": 100.0 * value / MFMA_BF16_PEAK_TFLOPS,
         "flag_wait_overhead_pct": 100.0 * (gated_ms - resident_ms) / resident_ms,

@@ -52,7 +52,7 @@ class CommContext:
 
     def __init__(self, rank: int, info: CommInfo, multi_info: bool = False, *,
                  device: Optional[torch.device] = None, link_delay_us: int = 0,
-                 wait_timeout_us: int = 2_000_000, copy_blocks: int = 0) -> None:
+                 wait_timeout_us: int = 2_000_000, copy_blocks: int = 0, flag_sets: int = 1) -> None:
         if info.local_world_size <= 0:
             info.local_world_size = info.world_size
         if info.local_world_size != info.world_size:
@@ -78,9 +78,22 @@ class CommContext:
                 return []
             return [torch.zeros((count,), dtype=SIGNAL_DTYPE, device=self.device) for _ in range(world)]
 
-        self.recv_signal_bufs = flag_arrays(info.recv_signal_num)
-        self.transit_signal_bufs = flag_arrays(info.transit_signal_num)
-        self.compute_signal_bufs = flag_arrays(info.compute_signal_num)
+        # One set of flag arrays is the reference's arrangement: reset_signals() zeroes it in front
+        # of every iteration, and the compute kernel can only be launched behind that fill.  With
+        # two sets reset_signals() switches to the other (already zero) set and the one just left
+        # is zeroed at the tail of the next execute(), off the compute stream's path: iterations
+        # then follow each other without a fill between the kernels.
+        if flag_sets not in (1, 2):
+            raise ValueError("flag_sets must be 1 or 2")
+        self._flag_sets = [
+            (flag_arrays(info.recv_signal_num), flag_arrays(info.transit_signal_num),
+             flag_arrays(info.compute_signal_num))
+            for _ in range(flag_sets)
+        ]
+        self._cur_set = 0
+        self._stale_set: Optional[int] = None
+        self._stale_whole_mesh = False
+        self.recv_signal_bufs, self.transit_signal_bufs, self.compute_signal_bufs = self._flag_sets[0]
         self.comm_buffers = {
             name: [torch.zeros(tuple(shape), dtype=dtype, device=self.device) for _ in range(world)]
             for name, (shape, dtype) in info.comm_buffer_sizes.items()
@@ -91,12 +104,35 @@ class CommContext:
 
     # ---- flags and stream ordering -------------------------------------------
 
-    def reset_signals(self, whole_mesh: bool = False) -> None:
-        """Zero this rank's flag words (every simulated rank's with `whole_mesh`)."""
-        for group in (self.recv_signal_bufs, self.transit_signal_bufs, self.compute_signal_bufs):
+    def _zero_set(self, index: int, whole_mesh: bool) -> None:
+        for group in self._flag_sets[index]:
             if group:
                 for r in (range(len(group)) if whole_mesh else (self.local_rank,)):
                     group[r].fill_(0)
+
+    def reset_signals(self, whole_mesh: bool = False) -> None:
+        """Zero this rank's flag words (every simulated rank's with `whole_mesh`).
+
+        With two flag sets: make the other set current (`recv_signal_bufs` etc. then name ITS
+        arrays - pass them to the kernels after this call) and leave the old one to be zeroed at
+        the end of the next execute().  That is only safe in the reference's call order,
+        reset_signals -> start_after(compute stream) -> execute -> kernels -> end_before: the
+        communication streams then start after the previous iteration's kernels, the last readers
+        of the old set."""
+        if len(self._flag_sets) == 1:
+            self._zero_set(0, whole_mesh)
+            return
+        self._stale_set = self._cur_set
+        self._stale_whole_mesh = whole_mesh
+        self._cur_set = 1 - self._cur_set
+        self.recv_signal_bufs, self.transit_signal_bufs, self.compute_signal_bufs = self._flag_sets[self._cur_set]
+
+    def _zero_stale_set(self) -> None:
+        if self._stale_set is None or not self.streams:
+            return
+        with torch.cuda.stream(self.streams[-1]):
+            self._zero_set(self._stale_set, self._stale_whole_mesh)
+        self._stale_set = None
 
     def start_after(self, stream: Optional[torch.cuda.Stream] = None) -> None:
         """Communication streams start once `stream` has reached this point."""
@@ -125,6 +161,7 @@ class CommContext:
             handle = int(stream.cuda_stream)
             for op in ops:
                 self._issue(op, self.rank, stream, handle, neglect_local)
+        self._zero_stale_set()
 
     def execute_mesh(self, neglect_local: bool = False) -> None:
         """Enqueue EVERY rank's ops on this rank's first communication stream, in an order that
@@ -162,6 +199,7 @@ class CommContext:
                     progressed = True
             if not progressed:
                 raise RuntimeError("the op lists wait for flags nobody writes: the plan cannot be replayed")
+        self._zero_stale_set()
 
     def _issue(self, op, owner: int, stream: torch.cuda.Stream, handle: int, neglect_local: bool) -> None:
         """Enqueue one op of rank `owner`'s list on `stream`."""

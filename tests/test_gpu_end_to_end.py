@@ -326,3 +326,76 @@ def test_ring_allgather_gemm_whole_mesh(hip, kind):
     got = log.cpu().tolist()
     for v in want:
         assert got[v["tile_id"]] == [v["pid"], v["wave"], v["pid_m"], v["pid_n"]], v
+
+
+def test_two_flag_sets_over_iterations(hip):
+    """AG+GEMM iterations with two flag sets: every iteration polls the set that the previous
+    one left zeroed, new data each time, eagerly and as a replayed graph of two iterations."""
+    from syncopate_amd.communication.comm_runtime.communication_context import CommContext
+    from syncopate_amd.communication.common_descriptors import build_all_gather_plan_1d_swizzle
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.gemm import gemm
+    from syncopate_amd.interface.wave_tables import gemm_consumer_tables
+
+    world, rank, M, K, N, BM, BN = 4, 1, 1024, 256, 512, 128, 128
+    rows = M // world
+    plans = {r: build_all_gather_plan_1d_swizzle((M, K), torch.bfloat16, 0, world, r, "a", "pull")
+             for r in range(world)}
+    schedules, info = _compile(plans)
+    tables = gemm_consumer_tables(schedules[rank]["a"], N)
+    ctx = CommContext(rank, info, flag_sets=2)
+    sets = [ctx._flag_sets[i][0][rank] for i in range(2)]
+    g = torch.Generator().manual_seed(4)
+    b = (0.02 * torch.randn(N, K, generator=g)).bfloat16()
+    bd = b.cuda()
+    c = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
+    dev_tables = dict(
+        cur_wave_sizes=torch.tensor(tables.block_shapes, dtype=torch.int32, device="cuda"),
+        wave_offsets=torch.tensor(tables.block_offsets, dtype=torch.int32, device="cuda"),
+        signal_offsets=torch.tensor(tables.signal_offsets, dtype=torch.int32, device="cuda"),
+        cum_tiles=tables.cum_tiles)
+
+    def load(a):
+        for r in range(world):
+            ctx.comm_buffers["a"][r][r * rows:(r + 1) * rows].copy_(a[r * rows:(r + 1) * rows])
+            if r != rank:       # what this rank holds of a peer's shard is stale until the pull lands
+                ctx.comm_buffers["a"][rank][r * rows:(r + 1) * rows].fill_(float("nan"))
+
+    def step():
+        cur = torch.cuda.current_stream()
+        ctx.reset_signals()
+        ctx.start_after(cur)
+        ctx.execute()
+        gemm(ctx.comm_buffers["a"][rank], bd, c, world, 16, BM, BN, 64, 8,
+             signal_ptr=ctx.recv_signal_bufs[rank], **dev_tables)
+        ctx.end_before(cur)
+
+    used = []
+    for it in range(4):
+        a = (0.02 * torch.randn(M, K, generator=g)).bfloat16()
+        load(a.cuda())
+        step()
+        check_status()
+        ctx.check_status()
+        assert _rel(c, numerics.gemm_fp32(a, b)) <= REL_TOL
+        current = ctx.recv_signal_bufs[rank]
+        other = sets[1] if current.data_ptr() == sets[0].data_ptr() else sets[0]
+        assert current.tolist() == [1] * (world - 1)
+        assert other.tolist() == [0] * (world - 1)      # zeroed behind this iteration's copies
+        used.append(current.data_ptr())
+    assert used[0] == used[2] and used[1] == used[3] and used[0] != used[1]
+
+    # two iterations as one graph (one per flag set), replayed with eager work in between
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+        step()
+    for it in range(3):
+        a = (0.02 * torch.randn(M, K, generator=g)).bfloat16()
+        load(a.cuda())
+        c.zero_()
+        graph.replay()
+        check_status()
+        ctx.check_status()
+        assert _rel(c, numerics.gemm_fp32(a, b)) <= REL_TOL
+        assert sorted(s.sum().item() for s in sets) == [0, world - 1]
