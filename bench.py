@@ -280,7 +280,7 @@ def run_producer(device, steps, warmup):
     def launch():
         counters.zero_()
         # 1024 tiles of 256 x 256: four full rounds of 256 programs
-        gemm_producer(a, b, c, flags, sizes, offsets, signals, 256, BM, BN, BK, GROUP_M, cum_tiles=m * n,
+        gemm_producer(a, b, c, flags, sizes, offsets, signals, 256, 256, 256, BK, GROUP_M, cum_tiles=m * n,
                       counter_buffer=counters, xcd_remap=False, eight_waves=EIGHT_WAVES)
 
     for _ in range(warmup):
@@ -325,6 +325,7 @@ def cpu_baseline(state):
 
 
 def main():
+    global BM, BN, NUM_SMS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
@@ -338,6 +339,8 @@ def main():
     ap.add_argument("--copy-blocks", type=int, default=0,
                     help="0: the producer's chunk copies are hipMemcpyAsync (default); N > 0: the library's "
                          "streaming copy kernel with N workgroups")
+    ap.add_argument("--tile", default=f"{BM}x{BN}", help="output tile of the consumer, e.g. 256x256 or 256x224")
+    ap.add_argument("--programs", type=int, default=NUM_SMS, help="persistent programs of the consumer")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one rank's share on ONE GPU: the other ranks of the mesh are "
@@ -347,6 +350,8 @@ def main():
     from syncopate_amd import _lib
 
     _lib.load()      # fail loudly if the HIP library has not been built
+    BM, BN = (int(x) for x in args.tile.lower().split("x"))
+    NUM_SMS = args.programs
     device = torch.device("cuda", 0)
     torch.cuda.set_device(device)
 

@@ -692,7 +692,8 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
     __shared__ int s_abort;
     // C staging of the epilogue: 32 rows x CS_COLS columns per wavefront, 64 columns where LDS allows
     constexpr int NWAVES = WGM * WGN;
-    constexpr int CS_COLS = (!REMOTE && Pipe::LDS_BYTES + NWAVES * 32 * (64 * 2 + 16) + 4096 <= 160 * 1024) ? 64 : 32;
+    constexpr int CS_COLS = (!REMOTE && (BN / WGN / 32) % 2 == 0 &&
+                             Pipe::LDS_BYTES + NWAVES * 32 * (64 * 2 + 16) + 4096 <= 160 * 1024) ? 64 : 32;
     __shared__ __attribute__((aligned(16))) unsigned char s_cstage[REMOTE ? 16 : NWAVES * 32 * (CS_COLS * 2 + 16)];
 
     const int tid = threadIdx.x;
@@ -994,6 +995,10 @@ static int dispatch_tile(const GemmParams& p, int bm, int bn, bool eight, int gr
         return SYN_EINVAL;
     }
     if (bm == 256 && bn == 256) return launch_gemm<T, PipeT, 256, 256, 2, 2, MODE>(p, grid, stream);
+    // 256x224: four wavefronts stacked in M, each 64 rows x 224 columns (2 x 7 MFMA tiles); N = 3584
+    // is 16 of these, and 32 x 16 tiles are two full rounds of 256 programs
+    if constexpr (PipeT<T, 256, 224, 4, 1>::K_ALIGN == 64)
+        if (bm == 256 && bn == 224) return launch_gemm<T, PipeT, 256, 224, 4, 1, MODE>(p, grid, stream);
     if (bm == 128 && bn == 256) return launch_gemm<T, PipeT, 128, 256, 2, 2, MODE>(p, grid, stream);
     if (bm == 256 && bn == 128) return launch_gemm<T, PipeT, 256, 128, 2, 2, MODE>(p, grid, stream);
     if (bm == 128 && bn == 128) return launch_gemm<T, PipeT, 128, 128, 2, 2, MODE>(p, grid, stream);
@@ -1072,8 +1077,8 @@ static int gemm_entry(const syn_gemm_desc* d, hipStream_t stream, int mode,
     p.c_ld = c_remote ? remote->c_ld : 0;
     p.c_atomic = (remote && remote->c_atomic_add) ? 1 : 0;
     const bool eight = (d->options & SYN_GEMM_EIGHT_WAVES) != 0;
-    // the ring needs whole groups of four 32-deep slabs
-    const bool ring = (d->options & SYN_GEMM_RING_PIPE) && d->K % 128 == 0;
+    // the ring needs whole groups of four 32-deep slabs (and does not exist for 224-wide tiles)
+    const bool ring = (d->options & SYN_GEMM_RING_PIPE) && d->K % 128 == 0 && d->block_n != 224;
 
     const int bm = d->block_m, bn = d->block_n;
     const bool two = (d->options & SYN_GEMM_TWO_STAGE) != 0;

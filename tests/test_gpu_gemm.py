@@ -225,3 +225,24 @@ def test_producer_counters_flags_and_result(hip, BM, BN):
     assert flags.tolist() == [1] * world
     assert _max_rel_err(c, numerics.gemm_fp32(a, b)) <= REL_TOL
     _check_visits(log, sizes, offsets, signals, M, N, BM, BN, 8, 256, M * N, True)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_consumer_256x224_tiles(hip, dtype):
+    """The 224-wide tile (four wavefronts stacked in M, 2 x 7 MFMA tiles each): N = 3584 is 16 of
+    them.  Ragged program counts, odd and even slab counts, both slab pipelines."""
+    from syncopate_amd.computation.gemm import gemm_consumer
+    from syncopate_amd.computation._launch import check_status
+
+    for M, N, K, world, num_sms, two_stage in [(1024, 448, 256, 2, 7, False), (2048, 896, 512, 4, 61, False),
+                                               (2048, 896, 320, 4, 256, True), (1024, 448, 192, 2, 3, False)]:
+        a, b = _inputs(M, N, K, dtype, seed=K)
+        sizes, offsets, signals = _row_waves(M, N, world, 1)
+        flags = torch.ones(world, dtype=torch.int64, device="cuda")
+        c = torch.zeros(M, N, dtype=dtype, device="cuda")
+        log = torch.full(((M // 256) * (N // 224), 4), -1, dtype=torch.int32, device="cuda")
+        gemm_consumer(a.cuda(), b.cuda(), c, flags, sizes, offsets, signals, world, num_sms, 256, 224, 64, 8,
+                      cum_tiles=M * N, visit_log=log, two_stage=two_stage, ring_pipe=(K == 512))
+        check_status()
+        assert _max_rel_err(c, numerics.gemm_fp32(a, b)) <= REL_TOL
+        _check_visits(log, sizes, offsets, signals, M, N, 256, 224, 8, num_sms, M * N, True)
