@@ -28,9 +28,9 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0      # MI355X dense bf16
 HBM_PEAK_GBPS = 8000.0
 # Bytes one launch of the 256x256 consumer kernel moves between L2 and the fabric: FETCH_SIZE and
 # WRITE_SIZE of two counter runs of `bench.py --resident-only`, scaled by the readings of the
-# library's copy kernel (profiles/ag_gemm_8192x8192x3584_bench_hbm_traffic.txt).  Counter runs
+# library's copy kernel (profiles/bench_kernels_hbm_traffic.txt).  Counter runs
 # serialise kernels, so this cannot be sampled while the benchmark itself runs.
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 996.5e6
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 823.1e6
 
 # AG+GEMM, BASELINE configuration 2
 M, K, N, WORLD, RANK = 8192, 8192, 3584, 8, 0
@@ -112,8 +112,17 @@ def run_ag_gemm(state, steps, warmup, resident_only=False, use_graph=True):
                 fused_step()
         return graph
 
-    fused_step()
-    fused_step()
+    if resident_only:
+        # counter runs serialise kernels: a gated consumer would wait for copies that can only
+        # start after it.  Only the producer runs, so that the gathered buffer is complete.
+        use_graph = False
+        ctx.reset_signals()
+        ctx.start_after(stream)
+        ctx.execute()
+        ctx.end_before(stream)
+    else:
+        fused_step()
+        fused_step()
     torch.cuda.synchronize()
     timed_in_graph = steps - steps % 2
     warm_graph = capture(2) if use_graph else None
@@ -410,7 +419,8 @@ def main():
         "max_rel_err_vs_fp32": err,
         "gathered_a_matches": gathered,
         "roofline": {
-            "kernel": "gemm_wave_kernel<bf16, PairPipe, 256x256, 4 wavefronts, consumer>",
+            "kernel": f"gemm_wave_kernel<bf16, {'EarlyPipe' if (BM, BN) in ((256, 256), (256, 224)) else 'SlabPipe<3 stages>'}, "
+                      f"{BM}x{BN}, {8 if EIGHT_WAVES else 4} wavefronts, consumer>",
             "bound": "mfma",
             "achieved": kernel_tflops,
             "peak": MFMA_BF16_PEAK_TFLOPS,
