@@ -37,6 +37,7 @@ M, K, N, WORLD, RANK = 8192, 8192, 3584, 8, 0
 BM, BN, BK, GROUP_M = 256, 256, 64, 8
 NUM_SMS = 224                        # 448 tiles = 2 per program; 32 of the 256 CUs stay free for the
                                      # copy kernels of the producer
+LEAD_OPS = 1                         # ops of the side stream the consumer launch waits for (see fused_step)
 EIGHT_WAVES = False                  # 256-thread workgroups: one wavefront per SIMD, 128x128 of C each
 
 
@@ -96,7 +97,8 @@ def run_ag_gemm(state, steps, warmup, resident_only=False, use_graph=True):
         cur = torch.cuda.current_stream()
         ctx.reset_signals()               # switches to the zeroed flag set
         ctx.start_after(cur)
-        ctx.execute()
+        ctx.execute(lead_ops=LEAD_OPS)
+        ctx.wait_lead(cur)                # the kernel starts behind the first chunk's copy
         consumer(ctx.recv_signal_bufs[RANK])
         ctx.end_before(cur)
 
@@ -334,7 +336,7 @@ def cpu_baseline(state):
 
 
 def main():
-    global BM, BN, NUM_SMS
+    global BM, BN, NUM_SMS, LEAD_OPS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
@@ -350,6 +352,8 @@ def main():
                          "streaming copy kernel with N workgroups")
     ap.add_argument("--tile", default=f"{BM}x{BN}", help="output tile of the consumer, e.g. 256x256 or 256x224")
     ap.add_argument("--programs", type=int, default=NUM_SMS, help="persistent programs of the consumer")
+    ap.add_argument("--lead-ops", type=int, default=LEAD_OPS,
+                    help="the consumer launch waits for this many leading ops of the side stream (0: none)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one rank's share on ONE GPU: the other ranks of the mesh are "
@@ -361,6 +365,7 @@ def main():
     _lib.load()      # fail loudly if the HIP library has not been built
     BM, BN = (int(x) for x in args.tile.lower().split("x"))
     NUM_SMS = args.programs
+    LEAD_OPS = args.lead_ops
     device = torch.device("cuda", 0)
     torch.cuda.set_device(device)
 

@@ -155,13 +155,30 @@ class CommContext:
             return self.recv_signal_bufs[rank]
         raise NotImplementedError(f"Signal type {signal_type} not implemented yet.")
 
-    def execute(self, neglect_local: bool = False) -> None:
-        """Enqueue this rank's ops, stream by stream, in list order."""
+    def execute(self, neglect_local: bool = False, lead_ops: int = 0) -> None:
+        """Enqueue this rank's ops, stream by stream, in list order.
+
+        `lead_ops` > 0 records an event behind the first `lead_ops` ops of every stream;
+        `wait_lead(stream)` makes a stream wait for them.  Launch order gives the copies that
+        head start over the compute kernel when everything is launched from the host; inside a
+        replayed graph the kernel and the first copy become ready at the same moment, the kernel
+        takes the compute units, and every chunk of the iteration arrives later."""
+        self._lead_events = []
         for stream, ops in zip(self.streams, self.info.operations[self.rank]):
             handle = int(stream.cuda_stream)
-            for op in ops:
+            for index, op in enumerate(ops):
                 self._issue(op, self.rank, stream, handle, neglect_local)
+                if lead_ops > 0 and index + 1 == min(lead_ops, len(ops)):
+                    event = torch.cuda.Event()
+                    event.record(stream)
+                    self._lead_events.append(event)
         self._zero_stale_set()
+
+    def wait_lead(self, stream: Optional[torch.cuda.Stream] = None) -> None:
+        """`stream` continues once the leading ops of the last execute(lead_ops=...) are done."""
+        stream = torch.cuda.current_stream(self.device) if stream is None else stream
+        for event in getattr(self, "_lead_events", []):
+            stream.wait_event(event)
 
     def execute_mesh(self, neglect_local: bool = False) -> None:
         """Enqueue EVERY rank's ops on this rank's first communication stream, in an order that
