@@ -3,7 +3,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 A step is one fused all-gather+GEMM iteration of rank 0 of a simulated mesh of 8
-(BASELINE configuration 2): flags reset, the 7 peer chunks of A (1024 x 8192 bf16 each)
+(M, K, N = 8192, 8192, 3584): flags reset, the 7 peer chunks of A (1024 x 8192 bf16 each)
 copied into the symmetric buffer on a side stream in the order the lowered schedule
 prescribes (copy, then flag), the consumer GEMM (8192 x 8192 x 3584) on the compute stream
 waiting on each chunk's flag.  All operands are resident in HBM before the timed region.
@@ -32,7 +32,7 @@ HBM_PEAK_GBPS = 8000.0
 # serialise kernels, so this cannot be sampled while the benchmark itself runs.
 GEMM_TRAFFIC_BYTES_PER_LAUNCH = 823.1e6
 
-# AG+GEMM, BASELINE configuration 2
+# AG+GEMM, the headline configuration
 M, K, N, WORLD, RANK = 8192, 8192, 3584, 8, 0
 BM, BN, BK, GROUP_M = 256, 256, 64, 8
 NUM_SMS = 224                        # 448 tiles = 2 per program; 32 of the 256 CUs stay free for the
@@ -210,7 +210,7 @@ def check_ag_gemm(state):
 
 
 def run_reduce(device, steps, warmup):
-    """GEMM+RS chunked reduce at BASELINE configuration 3: 8 x (1024, 8192) bf16 -> (1024, 8192).
+    """GEMM+RS chunked reduce of the headline GEMM+RS configuration: 8 x (1024, 8192) bf16 -> (1024, 8192).
     Launches rotate over three sets of operands (3 x 151 MB, more than the 256 MB of memory-side
     cache) so that every launch streams from HBM; the batch is timed as a whole."""
     from syncopate_amd.computation.reduce import ring_reduce
@@ -236,7 +236,7 @@ def run_reduce(device, steps, warmup):
 
 
 def run_attention(device, steps, warmup):
-    """All-gather attention at BASELINE configuration 5: 4096 local q rows, 32 heads, against 32768
+    """All-gather attention at the headline ring / all-gather configuration: 4096 local q rows, 32 heads, against 32768
     kv rows as 8 chunks of 4096 in double-ring arrival order (every chunk resident), head dim 128."""
     from syncopate_amd.computation._launch import check_status
     from syncopate_amd.computation.attn import attention_forward
@@ -271,7 +271,7 @@ def run_attention(device, steps, warmup):
 
 
 def run_producer(device, steps, warmup):
-    """GEMM+RS producer at BASELINE configuration 3: partial C (8192, 8192) = A (8192, 3584) B^T in
+    """GEMM+RS producer of the headline GEMM+RS configuration: partial C (8192, 8192) = A (8192, 3584) B^T in
     wave order 1..7, 0 with per-wave counters and flags."""
     from syncopate_amd.computation.gemm import gemm_producer
 

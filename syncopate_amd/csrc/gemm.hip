@@ -8,14 +8,18 @@
 // chunk of its row a lane fetches is XOR-swizzled with the row number so that the 128-bit
 // fragment reads of v_mfma_f32_32x32x16 are bank-conflict free over the 64 LDS banks.
 //
-// Two pipelines over the same tile walk, both with one barrier per slab and MFMA work on
-// both sides of it:
-//   slab   2 or 3 stages of 64-deep slabs: rows are whole 128-byte cache lines; one slab (two,
-//          where three stages fit the 160 KB of LDS: every tile but 256x256) in flight while
-//          another is multiplied; any K % 64 == 0.  The default.
+// Pipelines over the same tile walk (the 64 fills of a 256x256 slab take the texture path of a
+// compute unit about 1400 cycles, a k16 step of MFMAs 512: where the fills are issued matters):
+//   early  2 stages of 64-deep slabs, the LDS reads of a slab bunched at its start so that its
+//          stage is refilled during three of the four k16 steps; the default for the tiles of
+//          which only two stages fit the 160 KB of LDS (256x256, 256x224).
+//   slab   3 stages of 64-deep slabs, a slab's fills spread over the four k16 steps; the default
+//          for the other tiles.  With 2 stages (an option) all fills go out in one step.
+//          Rows are whole 128-byte cache lines; any K % 64 == 0.
 //   ring   4 stages of 32-deep slabs, three in flight; rows are half cache lines, which costs
 //          L1 fill bandwidth.  Needs K % 128 == 0.
-// A tile's first fills are issued before the previous tile's C is stored.
+// A tile's first fills are issued before the previous tile's C is stored; C leaves through a
+// per-wavefront LDS strip as whole cache lines.
 //
 // Consumer form: before the first tile of a wave whose signal offset is >= 0 lane 0 spins on
 // the flag word, then the whole workgroup takes an acquire fence (template.py:121-128).

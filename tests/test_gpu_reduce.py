@@ -37,7 +37,7 @@ def test_ring_reduce_bit_exact(hip, dtype, name, world, rows, N, acc_mode):
 
 
 def test_ring_reduce_full_size_properties(hip):
-    """BASELINE size (8 x (1024, 8192) bf16): integer-valued inputs make every partial sum
+    """Benchmark size (8 x (1024, 8192) bf16): integer-valued inputs make every partial sum
     exact, so the result must equal the integer sum whatever the order or rounding."""
     from syncopate_amd.computation.reduce import ring_reduce
 

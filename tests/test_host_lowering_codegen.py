@@ -213,7 +213,7 @@ def test_matches_reference_outputs(case):
 
 
 def test_baseline_closed_forms():
-    """The tables the BASELINE configurations lower to (W=8), as closed forms."""
+    """The tables the benchmarked configurations lower to (W=8), as closed forms."""
     c2 = _EXPECTED["ag_swizzle_pull_c2"]["schedules"]
     for r in range(8):
         s = c2[str(r)]["a"]
