@@ -216,6 +216,11 @@ typedef struct syn_attn_desc {
     int64_t k_strides[3];
     int64_t v_strides[3];
     int64_t o_strides[3];
+    int32_t* counters;              /* optional device int32[num_waves], zeroed: producer form (the
+                                       generated launcher's counter_ptr, transform/transformer.py:
+                                       880-901, 1125-1137): no flag is waited for; every finished
+                                       tile bumps counters[wave] and the tile that completes a wave
+                                       (Z*H*Q blocks of it) sets flags[signal_offsets[wave]] to 1   */
 } syn_attn_desc;
 
 int syn_attn_fwd(const syn_attn_desc* desc, syn_stream_t stream);

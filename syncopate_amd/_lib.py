@@ -118,6 +118,7 @@ class AttnDesc(ctypes.Structure):
         ("k_strides", c_int64 * 3),
         ("v_strides", c_int64 * 3),
         ("o_strides", c_int64 * 3),
+        ("counters", c_void_p),
     ]
 
 

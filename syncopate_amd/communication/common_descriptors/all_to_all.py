@@ -1,8 +1,9 @@
 """All-to-all plan builders.
 
 Behavioural restatement of syncopate/communication/common_descriptors/all_to_all.py:
-`build_all_to_all_plan` (dim-0 sharded, :11-169) and `build_all_to_all_plan_dim`
-(moves the sharding from one axis to another, :179-370).
+`build_all_to_all_plan` (dim-0 sharded, :11-169), `build_all_to_all_plan_dim`
+(moves the sharding from one axis to another, :179-370) and `build_all_to_all_plan_axis`
+(exchange along one axis, source and destination of one shape, :575-735).
 
 Op order matters to everything downstream (signal offsets, arrival waves):
 when communication produces the data a compute kernel will read
@@ -205,3 +206,56 @@ def build_all_to_all_plan_dim(
 
 
 __all__ = ["build_all_to_all_plan", "build_all_to_all_plan_dim"]
+
+
+def build_all_to_all_plan_axis(
+    shape: Sequence[int],
+    *,
+    dtype: torch.dtype,
+    mesh_size: int,
+    rank: int,
+    src_buffer: str,
+    dst_buffer: str,
+    split_axis: int,
+    transfer_kind: Literal["push", "pull"] = "push",
+    compute_producer: bool = False,
+) -> DevicePlan:
+    """All-to-all along `split_axis`, the same axis before and after: `shape` is the local source
+    tensor, slice p of the axis goes to rank p and lands there in slice `rank` of a destination
+    of the same shape, e.g. attention output [B, S, H/w, D] -> [B, w * S/w, H/w, D] with the
+    sequence blocks regrouped by sender."""
+    elem_size = dtype.itemsize
+    if mesh_size <= 0:
+        raise ValueError("mesh_size must be positive")
+    if elem_size <= 0:
+        raise ValueError("elem_size must be positive")
+    shape = tuple(shape)
+    if not shape:
+        raise ValueError("all_to_all expects at least one dimension in the source shape")
+    split_axis = normalize_axis(split_axis, len(shape))
+    ensure_divisible(shape[split_axis], mesh_size, axis=split_axis)
+    chunk = shape[split_axis] // mesh_size
+    if chunk == 0:
+        raise ValueError("all-to-all requires non-empty slices along the split axis")
+    if block_nbytes(shape, elem_size, {split_axis: chunk}) == 0:
+        raise ValueError("all-to-all transfer would be empty")
+    strides = row_major_strides(shape)
+
+    def slice_of(index: int) -> BufferRegion:
+        return BufferRegion.from_slices(
+            elem_size=elem_size, strides=strides,
+            slices=axis_box(shape, {split_axis: (index * chunk, (index + 1) * chunk)}))
+
+    plan = DevicePlan(dev=rank)
+    plan.src_shape = shape
+    plan.dst_shape = shape
+    plan.tensors_involved[src_buffer] = (torch.Size(shape), dtype)
+    plan.tensors_involved[dst_buffer] = (torch.Size(shape), dtype)
+    plan.local_regions.setdefault(src_buffer, []).append(slice_of(rank))
+
+    if transfer_kind not in {"push", "pull"}:
+        raise ValueError("transfer_kind must be 'push' or 'pull'")
+    peers = [(rank + step) % mesh_size for step in range(1, mesh_size)]
+    return _emit_exchange(plan, rank=rank, mesh_size=mesh_size, peers=peers, src_buffer=src_buffer,
+                          dst_buffer=dst_buffer, src_region_for=slice_of, dst_region_for=slice_of,
+                          transfer_kind=transfer_kind, compute_producer=compute_producer)

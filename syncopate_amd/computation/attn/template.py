@@ -59,6 +59,8 @@ def attention_forward(
     causal: bool = False,
     layout: str = "bhsd",
     num_programs: int = 0,
+    counter_ptr: Optional[torch.Tensor] = None,
+    output_buffer: Optional[torch.Tensor] = None,
     out: Optional[torch.Tensor] = None,
     return_lse: bool = False,
     visit_log: Optional[torch.Tensor] = None,
@@ -71,6 +73,12 @@ def attention_forward(
     above the diagonal are skipped, the diagonal block is masked.
     `num_programs` > 0 runs that many persistent workgroups over the tile ids
     instead of one workgroup per tile.
+    `counter_ptr` (int32, one zeroed word per wave) selects the producer form the transform
+    pass generates for attention that feeds an all-to-all
+    (tests/test_attn_all2all_transform.py:182-214): no flag is waited for; every finished tile
+    bumps its wave's counter and the tile that completes a wave sets the wave's flag in
+    `signal_ptr`.  `output_buffer` (alias of `out`) is the reference's name for the comm buffer
+    the result is written into.
     """
     dev = require_cuda(q, k, v, signal_ptr)
     if not (q.dtype == k.dtype == v.dtype):
@@ -121,6 +129,14 @@ def attention_forward(
         if caller_owned:
             remember_checked(tables, (num_waves, Z, H, Sq, Skv, cum_tiles, flags.numel()))
 
+    if output_buffer is not None:
+        if out is not None and out is not output_buffer:
+            raise ValueError("give out or output_buffer, not both")
+        out = output_buffer
+    if counter_ptr is not None:
+        if counter_ptr.dtype != torch.int32 or counter_ptr.device != dev or not counter_ptr.is_contiguous() \
+                or counter_ptr.numel() < num_waves:
+            raise ValueError("counter_ptr must be a contiguous int32 tensor with one word per wave on q's device")
     o = torch.empty(q.shape, dtype=q.dtype, device=dev) if out is None else out
     if o.shape != q.shape or o.dtype != q.dtype:
         raise ValueError("out must match q")
@@ -144,6 +160,7 @@ def attention_forward(
         block_m=BLOCK_M, block_n=BLOCK_N, causal=1 if causal else 0, num_programs=int(num_programs),
         sm_scale=float(sm_scale), cum_tiles=int(cum_tiles), spin_timeout_us=int(spin_timeout_us),
         q_strides=strides(q), k_strides=strides(k), v_strides=strides(v), o_strides=strides(o),
+        counters=None if counter_ptr is None else counter_ptr.data_ptr(),
     )
     with torch.cuda.device(dev):
         _lib.check("syn_attn_fwd", lib.syn_attn_fwd(ctypes.byref(desc), _lib.stream_handle(stream)))

@@ -47,6 +47,7 @@ struct AttnParams {
     const int32_t* signal_offsets;
     int32_t* visit_log;
     int32_t* status;
+    int32_t* counters;
     int64_t timeout_ticks;
     int32_t num_waves;
     int32_t Z, H, Sq, Skv;
@@ -194,7 +195,8 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
         const int kv_end = p.causal ? min(kv_hi, qb + 1) : kv_hi;
         if (kv_lo >= kv_end) continue;
 
-        if (sig >= 0) {
+        // producer form (counters given): the wave's flag is one this kernel SETS, nothing to wait for
+        if (sig >= 0 && p.counters == nullptr) {
             if (tid == 0) {
                 const bool ok = spin_until_equal(p.flags + sig, 1ull, p.timeout_ticks);
                 if (!ok) {
@@ -452,6 +454,15 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
         if (tid == 0) {
             __hip_atomic_store(p.first + lock_idx, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __hip_atomic_store(p.lock + lock_idx, 0, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+            // producer form (generated epilogue, transform/transformer.py:880-901): count the tile
+            // in its wave; the tile that completes the wave (all z, h and q blocks of it: the kv
+            // range is not counted) publishes the wave's flag
+            if (p.counters != nullptr && sig >= 0) {
+                const int wave_tiles = p.wave_sizes[w * 4 + 0] * size_h * nq;
+                const int done = __hip_atomic_fetch_add(p.counters + w, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+                if (done == wave_tiles - 1)
+                    __hip_atomic_store(p.flags + sig, 1ull, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+            }
         }
     }
 }
@@ -531,6 +542,7 @@ int syn_attn_fwd(const syn_attn_desc* d, syn_stream_t stream) {
     p.signal_offsets = d->signal_offsets;
     p.visit_log = d->visit_log;
     p.status = d->status;
+    p.counters = d->counters;
     p.timeout_ticks = timeout_ticks(d->spin_timeout_us);
     p.num_waves = d->num_waves;
     p.Z = d->Z;

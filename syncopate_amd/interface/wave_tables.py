@@ -108,3 +108,17 @@ def all2all_attn_tables(schedule: RawSchedule, axes: Dict[str, int]) -> AttnWave
             emit(p, w, w, p, w)
             emit(w, p, w, p, p)
     return AttnWaveTables(offsets, sizes, signals, cums, total)
+
+
+def attn_producer_tables(schedule: RawSchedule, axes: Dict[str, int], kv_len: int) -> AttnWaveTables:
+    """Attention that PRODUCES the source of an all-to-all along the sequence axis: one wave per
+    outgoing sequence chunk of the output, every q block of it against the whole K/V; the signals
+    are the COMPUTE_DONE flags the kernel sets (tests/test_attn_all2all_transform.py:57-85)."""
+    b, h, s = axes["batch"], axes["head"], axes["seq"]
+    offsets, sizes, cums, total = [], [], [], 0
+    for off, shape in zip(schedule.gen_block_offset_lists(), schedule.gen_block_shape_lists()):
+        offsets.append([off[b], off[h], off[s], 0])
+        sizes.append([shape[b], shape[h], shape[s], kv_len])
+        total += shape[b] * shape[h] * shape[s]
+        cums.append(total)
+    return AttnWaveTables(offsets, sizes, schedule.gen_signal_lists(), cums, total)

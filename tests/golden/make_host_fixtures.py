@@ -83,6 +83,16 @@ CASES = {
                                dict(shape=(2, 2, 12, 3), dtype="float32", src_buffer="src", dst_buffer="dst",
                                     src_split_axis=1, dst_split_axis=2, transfer_kind="push",
                                     peer_order="counter-clockwise"), 4, [True, False]),
+    "a2a_axis_push_producer_attn": ("build_all_to_all_plan_axis",
+                                    dict(shape=(2, 12288, 8, 128), dtype="float16", src_buffer="src",
+                                         dst_buffer="dst", split_axis=1, transfer_kind="push",
+                                         compute_producer=True), 4, [True]),
+    "a2a_axis_pull_small": ("build_all_to_all_plan_axis",
+                            dict(shape=(2, 8, 3), dtype="float32", src_buffer="src", dst_buffer="dst",
+                                 split_axis=-2, transfer_kind="pull", compute_producer=False), 4, [True, False]),
+    "a2a_axis_push_w8": ("build_all_to_all_plan_axis",
+                         dict(shape=(1, 16384, 4, 128), dtype="bfloat16", src_buffer="src", dst_buffer="dst",
+                              split_axis=1, transfer_kind="push", compute_producer=True), 8, [True]),
     "rs_direct_push": ("build_reduce_scatter_direct_reduce_plan",
                        dict(shape=(64, 32), dtype="float16", axis=0, src_buffer="src", dst_buffer="dst",
                             transfer_kind="push"), 4, [False]),

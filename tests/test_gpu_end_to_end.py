@@ -399,3 +399,67 @@ def test_two_flag_sets_over_iterations(hip):
         ctx.check_status()
         assert _rel(c, numerics.gemm_fp32(a, b)) <= REL_TOL
         assert sorted(s.sum().item() for s in sets) == [0, world - 1]
+
+
+@pytest.mark.parametrize("rank,dtype,causal", [(1, torch.float16, False), (3, torch.bfloat16, False),
+                                                (0, torch.bfloat16, True)])
+def test_attention_to_all2all_iteration(hip, rank, dtype, causal):
+    """Attention as the PRODUCER of an all-to-all along the sequence axis
+    (tests/test_attn_all2all_transform.py:105-214 of the reference): the kernel writes its output
+    into the comm buffer wave by wave (one wave per destination rank), counts finished tiles per
+    wave and sets the wave's COMPUTE_DONE flag; the side stream waits for each flag and pushes
+    that sequence chunk to its owner."""
+    from syncopate_amd.communication.comm_runtime.communication_context import CommContext
+    from syncopate_amd.communication.common_descriptors import build_all_to_all_plan_axis
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.attn import attention_forward
+    from syncopate_amd.interface.wave_tables import attn_producer_tables
+
+    world, B, Hp, D = 4, 2, 2, 128
+    SEQ = world * 256
+    chunk = SEQ // world
+    g = torch.Generator().manual_seed(21 + rank)
+    q, k, v = (torch.randn(B, SEQ, Hp, D, generator=g).to(dtype) for _ in range(3))
+
+    plans = {r: build_all_to_all_plan_axis(shape=(B, SEQ, Hp, D), dtype=dtype, mesh_size=world, rank=r,
+                                           src_buffer="src", dst_buffer="dst", split_axis=1,
+                                           transfer_kind="push", compute_producer=True)
+             for r in range(world)}
+    schedules, info = _compile(plans)
+    tables = attn_producer_tables(schedules[rank]["src"], {"batch": 0, "head": 2, "seq": 1}, SEQ)
+    # remote chunks first, in the order of the pushes, the rank's own chunk last
+    assert [off[2] // chunk for off in tables.wave_offsets] == [(rank + 1 + i) % world for i in range(world)]
+    assert tables.signal_offsets == list(range(world))
+
+    ctx = CommContext(rank, info)
+    src = ctx.comm_buffers["src"][rank]
+    src.fill_(float("nan"))              # a chunk shipped before its tiles were stored would carry NaNs
+    flags = ctx.compute_signal_bufs[rank]
+    counters = torch.zeros(flags.numel(), dtype=torch.int32, device="cuda")
+    comm_stream = torch.cuda.Stream()
+    main = torch.cuda.current_stream()
+
+    ctx.reset_signals()
+    comm_stream.wait_stream(main)
+    attention_forward(q.cuda(), k.cuda(), v.cuda(), D ** -0.5, layout="bshd", causal=causal,
+                      output_buffer=src, counter_ptr=counters, signal_ptr=flags,
+                      wave_offsets=tables.wave_offsets, wave_sizes=tables.wave_sizes, cum_wave_sizes=tables.cum_wave_sizes,
+                      signal_offsets=tables.signal_offsets, cum_tiles=tables.cum_tiles)
+    ctx.start_after(comm_stream)
+    ctx.execute()
+    ctx.end_before(comm_stream)
+    main.wait_stream(comm_stream)
+    check_status()
+    ctx.check_status()
+
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        q.float().transpose(1, 2), k.float().transpose(1, 2), v.float().transpose(1, 2),
+        scale=D ** -0.5, is_causal=causal).transpose(1, 2)
+    assert _rel(src, ref) <= REL_TOL
+    assert flags.tolist() == [1] * world
+    assert counters.tolist() == [B * Hp * (chunk // 128)] * world
+    for peer in range(world):
+        got = ctx.comm_buffers["dst"][peer][:, rank * chunk:(rank + 1) * chunk]
+        assert torch.equal(got, src[:, peer * chunk:(peer + 1) * chunk])      # bit for bit, no NaNs
+        if peer != rank:
+            assert ctx.recv_signal_bufs[peer].sum().item() == 1

@@ -434,3 +434,30 @@ def test_all2all_attention_tables():
     assert t.wave_sizes == [[1, 2, 128, 128]] * 9
     assert t.signal_offsets == [0, 1, 1, 1, 2, 2, 2, 2, 2]
     assert t.cum_wave_sizes == [256 * (i + 1) for i in range(9)] and t.cum_tiles == 2304
+
+
+def test_attention_producer_tables_by_hand():
+    """Attention that feeds an all-to-all along the sequence axis (bshd, W=2, rank 1): the rank's
+    pushes go to rank 0 first, its own chunk last; one wave per outgoing sequence chunk, all of
+    K/V per wave, flags = the COMPUTE_DONE offsets 0, 1 in op order
+    (reference: tests/test_attn_all2all_transform.py:57-85, 137-163)."""
+    import torch
+
+    from syncopate_amd.communication.code_gen import CommGenerator
+    from syncopate_amd.communication.common_descriptors import build_all_to_all_plan_axis
+    from syncopate_amd.interface import lower_comm_plan_to_raw_schedules
+    from syncopate_amd.interface.wave_tables import attn_producer_tables
+
+    B, SEQ, Hp, D, world = 3, 512, 2, 128, 2
+    plans = {r: build_all_to_all_plan_axis(shape=(B, SEQ, Hp, D), dtype=torch.float16, mesh_size=world, rank=r,
+                                           src_buffer="src", dst_buffer="dst", split_axis=1,
+                                           transfer_kind="push", compute_producer=True) for r in range(world)}
+    gen = CommGenerator(plans)
+    gen.plan_signals()
+    schedule = lower_comm_plan_to_raw_schedules(gen)[1]["src"]
+    t = attn_producer_tables(schedule, {"batch": 0, "head": 2, "seq": 1}, SEQ)
+    assert t.wave_offsets == [[0, 0, 0, 0], [0, 0, 256, 0]]
+    assert t.wave_sizes == [[3, 2, 256, 512], [3, 2, 256, 512]]
+    assert t.signal_offsets == [0, 1]
+    assert t.cum_wave_sizes == [3 * 2 * 256, 2 * 3 * 2 * 256]
+    assert t.cum_tiles == 3 * 2 * 512
