@@ -5,7 +5,12 @@ from .all_gather import (
     build_double_ring_all_gather_plan,
     build_ring_all_gather_plan,
 )
-from .all_to_all import build_all_to_all_plan, build_all_to_all_plan_axis, build_all_to_all_plan_dim
+from .all_to_all import (
+    build_all_to_all_plan,
+    build_all_to_all_plan_axis,
+    build_all_to_all_plan_dim,
+    build_all_to_all_plan_dim_waves,
+)
 from .reduce_scatter import build_reduce_scatter_direct_reduce_plan
 
 __all__ = [
@@ -15,5 +20,6 @@ __all__ = [
     "build_all_to_all_plan",
     "build_all_to_all_plan_dim",
     "build_all_to_all_plan_axis",
+    "build_all_to_all_plan_dim_waves",
     "build_reduce_scatter_direct_reduce_plan",
 ]

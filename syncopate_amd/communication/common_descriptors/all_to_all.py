@@ -2,8 +2,10 @@
 
 Behavioural restatement of syncopate/communication/common_descriptors/all_to_all.py:
 `build_all_to_all_plan` (dim-0 sharded, :11-169), `build_all_to_all_plan_dim`
-(moves the sharding from one axis to another, :179-370) and `build_all_to_all_plan_axis`
-(exchange along one axis, source and destination of one shape, :575-735).
+(moves the sharding from one axis to another, :179-370), `build_all_to_all_plan_dim_waves`
+(the same, with every destination shard delivered in waves, :373-572) and
+`build_all_to_all_plan_axis` (exchange along one axis, source and destination of one shape,
+:575-735).
 
 Op order matters to everything downstream (signal offsets, arrival waves):
 when communication produces the data a compute kernel will read
@@ -259,3 +261,114 @@ def build_all_to_all_plan_axis(
     return _emit_exchange(plan, rank=rank, mesh_size=mesh_size, peers=peers, src_buffer=src_buffer,
                           dst_buffer=dst_buffer, src_region_for=slice_of, dst_region_for=slice_of,
                           transfer_kind=transfer_kind, compute_producer=compute_producer)
+
+
+def build_all_to_all_plan_dim_waves(
+    shape: Sequence[int],
+    *,
+    dtype: torch.dtype,
+    mesh_size: int,
+    rank: int,
+    src_buffer: str,
+    dst_buffer: str,
+    src_split_axis: int,
+    dst_split_axis: int,
+    num_waves: int,
+    transfer_kind: Literal["push", "pull"] = "push",
+    compute_producer: bool = False,
+    peer_order: Literal["clockwise", "counter-clockwise"] = "clockwise",
+) -> DevicePlan:
+    """`build_all_to_all_plan_dim` with every destination shard cut into `num_waves` slices along
+    `dst_split_axis`, so that a receiver can start on the first slices while the rest is on its
+    way.  Wave-major op order: for each wave, one op per peer starting with the rank itself (a
+    local copy, treated like any other peer: first in the round, with its own compute dependency
+    when a kernel produces the source)."""
+    elem_size = dtype.itemsize
+    if mesh_size <= 0:
+        raise ValueError("mesh_size must be positive")
+    if elem_size <= 0:
+        raise ValueError("elem_size must be positive")
+    if num_waves <= 0:
+        raise ValueError("num_waves must be positive")
+    shape = tuple(shape)
+    if not shape:
+        raise ValueError("all_to_all expects at least one dimension in the source shape")
+    ndim = len(shape)
+    src_split_axis = normalize_axis(src_split_axis, ndim)
+    dst_split_axis = normalize_axis(dst_split_axis, ndim)
+    if src_split_axis == dst_split_axis:
+        raise ValueError("src_split_axis and dst_split_axis must differ")
+    src_chunk = shape[src_split_axis]
+    if src_chunk <= 0:
+        raise ValueError("all-to-all requires non-empty slices along the split axis")
+    ensure_divisible(shape[dst_split_axis], mesh_size, axis=dst_split_axis)
+    dst_chunk = shape[dst_split_axis] // mesh_size
+    if dst_chunk == 0:
+        raise ValueError("all-to-all requires non-empty slices along the destination axis")
+    ensure_divisible(dst_chunk, num_waves, "num_waves")
+    wave_chunk = dst_chunk // num_waves
+    if wave_chunk == 0:
+        raise ValueError("wave splitting produced an empty chunk along dst_split_axis")
+    if block_nbytes(shape, elem_size, {src_split_axis: src_chunk, dst_split_axis: wave_chunk}) == 0:
+        raise ValueError("all-to-all transfer would be empty")
+
+    dst_shape = list(shape)
+    dst_shape[src_split_axis] = src_chunk * mesh_size
+    dst_shape[dst_split_axis] = dst_chunk
+    src_strides = row_major_strides(shape)
+    dst_strides = row_major_strides(dst_shape)
+
+    def outgoing(dest_peer: int, wave: int) -> BufferRegion:
+        """Wave `wave` of what this rank holds for `dest_peer` (wave None: all of it)."""
+        lo = dest_peer * dst_chunk + (0 if wave is None else wave * wave_chunk)
+        hi = lo + (dst_chunk if wave is None else wave_chunk)
+        return BufferRegion.from_slices(
+            elem_size=elem_size, strides=src_strides,
+            slices=axis_box(shape, {src_split_axis: (0, src_chunk), dst_split_axis: (lo, hi)}))
+
+    def landing(source_rank: int, wave: int) -> BufferRegion:
+        """Where wave `wave` of `source_rank`'s contribution lands in a destination buffer."""
+        return BufferRegion.from_slices(
+            elem_size=elem_size, strides=dst_strides,
+            slices=axis_box(dst_shape, {src_split_axis: (source_rank * src_chunk, (source_rank + 1) * src_chunk),
+                                        dst_split_axis: (wave * wave_chunk, (wave + 1) * wave_chunk)}))
+
+    plan = DevicePlan(dev=rank)
+    plan.src_shape = shape
+    plan.dst_shape = tuple(dst_shape)
+    plan.tensors_involved[src_buffer] = (torch.Size(shape), dtype)
+    plan.tensors_involved[dst_buffer] = (torch.Size(dst_shape), dtype)
+    plan.local_regions.setdefault(src_buffer, []).append(outgoing(rank, None))
+
+    if transfer_kind not in {"push", "pull"}:
+        raise ValueError("transfer_kind must be 'push' or 'pull'")
+    if peer_order not in {"clockwise", "counter-clockwise"}:
+        raise ValueError("peer_order must be 'clockwise' or 'counter-clockwise'")
+    direction = 1 if peer_order == "clockwise" else -1
+    peers = [(rank + direction * step) % mesh_size for step in range(mesh_size)]     # the rank itself first
+
+    def produced_by(compute_rank: int, region: BufferRegion) -> List:
+        if not compute_producer:
+            return []
+        return [ComputeDependency(compute_rank=compute_rank, src_region=region, signal=None)]
+
+    for wave in range(num_waves):
+        for peer in peers:
+            if peer == rank:
+                piece = outgoing(rank, wave)
+                op = Transfer(op=TransferOp.LOCAL_COPY, src_buf=src_buffer, dst_buf=dst_buffer, src_region=piece,
+                              dst_region=landing(rank, wave),
+                              chunk_idx=(rank * mesh_size + rank) * num_waves + wave,
+                              dependency=produced_by(rank, piece))
+            elif transfer_kind == "push":
+                piece = outgoing(peer, wave)
+                op = Transfer(op=TransferOp.PUSH, src_buf=src_buffer, src_region=piece, peer=peer,
+                              chunk_idx=(rank * mesh_size + peer) * num_waves + wave, dst_buf=dst_buffer,
+                              dst_region=landing(rank, wave), dependency=produced_by(rank, piece))
+            else:
+                piece = outgoing(rank, wave)       # the same box of the peer's source
+                op = Transfer(op=TransferOp.PULL, dst_buf=dst_buffer, dst_region=landing(peer, wave), peer=peer,
+                              chunk_idx=(peer * mesh_size + rank) * num_waves + wave, src_buf=src_buffer,
+                              src_region=piece, dependency=produced_by(peer, piece))
+            plan.add_op(op)
+    return plan

@@ -93,6 +93,18 @@ CASES = {
     "a2a_axis_push_w8": ("build_all_to_all_plan_axis",
                          dict(shape=(1, 16384, 4, 128), dtype="bfloat16", src_buffer="src", dst_buffer="dst",
                               split_axis=1, transfer_kind="push", compute_producer=True), 8, [True]),
+    "a2a_dim_waves_push_small": ("build_all_to_all_plan_dim_waves",
+                                 dict(shape=(2, 8, 2), dtype="float32", src_buffer="src", dst_buffer="dst",
+                                      src_split_axis=2, dst_split_axis=1, num_waves=2, transfer_kind="push"),
+                                 4, [True, False]),
+    "a2a_dim_waves_pull_producer": ("build_all_to_all_plan_dim_waves",
+                                    dict(shape=(6, 4), dtype="float16", src_buffer="src", dst_buffer="dst",
+                                         src_split_axis=1, dst_split_axis=0, num_waves=3, transfer_kind="pull",
+                                         compute_producer=True, peer_order="counter-clockwise"), 2, [True]),
+    "a2a_dim_waves_push_producer_gemm": ("build_all_to_all_plan_dim_waves",
+                                         dict(shape=(8192, 1024), dtype="bfloat16", src_buffer="src",
+                                              dst_buffer="dst", src_split_axis=1, dst_split_axis=0, num_waves=4,
+                                              transfer_kind="push", compute_producer=True), 8, [True]),
     "rs_direct_push": ("build_reduce_scatter_direct_reduce_plan",
                        dict(shape=(64, 32), dtype="float16", axis=0, src_buffer="src", dst_buffer="dst",
                             transfer_kind="push"), 4, [False]),

@@ -288,3 +288,25 @@ def test_device_plan_text_and_streams():
     split = _gather(0, "pull", shape=(16, 4)).split_xfers(2)
     assert [x.chunk_idx for x in split.xfers] == [2, 3, 4, 5, 6, 7]
     assert [x.nbytes for x in split.xfers] == [16] * 6
+
+
+def test_all_to_all_dim_waves_splits_destination_axis():
+    """Literal vectors of the reference's tests/test_descriptor.py:192-221."""
+    import torch
+
+    from syncopate_amd.communication.common_descriptors import build_all_to_all_plan_dim_waves
+
+    mesh_size, num_waves = 2, 3
+    plan = build_all_to_all_plan_dim_waves(shape=(6, 2), dtype=torch.float32, mesh_size=mesh_size, rank=0,
+                                           src_buffer="src", dst_buffer="dst", src_split_axis=1,
+                                           dst_split_axis=0, num_waves=num_waves, transfer_kind="push")
+    assert plan.dst_shape == (3, 4)
+    assert len(plan.xfers) == (mesh_size - 1) * num_waves
+    assert len(plan.local_copies) == num_waves
+    assert [xf.src_region.describe() for xf in plan.xfers] == ["[3:4, 0:2]", "[4:5, 0:2]", "[5:6, 0:2]"]
+    assert [xf.dst_region.describe() for xf in plan.xfers] == ["[0:1, 0:2]", "[1:2, 0:2]", "[2:3, 0:2]"]
+    assert [c.dst_region.describe() for c in plan.local_copies] == ["[0:1, 0:2]", "[1:2, 0:2]", "[2:3, 0:2]"]
+    assert sorted([xf.chunk_idx for xf in plan.xfers] + [c.chunk_idx for c in plan.local_copies]) == [0, 1, 2, 3, 4, 5]
+    with pytest.raises(ValueError):
+        build_all_to_all_plan_dim_waves(shape=(6, 2), dtype=torch.float32, mesh_size=2, rank=0, src_buffer="s",
+                                        dst_buffer="d", src_split_axis=1, dst_split_axis=0, num_waves=2)
