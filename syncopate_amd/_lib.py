@@ -28,6 +28,7 @@ SYN_GEMM_EIGHT_WAVES = 2
 SYN_GEMM_RING_PIPE = 4
 SYN_GEMM_NO_K_STAGGER = 8
 SYN_GEMM_TWO_STAGE = 16
+SYN_ELEM_BF16, SYN_ELEM_FP16, SYN_ELEM_FP32, SYN_ELEM_1B, SYN_ELEM_2B, SYN_ELEM_4B, SYN_ELEM_8B = range(7)
 
 _ERRORS = {
     SYN_EINVAL: "SYN_EINVAL (malformed argument or unsupported configuration)",
@@ -145,6 +146,8 @@ _SIGNATURES = {
     ),
     "syn_copy_async": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p]),
     "syn_copy_kernel_async": (c_int32, [c_void_p, c_void_p, c_int64, c_int32, c_void_p]),
+    "syn_box_copy_async": (c_int32, [c_void_p, c_void_p, c_int32, POINTER(c_int64), POINTER(c_int64),
+                                     POINTER(c_int64), c_int32, c_int32, c_int32, c_void_p]),
     "syn_flag_set": (c_int32, [c_void_p, c_uint64, c_void_p]),
     "syn_flag_wait": (c_int32, [c_void_p, c_uint64, c_int64, c_void_p, c_void_p]),
     "syn_delay_us": (c_int32, [c_int64, c_void_p]),

@@ -37,6 +37,8 @@ from .operations import (
     SMCopyOp,
     WaitIntraNodeSignal,
 )
+from .persistent_copy import persistent_copy_last_contig
+from .streams import pick_side_streams
 
 SIGNAL_DTYPE = torch.int64   # 8-byte flag words, value 1 = set
 
@@ -52,7 +54,8 @@ class CommContext:
 
     def __init__(self, rank: int, info: CommInfo, multi_info: bool = False, *,
                  device: Optional[torch.device] = None, link_delay_us: int = 0,
-                 wait_timeout_us: int = 2_000_000, copy_blocks: int = 0, flag_sets: int = 1) -> None:
+                 wait_timeout_us: int = 2_000_000, copy_blocks: int = 0, flag_sets: int = 1,
+                 compute_stream: Optional[torch.cuda.Stream] = None) -> None:
         if info.local_world_size <= 0:
             info.local_world_size = info.world_size
         if info.local_world_size != info.world_size:
@@ -99,8 +102,12 @@ class CommContext:
             for name, (shape, dtype) in info.comm_buffer_sizes.items()
         }
         self.status = torch.zeros(_lib.SYN_STATUS_WORDS, dtype=torch.int32, device=self.device)
-        self.streams = [torch.cuda.Stream(device=self.device) for _ in info.operations[self.rank]]
-        self.compute_stream = None
+        # one stream per op list, none of them on the hardware queue of the stream the compute
+        # kernels are launched on (the current stream unless `compute_stream` names it): a flag
+        # wait spinning on a shared queue would hold back the very kernel that sets the flag
+        self.compute_stream = (torch.cuda.current_stream(self.device) if compute_stream is None
+                               else compute_stream)
+        self.streams = pick_side_streams(len(info.operations[self.rank]), self.compute_stream, self.device)
 
     # ---- flags and stream ordering -------------------------------------------
 
@@ -141,7 +148,10 @@ class CommContext:
             comm_stream.wait_stream(stream)
 
     def end_before(self, stream: Optional[torch.cuda.Stream] = None) -> None:
-        """`stream` continues only after all communication streams have drained."""
+        """`stream` continues only after all communication streams have drained.  Call it after
+        the compute kernels have been launched: a join enqueued before them on a stream that
+        happens to share their hardware queue would hold them back, and with them the flags the
+        communication streams are waiting for."""
         stream = torch.cuda.current_stream(self.device) if stream is None else stream
         for comm_stream in self.streams:
             stream.wait_stream(comm_stream)
@@ -164,6 +174,7 @@ class CommContext:
         replayed graph the kernel and the first copy become ready at the same moment, the kernel
         takes the compute units, and every chunk of the iteration arrives later."""
         self._lead_events = []
+        self._check_copy_units(self.info.operations[self.rank])
         for stream, ops in zip(self.streams, self.info.operations[self.rank]):
             handle = int(stream.cuda_stream)
             for index, op in enumerate(ops):
@@ -194,6 +205,7 @@ class CommContext:
         handle = int(stream.cuda_stream)
         world = self.info.local_world_size
         lists = [(r, ops) for r in range(world) for ops in self.info.operations[r]]
+        self._check_copy_units(ops for _, ops in lists)
         cursor = [0] * len(lists)
         written = set()                  # (signal type, rank, offset) already enqueued as a write
         for r in range(world):
@@ -217,6 +229,11 @@ class CommContext:
             if not progressed:
                 raise RuntimeError("the op lists wait for flags nobody writes: the plan cannot be replayed")
         self._zero_stale_set()
+
+    def _check_copy_units(self, op_lists) -> None:
+        # before anything is enqueued (communication_context.py:164 asserts it per op)
+        if self.info.num_copy_sms <= 0 and any(isinstance(op, SMCopyOp) for ops in op_lists for op in ops):
+            raise ValueError("box copies run on compute units: set CommInfo.num_copy_sms first")
 
     def _issue(self, op, owner: int, stream: torch.cuda.Stream, handle: int, neglect_local: bool) -> None:
         """Enqueue one op of rank `owner`'s list on `stream`."""
@@ -263,13 +280,12 @@ class CommContext:
             dst = self.comm_buffers[op.dst][op.dst_rank % world]
             src_box = src[tuple(slice(ax.start, ax.end) for ax in op.src_slice)]
             dst_box = dst[tuple(slice(ax.start, ax.end) for ax in op.dst_slice)]
-            with torch.cuda.stream(stream):
-                if op.reduce_op is None:
-                    dst_box.copy_(src_box.reshape(dst_box.shape))
-                elif op.reduce_op == ReduceOp.SUM:
-                    dst_box.add_(src_box.reshape(dst_box.shape))
-                else:
-                    raise NotImplementedError(f"reduce op {op.reduce_op} in a box copy")
+            if op.reduce_op is not None and op.reduce_op != ReduceOp.SUM:
+                raise NotImplementedError(f"reduce op {op.reduce_op} in a box copy")
+            if self.link_delay_us and op.src_rank != op.dst_rank:
+                _lib.check("syn_delay_us", lib.syn_delay_us(self.link_delay_us, handle))
+            persistent_copy_last_contig(src_box, dst_box, num_sms=self.info.num_copy_sms,
+                                        reduce_op=op.reduce_op, stream=stream)
         elif isinstance(op, CollectiveComm):
             raise NotImplementedError(
                 "library collectives need the other ranks to be real processes; "

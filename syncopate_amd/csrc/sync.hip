@@ -47,6 +47,180 @@ stream_copy_kernel(u32x4_t* __restrict__ dst, const u32x4_t* __restrict__ src, i
     for (; i < vecs; i += stride) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
 }
 
+// Box copy: a box of up to 5 dimensions, contiguous along the last one in source and
+// destination, byte strides otherwise arbitrary; optionally dst += src by atomic adds, so that
+// several senders may accumulate into one destination at a time.  The box is a list of rows
+// (the last dimension); a row is cut into units of 16, 8, 4, 2 or 1 bytes - the largest that
+// divides the row length, both base addresses and every stride - and the units are dealt to the
+// lanes grid-stride, four in flight per lane.  Counterpart of the reference's SM-driven copies
+// (comm_runtime/non_tma_persistent_copy.py:106-304, tma_persistent_copy.py), which the generated
+// op lists use with copy_engine=False (SMCopyOp) and for reduce-scatter by direct reduction.
+struct BoxParams {
+    unsigned char* dst;
+    const unsigned char* src;
+    int64_t outer[4];          // extents of the dimensions in front of the last, leading ones padded with 1
+    int64_t src_stride[4];     // in bytes
+    int64_t dst_stride[4];
+    int64_t row_units;         // units per row
+    int64_t total_units;
+    int32_t n_outer;           // how many of outer[] (counted from the back) are real
+};
+
+constexpr int kBoxThreads = 1024;
+constexpr int kBoxInFlight = 4;
+
+template <int BYTES> struct BoxUnit;
+template <> struct BoxUnit<16> { typedef u32x4_t type; };
+template <> struct BoxUnit<8> { typedef uint64_t type; };
+template <> struct BoxUnit<4> { typedef uint32_t type; };
+template <> struct BoxUnit<2> { typedef uint16_t type; };
+template <> struct BoxUnit<1> { typedef uint8_t type; };
+
+// unit index -> byte offsets of the unit in source and destination
+template <typename IdxT, int UNIT>
+__device__ __forceinline__ void box_locate(const BoxParams& p, IdxT u, int64_t& so, int64_t& dof) {
+    IdxT row = u / (IdxT)p.row_units;
+    const IdxT col = u - row * (IdxT)p.row_units;
+    so = (int64_t)col * UNIT;
+    dof = so;
+    for (int d = 3; d >= 4 - p.n_outer; --d) {
+        const IdxT q = row / (IdxT)p.outer[d];
+        const IdxT i = row - q * (IdxT)p.outer[d];
+        so += (int64_t)i * p.src_stride[d];
+        dof += (int64_t)i * p.dst_stride[d];
+        row = q;
+    }
+}
+
+template <typename IdxT, int UNIT>
+__global__ void __launch_bounds__(kBoxThreads) box_copy_kernel(const BoxParams p) {
+    typedef typename BoxUnit<UNIT>::type unit_t;
+    const IdxT total = (IdxT)p.total_units;
+    const IdxT stride = (IdxT)gridDim.x * kBoxThreads;
+    for (IdxT base = (IdxT)blockIdx.x * kBoxThreads + threadIdx.x; base < total; base += kBoxInFlight * stride) {
+        unit_t v[kBoxInFlight];
+        int64_t dof[kBoxInFlight];
+#pragma unroll
+        for (int k = 0; k < kBoxInFlight; ++k) {
+            const IdxT u = base + (IdxT)k * stride;
+            if (u < total) {
+                int64_t so;
+                box_locate<IdxT, UNIT>(p, u, so, dof[k]);
+                v[k] = __builtin_nontemporal_load(reinterpret_cast<const unit_t*>(p.src + so));
+            } else {
+                dof[k] = -1;
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < kBoxInFlight; ++k)
+            if (dof[k] >= 0) *reinterpret_cast<unit_t*>(p.dst + dof[k]) = v[k];
+    }
+}
+
+// dst += v for one unit of UNIT bytes holding elements of type T, by no-return atomics
+template <typename T, int UNIT> struct BoxAdd;
+
+template <int UNIT> struct BoxAdd<float, UNIT> {
+    typedef typename BoxUnit<UNIT>::type unit_t;
+    static __device__ __forceinline__ void apply(unsigned char* dst, unit_t v) {
+        float vals[UNIT / 4];
+        __builtin_memcpy(vals, &v, UNIT);
+#pragma unroll
+        for (int e = 0; e < UNIT / 4; ++e)
+            __hip_atomic_fetch_add(reinterpret_cast<float*>(dst) + e, vals[e], __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+    }
+};
+
+template <typename T> __device__ __forceinline__ void packed_add(unsigned char* dst, uint32_t two);
+template <> __device__ __forceinline__ void packed_add<__bf16>(unsigned char* dst, uint32_t two) {
+    typedef __bf16 v2 __attribute__((ext_vector_type(2)));
+    typedef __attribute__((address_space(1))) v2* gptr;
+    __builtin_amdgcn_global_atomic_fadd_v2bf16((gptr)dst, __builtin_bit_cast(v2, two));
+}
+template <> __device__ __forceinline__ void packed_add<_Float16>(unsigned char* dst, uint32_t two) {
+    typedef _Float16 v2 __attribute__((ext_vector_type(2)));
+    typedef __attribute__((address_space(1))) v2* gptr;
+    __builtin_amdgcn_global_atomic_fadd_v2f16((gptr)dst, __builtin_bit_cast(v2, two));
+}
+
+// 16-bit elements: pairs go through the packed atomics; a single element (a box that starts or
+// ends on an odd element) through compare-and-swap on the 32-bit word around it
+template <typename T, int UNIT> struct BoxAdd {
+    typedef typename BoxUnit<UNIT>::type unit_t;
+    static __device__ __forceinline__ void apply(unsigned char* dst, unit_t v) {
+        if constexpr (UNIT >= 4) {
+            uint32_t words[UNIT / 4];
+            __builtin_memcpy(words, &v, UNIT);
+#pragma unroll
+            for (int e = 0; e < UNIT / 4; ++e) packed_add<T>(dst + 4 * e, words[e]);
+        } else {
+            const uintptr_t addr = reinterpret_cast<uintptr_t>(dst);
+            uint32_t* word = reinterpret_cast<uint32_t*>(addr & ~(uintptr_t)3);
+            const int shift = (addr & 2) ? 16 : 0;
+            const float add = (float)__builtin_bit_cast(T, (uint16_t)v);
+            uint32_t seen = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (;;) {
+                const T cur = __builtin_bit_cast(T, (uint16_t)(seen >> shift));
+                const uint32_t sum = __builtin_bit_cast(uint16_t, (T)((float)cur + add));
+                const uint32_t want = (seen & ~(0xffffu << shift)) | (sum << shift);
+                if (__hip_atomic_compare_exchange_strong(word, &seen, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                                         __HIP_MEMORY_SCOPE_AGENT))
+                    break;
+            }
+        }
+    }
+};
+
+template <typename T, typename IdxT, int UNIT>
+__global__ void __launch_bounds__(kBoxThreads) box_add_kernel(const BoxParams p) {
+    typedef typename BoxUnit<UNIT>::type unit_t;
+    const IdxT total = (IdxT)p.total_units;
+    const IdxT stride = (IdxT)gridDim.x * kBoxThreads;
+    for (IdxT base = (IdxT)blockIdx.x * kBoxThreads + threadIdx.x; base < total; base += kBoxInFlight * stride) {
+        unit_t v[kBoxInFlight];
+        int64_t dof[kBoxInFlight];
+#pragma unroll
+        for (int k = 0; k < kBoxInFlight; ++k) {
+            const IdxT u = base + (IdxT)k * stride;
+            if (u < total) {
+                int64_t so;
+                box_locate<IdxT, UNIT>(p, u, so, dof[k]);
+                v[k] = __builtin_nontemporal_load(reinterpret_cast<const unit_t*>(p.src + so));
+            } else {
+                dof[k] = -1;
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < kBoxInFlight; ++k)
+            if (dof[k] >= 0) BoxAdd<T, UNIT>::apply(p.dst + dof[k], v[k]);
+    }
+}
+
+template <typename IdxT>
+static void launch_box_copy(const BoxParams& p, int unit, int blocks, hipStream_t s) {
+    const dim3 g(blocks), b(kBoxThreads);
+    switch (unit) {
+        case 16: hipLaunchKernelGGL((box_copy_kernel<IdxT, 16>), g, b, 0, s, p); break;
+        case 8: hipLaunchKernelGGL((box_copy_kernel<IdxT, 8>), g, b, 0, s, p); break;
+        case 4: hipLaunchKernelGGL((box_copy_kernel<IdxT, 4>), g, b, 0, s, p); break;
+        case 2: hipLaunchKernelGGL((box_copy_kernel<IdxT, 2>), g, b, 0, s, p); break;
+        default: hipLaunchKernelGGL((box_copy_kernel<IdxT, 1>), g, b, 0, s, p); break;
+    }
+}
+
+template <typename T, typename IdxT>
+static void launch_box_add(const BoxParams& p, int unit, int blocks, hipStream_t s) {
+    const dim3 g(blocks), b(kBoxThreads);
+    if (unit == 16) {
+        hipLaunchKernelGGL((box_add_kernel<T, IdxT, 16>), g, b, 0, s, p);
+    } else if (unit >= 4) {
+        hipLaunchKernelGGL((box_add_kernel<T, IdxT, 4>), g, b, 0, s, p);
+    } else {
+        if constexpr (sizeof(T) == 2) hipLaunchKernelGGL((box_add_kernel<T, IdxT, 2>), g, b, 0, s, p);
+    }
+}
+
 __global__ void __launch_bounds__(64) delay_kernel(int64_t ticks) {
     if (threadIdx.x == 0) {
         const uint64_t t0 = wall_clock64();
@@ -74,6 +248,76 @@ int syn_copy_kernel_async(void* dst, const void* src, int64_t nbytes, int32_t nu
     hipLaunchKernelGGL(syn::stream_copy_kernel, dim3(num_blocks), dim3(256), 0,
                        reinterpret_cast<hipStream_t>(stream), reinterpret_cast<syn::u32x4_t*>(dst),
                        reinterpret_cast<const syn::u32x4_t*>(src), nbytes / 16);
+    return (int)hipGetLastError();
+}
+
+int syn_box_copy_async(void* dst, const void* src, int32_t ndim, const int64_t* shape,
+                       const int64_t* src_strides, const int64_t* dst_strides, int32_t elem_kind,
+                       int32_t reduce_sum, int32_t num_blocks, syn_stream_t stream) {
+    using namespace syn;
+    if (!dst || !src || !shape || !src_strides || !dst_strides) return SYN_EINVAL;
+    if (ndim < 1 || ndim > 5) return SYN_EINVAL;
+    if (num_blocks <= 0) return SYN_EINVAL;
+    int elem = 0;
+    switch (elem_kind) {
+        case SYN_ELEM_BF16: case SYN_ELEM_FP16: case SYN_ELEM_2B: elem = 2; break;
+        case SYN_ELEM_FP32: case SYN_ELEM_4B: elem = 4; break;
+        case SYN_ELEM_1B: elem = 1; break;
+        case SYN_ELEM_8B: elem = 8; break;
+        default: return SYN_EINVAL;
+    }
+    const bool sum = reduce_sum != 0;
+    if (sum && elem_kind != SYN_ELEM_BF16 && elem_kind != SYN_ELEM_FP16 && elem_kind != SYN_ELEM_FP32)
+        return SYN_EINVAL;                                   // sums need a float type
+    if (src_strides[ndim - 1] != 1 || dst_strides[ndim - 1] != 1) return SYN_EINVAL;   // rows are contiguous
+    if (shape[ndim - 1] <= 0) return SYN_EINVAL;
+    const uintptr_t da = reinterpret_cast<uintptr_t>(dst), sa = reinterpret_cast<uintptr_t>(src);
+    if (da % elem || sa % elem) return SYN_EINVAL;
+    BoxParams p;
+    p.dst = reinterpret_cast<unsigned char*>(dst);
+    p.src = reinterpret_cast<const unsigned char*>(src);
+    p.n_outer = ndim - 1;
+    const int64_t row_bytes = shape[ndim - 1] * elem;
+    // every address of the box is a multiple of the unit when these all are
+    uint64_t mix = (uint64_t)da | (uint64_t)sa | (uint64_t)row_bytes | 16u;
+    int64_t rows = 1;
+    for (int d = 0; d < 4; ++d) {
+        const int from = ndim - 1 - (4 - d);     // outer[3] is the dimension next to the last
+        if (from >= 0) {
+            if (shape[from] <= 0 || src_strides[from] < 0 || dst_strides[from] < 0) return SYN_EINVAL;
+            p.outer[d] = shape[from];
+            p.src_stride[d] = src_strides[from] * elem;
+            p.dst_stride[d] = dst_strides[from] * elem;
+            if (shape[from] > 1) mix |= (uint64_t)p.src_stride[d] | (uint64_t)p.dst_stride[d];
+            rows *= shape[from];
+        } else {
+            p.outer[d] = 1;
+            p.src_stride[d] = p.dst_stride[d] = 0;
+        }
+    }
+    int unit = (int)(mix & (~mix + 1));          // lowest set bit: 1, 2, 4, 8 or 16
+    if (sum && unit == 8) unit = 4;              // sums come in 16-byte groups, pairs/floats, single elements
+    p.row_units = row_bytes / unit;
+    p.total_units = rows * p.row_units;
+    const int64_t needed = (p.total_units + kBoxThreads - 1) / kBoxThreads;
+    const int blocks = (int)(needed < num_blocks ? needed : num_blocks);
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    // 32-bit index arithmetic is several times cheaper; below 2^29 units no index of the
+    // four-deep grid-stride loop can wrap (stride <= total + 1023)
+    const bool narrow = p.total_units < (int64_t)1 << 29;
+    if (!sum) {
+        if (narrow) launch_box_copy<uint32_t>(p, unit, blocks, s);
+        else launch_box_copy<uint64_t>(p, unit, blocks, s);
+    } else if (elem_kind == SYN_ELEM_BF16) {
+        if (narrow) launch_box_add<__bf16, uint32_t>(p, unit, blocks, s);
+        else launch_box_add<__bf16, uint64_t>(p, unit, blocks, s);
+    } else if (elem_kind == SYN_ELEM_FP16) {
+        if (narrow) launch_box_add<_Float16, uint32_t>(p, unit, blocks, s);
+        else launch_box_add<_Float16, uint64_t>(p, unit, blocks, s);
+    } else {
+        if (narrow) launch_box_add<float, uint32_t>(p, unit, blocks, s);
+        else launch_box_add<float, uint64_t>(p, unit, blocks, s);
+    }
     return (int)hipGetLastError();
 }
 

@@ -463,3 +463,94 @@ def test_attention_to_all2all_iteration(hip, rank, dtype, causal):
         assert torch.equal(got, src[:, peer * chunk:(peer + 1) * chunk])      # bit for bit, no NaNs
         if peer != rank:
             assert ctx.recv_signal_bufs[peer].sum().item() == 1
+
+
+@pytest.mark.parametrize("kind,rank", [("pull", 1), ("pull", 3), ("push", 2)])
+def test_gemm_rs_sm_reduce_iteration(hip, kind, rank):
+    """Reduce-scatter by direct reduction with box copies on compute units
+    (tests/test_gemm_rs_sm_reduce.py:95-175): every rank's producer GEMM writes its partial product
+    and one COMPUTE_DONE flag per chunk; `pull`: this rank's side stream waits for each peer's
+    chunk and adds it into its own result; `push`: it adds its own chunks into the peers' results."""
+    from syncopate_amd.communication.code_gen import CodeGenOptions, CommGenerator
+    from syncopate_amd.communication.comm_runtime.communication_context import CommContext
+    from syncopate_amd.communication.common_descriptors import build_reduce_scatter_direct_reduce_plan
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.gemm import gemm_producer
+    from syncopate_amd.interface import lower_comm_plan_to_raw_schedules
+    from syncopate_amd.interface.wave_tables import gemm_producer_tables
+
+    world, M, N, K, BM, BN, programs = 4, 1024, 512, 256, 128, 128, 24
+    rows = M // world
+    dtype = torch.float16
+    plans = {r: build_reduce_scatter_direct_reduce_plan(shape=(M, N), dtype=dtype, axis=0, mesh_size=world,
+                                                        rank=r, src_buffer="src", dst_buffer="dst",
+                                                        transfer_kind=kind) for r in range(world)}
+    gen = CommGenerator(plans)
+    gen.plan_signals()
+    schedules = lower_comm_plan_to_raw_schedules(gen)
+    info = gen.generate_code_for_plan(options=CodeGenOptions(copy_engine=False, use_tma=False))
+    info.local_world_size = info.world_size
+    ctx = CommContext(rank, info)
+    with pytest.raises(ValueError):
+        ctx.execute()                     # box copies need compute units: num_copy_sms is still 0
+    torch.cuda.synchronize()
+    info.num_copy_sms = 10
+
+    g = torch.Generator().manual_seed(23)
+    a = [(0.1 * torch.randn(M, K, generator=g)).to(dtype) for _ in range(world)]
+    b = [(0.1 * torch.randn(N, K, generator=g)).to(dtype) for _ in range(world)]
+    start = (0.25 * torch.randn(world, rows, N, generator=g)).to(dtype)
+    for r in range(world):
+        ctx.comm_buffers["src"][r].fill_(float("nan"))     # a chunk added before it was stored shows
+        ctx.comm_buffers["dst"][r].copy_(start[r].cuda())
+    ctx.reset_signals(whole_mesh=True)
+    ctx.start_after()
+    ctx.execute()                                          # the side stream waits for the flags
+    runs = range(world) if kind == "pull" else [rank]
+    for r in runs:
+        tables = gemm_producer_tables(schedules[r]["src"])
+        gemm_producer(a[r].cuda(), b[r].cuda(), ctx.comm_buffers["src"][r], ctx.compute_signal_bufs[r],
+                      tables.block_shapes, tables.block_offsets, tables.signal_offsets, programs, BM, BN, 64, 8,
+                      cum_tiles=tables.cum_tiles)
+    ctx.end_before()
+    check_status()
+    ctx.check_status()
+
+    partial = {r: ctx.comm_buffers["src"][r].cpu() for r in runs}
+    for r in runs:
+        assert _rel(partial[r], numerics.gemm_fp32(a[r], b[r])) <= REL_TOL
+    tiny = torch.finfo(dtype).tiny
+
+    def add_once(acc, term, fragile):
+        """One addition in the element type; `fragile` collects the elements where an operand or
+        the sum is subnormal (atomic units may flush those), which are compared by tolerance."""
+        out = (acc.float() + term.float()).to(dtype)
+        for t in (acc, term, out):
+            fragile |= (t.abs() < tiny) & (t != 0)
+        return out
+
+    def same(got, want, fragile):
+        assert torch.equal(got[~fragile], want[~fragile])
+        assert fragile.float().mean().item() < 0.01
+        torch.testing.assert_close(got[fragile].float(), want[fragile].float(), atol=1e-3, rtol=0)
+
+    if kind == "pull":
+        # additions in the op list's order, one rounding each
+        order = [op.src_rank for ops in info.operations[rank] for op in ops if hasattr(op, "src_slice")]
+        assert sorted(order) == list(range(world)) and order[-1] == rank
+        want = start[rank].clone()
+        fragile = torch.zeros(rows, N, dtype=torch.bool)
+        for r in order:
+            want = add_once(want, partial[r][rank * rows:(rank + 1) * rows], fragile)
+        same(ctx.comm_buffers["dst"][rank].cpu(), want, fragile)
+        assert ctx.recv_signal_bufs[rank].tolist() == [1] * world
+        total = start[rank].double() + sum(numerics.gemm_fp32(a[r], b[r])[rank * rows:(rank + 1) * rows].double()
+                                           for r in range(world))
+        # the reference's bound for this path (tests/test_gemm_rs_sm_reduce.py:175)
+        torch.testing.assert_close(ctx.comm_buffers["dst"][rank].cpu().double(), total, atol=1e-2, rtol=1e-2)
+    else:
+        for peer in range(world):
+            fragile = torch.zeros(rows, N, dtype=torch.bool)
+            want = add_once(start[peer], partial[rank][peer * rows:(peer + 1) * rows], fragile)
+            same(ctx.comm_buffers["dst"][peer].cpu(), want, fragile)
+            assert ctx.recv_signal_bufs[peer].tolist() == [1 if i == rank else 0 for i in range(world)]

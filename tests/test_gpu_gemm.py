@@ -123,6 +123,7 @@ def test_consumer_gated_by_side_stream_producer(hip):
     """Chunks land in the symmetric buffer on a side stream (copy, then flag) while the
     consumer is already running; the result must be bitwise the resident one."""
     from syncopate_amd import _lib
+    from syncopate_amd.communication.comm_runtime.streams import pick_side_streams
     from syncopate_amd.computation.gemm import gemm_consumer
     from syncopate_amd.computation._launch import check_status
 
@@ -141,7 +142,8 @@ def test_consumer_gated_by_side_stream_producer(hip):
     symm[rank * rows:(rank + 1) * rows].copy_(staged[rank * rows:(rank + 1) * rows])
     flags.zero_()
     c = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
-    side = torch.cuda.Stream()
+    # a stream on the compute stream's hardware queue would leave the copies stuck behind the polling kernel
+    side = pick_side_streams(1)[0]
     torch.cuda.synchronize()
     main = torch.cuda.current_stream()
     side.wait_stream(main)
