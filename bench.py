@@ -235,6 +235,37 @@ def run_reduce(device, steps, warmup):
     return ms, nbytes
 
 
+def run_box_copies(device, steps, warmup):
+    """Box copies on compute units (the SM copy ops of reduce-scatter by direct reduction): one
+    rank's (8192, 8192) bf16 partial product added into / copied onto a result of the same shape
+    with 256 workgroups.  Operands rotate over three sets (6 x 134 MB) so that every launch
+    streams from HBM.  Returns {form: (ms, HBM bytes per launch)}."""
+    from syncopate_amd.communication.comm_runtime.persistent_copy import persistent_copy_last_contig
+    from syncopate_amd.communication.descriptor import ReduceOp
+
+    rows, n, sets, blocks = 8192, 8192, 3, 256
+    torch.manual_seed(3)
+    src = [torch.randn(rows, n, device=device).bfloat16() for _ in range(sets)]
+    dst = [torch.zeros(rows, n, dtype=torch.bfloat16, device=device) for _ in range(sets)]
+    stream = torch.cuda.current_stream()
+    nbytes = rows * n * 2
+    forms = {"copy": (None, False, 2 * nbytes), "add_exclusive": (ReduceOp.SUM, True, 3 * nbytes),
+             "add_atomic": (ReduceOp.SUM, False, 3 * nbytes)}
+    result = {}
+    for name, (op, exclusive, traffic) in forms.items():
+        for i in range(max(warmup, sets)):
+            persistent_copy_last_contig(src[i % sets], dst[i % sets], num_sms=blocks, reduce_op=op, exclusive=exclusive)
+        torch.cuda.synchronize()
+        begin, end = _events(1)[0], _events(1)[0]
+        begin.record(stream)
+        for i in range(steps):
+            persistent_copy_last_contig(src[i % sets], dst[i % sets], num_sms=blocks, reduce_op=op, exclusive=exclusive)
+        end.record(stream)
+        torch.cuda.synchronize()
+        result[name] = (begin.elapsed_time(end) / steps, traffic)
+    return result
+
+
 def run_attention(device, steps, warmup):
     """All-gather attention at the headline ring / all-gather configuration: 4096 local q rows, 32 heads, against 32768
     kv rows as 8 chunks of 4096 in double-ring arrival order (every chunk resident), head dim 128."""
@@ -375,6 +406,7 @@ def main():
     traffic_calibration(device)
     err, gathered = check_ag_gemm(state)
     reduce_ms, reduce_bytes = run_reduce(device, max(args.steps, 30), args.warmup)
+    boxes = run_box_copies(device, max(args.steps, 20), args.warmup)
     attn_ms, attn_flop, attn_err = run_attention(device, 5, 2)
     prod_ms, prod_flop = run_producer(device, args.steps, args.warmup)
 
@@ -414,6 +446,8 @@ def main():
         "rs_reduce_GBps": reduce_bytes / (reduce_ms * 1e-3) / 1e9,
         "rs_reduce_us": reduce_ms * 1e3,
         "rs_reduce_pct_hbm_peak": 100.0 * reduce_bytes / (reduce_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+        "box_copy_GBps": {name: traffic / (ms * 1e-3) / 1e9 for name, (ms, traffic) in boxes.items()},
+        "box_copy_us": {name: ms * 1e3 for name, (ms, _) in boxes.items()},
         "rs_producer_tflops": prod_flop / (prod_ms * 1e-3) / 1e12,
         "rs_producer_pct_bf16_mfma_peak": 100.0 * prod_flop / (prod_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
         "attn_tflops": attn_flop / (attn_ms * 1e-3) / 1e12,

@@ -252,17 +252,23 @@ int syn_copy_kernel_async(void* dst, const void* src, int64_t nbytes, int32_t nu
 #define SYN_ELEM_2B 4
 #define SYN_ELEM_4B 5
 #define SYN_ELEM_8B 6
-/* Copy (reduce_sum = 0) or accumulate (reduce_sum = 1: dst += src by atomic adds, so several
- * senders may add into one destination at a time) a box of 1..5 dimensions with at most
- * `num_blocks` 1024-thread workgroups.  `shape` and the strides count elements; the last
- * dimension is contiguous (stride 1) on both sides.  Accesses are 16 bytes wide when row length,
- * base addresses and strides allow, narrower otherwise, down to one element.  Counterpart of the
- * reference's SM-driven copies persistent_naive_copy_last_contig / persistent_tma_copy_last_contig
- * (comm_runtime/non_tma_persistent_copy.py:106-304, tma_persistent_copy.py), which replay SMCopyOp
- * (communication_context.py:161-189); five dimensions at most there too (MAX_RANK). */
+/* What syn_box_copy_async does with the destination */
+#define SYN_BOX_COPY 0            /* dst = src */
+#define SYN_BOX_ADD_ATOMIC 1      /* dst += src by atomic adds: several senders may add into one
+                                     destination at a time (the reference's tl.atomic_add) */
+#define SYN_BOX_ADD_EXCLUSIVE 2   /* dst += src by plain read-modify-write, several times faster:
+                                     for a destination that has one writer at a time */
+/* Copy or accumulate (one rounding in the element type per addition) a box of 1..5 dimensions
+ * with at most `num_blocks` 1024-thread workgroups.  `shape` and the strides count elements; the
+ * last dimension is contiguous (stride 1) on both sides.  Accesses are 16 bytes wide when row
+ * length, base addresses and strides allow, narrower otherwise, down to one element.  Counterpart
+ * of the reference's SM-driven copies persistent_naive_copy_last_contig /
+ * persistent_tma_copy_last_contig (comm_runtime/non_tma_persistent_copy.py:106-304,
+ * tma_persistent_copy.py), which replay SMCopyOp (communication_context.py:161-189); five
+ * dimensions at most there too (MAX_RANK). */
 int syn_box_copy_async(void* dst, const void* src, int32_t ndim, const int64_t* shape,
                        const int64_t* src_strides, const int64_t* dst_strides, int32_t elem_kind,
-                       int32_t reduce_sum, int32_t num_blocks, syn_stream_t stream);
+                       int32_t reduce_mode, int32_t num_blocks, syn_stream_t stream);
 int syn_flag_set(uint64_t* flag, uint64_t value, syn_stream_t stream);
 int syn_flag_wait(const uint64_t* flag, uint64_t value, int64_t spin_timeout_us,
                   int32_t* status, syn_stream_t stream);

@@ -102,6 +102,7 @@ class CommContext:
             for name, (shape, dtype) in info.comm_buffer_sizes.items()
         }
         self.status = torch.zeros(_lib.SYN_STATUS_WORDS, dtype=torch.int32, device=self.device)
+        self._sole_writer_ops = self._find_sole_writer_ops()
         # one stream per op list, none of them on the hardware queue of the stream the compute
         # kernels are launched on (the current stream unless `compute_stream` names it): a flag
         # wait spinning on a shared queue would hold back the very kernel that sets the flag
@@ -230,6 +231,36 @@ class CommContext:
                 raise RuntimeError("the op lists wait for flags nobody writes: the plan cannot be replayed")
         self._zero_stale_set()
 
+    def _find_sole_writer_ops(self) -> set:
+        """Accumulating box copies whose destination box nobody outside their own op list writes
+        (the lists of every rank are known here).  One list is one stream, so such a box has one
+        writer at a time and the sum need not be atomic: reduce-scatter by direct reduction in
+        its pull form, where each rank adds its peers' chunks into its own result.  In the push
+        form every rank adds into every other rank's result and the sums stay atomic."""
+        writers = []          # (list key, buffer name, rank, box or None for a byte-range copy)
+        for r, lists in enumerate(self.info.operations):
+            for i, ops in enumerate(lists):
+                for op in ops:
+                    if isinstance(op, SMCopyOp):
+                        box = tuple((ax.start, ax.end) for ax in op.dst_slice)
+                        writers.append(((r, i), op.dst, op.dst_rank, box, op))
+                    elif isinstance(op, CopyEngineOp):
+                        writers.append(((r, i), op.dst, op.dst_rank, None, op))
+
+        def overlap(a, b) -> bool:
+            if a is None or b is None or len(a) != len(b):
+                return True
+            return all(lo1 < hi2 and lo2 < hi1 for (lo1, hi1), (lo2, hi2) in zip(a, b))
+
+        sole = set()
+        for key, name, rank, box, op in writers:
+            if not isinstance(op, SMCopyOp) or op.reduce_op is None:
+                continue
+            if all(k == key or n != name or rk != rank or not overlap(box, bx)
+                   for k, n, rk, bx, _ in writers):
+                sole.add(id(op))
+        return sole
+
     def _check_copy_units(self, op_lists) -> None:
         # before anything is enqueued (communication_context.py:164 asserts it per op)
         if self.info.num_copy_sms <= 0 and any(isinstance(op, SMCopyOp) for ops in op_lists for op in ops):
@@ -285,7 +316,8 @@ class CommContext:
             if self.link_delay_us and op.src_rank != op.dst_rank:
                 _lib.check("syn_delay_us", lib.syn_delay_us(self.link_delay_us, handle))
             persistent_copy_last_contig(src_box, dst_box, num_sms=self.info.num_copy_sms,
-                                        reduce_op=op.reduce_op, stream=stream)
+                                        reduce_op=op.reduce_op, stream=stream,
+                                        exclusive=id(op) in self._sole_writer_ops)
         elif isinstance(op, CollectiveComm):
             raise NotImplementedError(
                 "library collectives need the other ranks to be real processes; "

@@ -67,7 +67,9 @@ struct BoxParams {
 };
 
 constexpr int kBoxThreads = 1024;
-constexpr int kBoxInFlight = 4;
+// loads in flight per lane: 64 bytes' worth, at most 16 (twice that gains nothing: a compute unit moves about
+// 32 bytes per clock through its vector memory path either way)
+template <int UNIT> struct BoxDepth { static constexpr int value = UNIT >= 16 ? 4 : (UNIT == 8 ? 8 : 16); };
 
 template <int BYTES> struct BoxUnit;
 template <> struct BoxUnit<16> { typedef u32x4_t type; };
@@ -95,6 +97,7 @@ __device__ __forceinline__ void box_locate(const BoxParams& p, IdxT u, int64_t& 
 template <typename IdxT, int UNIT>
 __global__ void __launch_bounds__(kBoxThreads) box_copy_kernel(const BoxParams p) {
     typedef typename BoxUnit<UNIT>::type unit_t;
+    constexpr int kBoxInFlight = BoxDepth<UNIT>::value;
     const IdxT total = (IdxT)p.total_units;
     const IdxT stride = (IdxT)gridDim.x * kBoxThreads;
     for (IdxT base = (IdxT)blockIdx.x * kBoxThreads + threadIdx.x; base < total; base += kBoxInFlight * stride) {
@@ -172,9 +175,25 @@ template <typename T, int UNIT> struct BoxAdd {
     }
 };
 
-template <typename T, typename IdxT, int UNIT>
+// dst += v for one unit by a plain read-modify-write: for a destination with one writer at a time
+template <typename T, int UNIT>
+__device__ __forceinline__ void box_add_plain(unsigned char* dst, typename BoxUnit<UNIT>::type v) {
+    typedef typename BoxUnit<UNIT>::type unit_t;
+    constexpr int kN = UNIT / (int)sizeof(T);
+    unit_t cur = *reinterpret_cast<const unit_t*>(dst);
+    T a[kN], b[kN];
+    __builtin_memcpy(a, &cur, UNIT);
+    __builtin_memcpy(b, &v, UNIT);
+#pragma unroll
+    for (int e = 0; e < kN; ++e) a[e] = (T)((float)a[e] + (float)b[e]);     // one rounding, as an add in T
+    __builtin_memcpy(&cur, a, UNIT);
+    *reinterpret_cast<unit_t*>(dst) = cur;
+}
+
+template <typename T, typename IdxT, int UNIT, bool ATOMIC>
 __global__ void __launch_bounds__(kBoxThreads) box_add_kernel(const BoxParams p) {
     typedef typename BoxUnit<UNIT>::type unit_t;
+    constexpr int kBoxInFlight = BoxDepth<UNIT>::value;
     const IdxT total = (IdxT)p.total_units;
     const IdxT stride = (IdxT)gridDim.x * kBoxThreads;
     for (IdxT base = (IdxT)blockIdx.x * kBoxThreads + threadIdx.x; base < total; base += kBoxInFlight * stride) {
@@ -192,8 +211,11 @@ __global__ void __launch_bounds__(kBoxThreads) box_add_kernel(const BoxParams p)
             }
         }
 #pragma unroll
-        for (int k = 0; k < kBoxInFlight; ++k)
-            if (dof[k] >= 0) BoxAdd<T, UNIT>::apply(p.dst + dof[k], v[k]);
+        for (int k = 0; k < kBoxInFlight; ++k) {
+            if (dof[k] < 0) continue;
+            if constexpr (ATOMIC) BoxAdd<T, UNIT>::apply(p.dst + dof[k], v[k]);
+            else box_add_plain<T, UNIT>(p.dst + dof[k], v[k]);
+        }
     }
 }
 
@@ -209,15 +231,28 @@ static void launch_box_copy(const BoxParams& p, int unit, int blocks, hipStream_
     }
 }
 
-template <typename T, typename IdxT>
+template <typename T, typename IdxT, bool ATOMIC>
 static void launch_box_add(const BoxParams& p, int unit, int blocks, hipStream_t s) {
     const dim3 g(blocks), b(kBoxThreads);
     if (unit == 16) {
-        hipLaunchKernelGGL((box_add_kernel<T, IdxT, 16>), g, b, 0, s, p);
-    } else if (unit >= 4) {
-        hipLaunchKernelGGL((box_add_kernel<T, IdxT, 4>), g, b, 0, s, p);
+        if constexpr (!ATOMIC) hipLaunchKernelGGL((box_add_kernel<T, IdxT, 16, false>), g, b, 0, s, p);
+    } else if (unit == 8) {
+        if constexpr (!ATOMIC) hipLaunchKernelGGL((box_add_kernel<T, IdxT, 8, false>), g, b, 0, s, p);
+    } else if (unit == 4) {
+        hipLaunchKernelGGL((box_add_kernel<T, IdxT, 4, ATOMIC>), g, b, 0, s, p);
     } else {
-        if constexpr (sizeof(T) == 2) hipLaunchKernelGGL((box_add_kernel<T, IdxT, 2>), g, b, 0, s, p);
+        if constexpr (sizeof(T) == 2) hipLaunchKernelGGL((box_add_kernel<T, IdxT, 2, ATOMIC>), g, b, 0, s, p);
+    }
+}
+
+template <typename T>
+static void launch_box_add_any(const BoxParams& p, int unit, int blocks, bool narrow, bool atomic, hipStream_t s) {
+    if (atomic) {
+        if (narrow) launch_box_add<T, uint32_t, true>(p, unit, blocks, s);
+        else launch_box_add<T, uint64_t, true>(p, unit, blocks, s);
+    } else {
+        if (narrow) launch_box_add<T, uint32_t, false>(p, unit, blocks, s);
+        else launch_box_add<T, uint64_t, false>(p, unit, blocks, s);
     }
 }
 
@@ -253,7 +288,7 @@ int syn_copy_kernel_async(void* dst, const void* src, int64_t nbytes, int32_t nu
 
 int syn_box_copy_async(void* dst, const void* src, int32_t ndim, const int64_t* shape,
                        const int64_t* src_strides, const int64_t* dst_strides, int32_t elem_kind,
-                       int32_t reduce_sum, int32_t num_blocks, syn_stream_t stream) {
+                       int32_t reduce_mode, int32_t num_blocks, syn_stream_t stream) {
     using namespace syn;
     if (!dst || !src || !shape || !src_strides || !dst_strides) return SYN_EINVAL;
     if (ndim < 1 || ndim > 5) return SYN_EINVAL;
@@ -266,7 +301,9 @@ int syn_box_copy_async(void* dst, const void* src, int32_t ndim, const int64_t* 
         case SYN_ELEM_8B: elem = 8; break;
         default: return SYN_EINVAL;
     }
-    const bool sum = reduce_sum != 0;
+    if (reduce_mode < SYN_BOX_COPY || reduce_mode > SYN_BOX_ADD_EXCLUSIVE) return SYN_EINVAL;
+    const bool sum = reduce_mode != SYN_BOX_COPY;
+    const bool atomic = reduce_mode == SYN_BOX_ADD_ATOMIC;
     if (sum && elem_kind != SYN_ELEM_BF16 && elem_kind != SYN_ELEM_FP16 && elem_kind != SYN_ELEM_FP32)
         return SYN_EINVAL;                                   // sums need a float type
     if (src_strides[ndim - 1] != 1 || dst_strides[ndim - 1] != 1) return SYN_EINVAL;   // rows are contiguous
@@ -296,27 +333,28 @@ int syn_box_copy_async(void* dst, const void* src, int32_t ndim, const int64_t* 
         }
     }
     int unit = (int)(mix & (~mix + 1));          // lowest set bit: 1, 2, 4, 8 or 16
-    if (sum && unit == 8) unit = 4;              // sums come in 16-byte groups, pairs/floats, single elements
+    // atomic sums go by 4-byte words (a pair of 16-bit elements, one float): the lanes of a
+    // wavefront then hit consecutive words, which the atomic units take 3.6 times faster than
+    // four words per lane (measured on a 134 MB box); a single 16-bit element where the box
+    // starts or ends on an odd one
+    if (atomic && unit > 4) unit = 4;
     p.row_units = row_bytes / unit;
     p.total_units = rows * p.row_units;
     const int64_t needed = (p.total_units + kBoxThreads - 1) / kBoxThreads;
     const int blocks = (int)(needed < num_blocks ? needed : num_blocks);
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-    // 32-bit index arithmetic is several times cheaper; below 2^29 units no index of the
-    // four-deep grid-stride loop can wrap (stride <= total + 1023)
-    const bool narrow = p.total_units < (int64_t)1 << 29;
+    // 32-bit index arithmetic is several times cheaper; below 2^27 units no index of the
+    // grid-stride loop (up to 16 deep, stride <= total + 1023) can wrap
+    const bool narrow = p.total_units < (int64_t)1 << 27;
     if (!sum) {
         if (narrow) launch_box_copy<uint32_t>(p, unit, blocks, s);
         else launch_box_copy<uint64_t>(p, unit, blocks, s);
     } else if (elem_kind == SYN_ELEM_BF16) {
-        if (narrow) launch_box_add<__bf16, uint32_t>(p, unit, blocks, s);
-        else launch_box_add<__bf16, uint64_t>(p, unit, blocks, s);
+        launch_box_add_any<__bf16>(p, unit, blocks, narrow, atomic, s);
     } else if (elem_kind == SYN_ELEM_FP16) {
-        if (narrow) launch_box_add<_Float16, uint32_t>(p, unit, blocks, s);
-        else launch_box_add<_Float16, uint64_t>(p, unit, blocks, s);
+        launch_box_add_any<_Float16>(p, unit, blocks, narrow, atomic, s);
     } else {
-        if (narrow) launch_box_add<float, uint32_t>(p, unit, blocks, s);
-        else launch_box_add<float, uint64_t>(p, unit, blocks, s);
+        launch_box_add_any<float>(p, unit, blocks, narrow, atomic, s);
     }
     return (int)hipGetLastError();
 }

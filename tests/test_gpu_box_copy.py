@@ -71,9 +71,10 @@ def _ulps(a, b, dtype):
     return (a.contiguous().view(bits).long() - b.contiguous().view(bits).long()).abs().max().item()
 
 
+@pytest.mark.parametrize("exclusive", [False, True])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("case", range(len(BOXES)))
-def test_sum_adds_once_in_the_element_type(hip, dtype, case):
+def test_sum_adds_once_in_the_element_type(hip, dtype, case, exclusive):
     from syncopate_amd.communication.comm_runtime.persistent_copy import persistent_tma_copy_last_contig
     from syncopate_amd.communication.descriptor import ReduceOp
 
@@ -88,13 +89,14 @@ def test_sum_adds_once_in_the_element_type(hip, dtype, case):
     s_view, d_view = sdev[ssl], ddev[dsl]
     if s_view.dim() != d_view.dim():
         d_view = d_view.reshape((1,) * (s_view.dim() - d_view.dim()) + tuple(d_view.shape))
-    persistent_tma_copy_last_contig(s_view, d_view, num_sms=16, reduce_op=ReduceOp.SUM)
+    persistent_tma_copy_last_contig(s_view, d_view, num_sms=16, reduce_op=ReduceOp.SUM, exclusive=exclusive)
     torch.cuda.synchronize()
     got = ddev.cpu()
     outside = torch.ones(dshape, dtype=torch.bool)
     outside[dsl] = False
     assert torch.equal(got[outside].view(torch.uint8), dst[outside].view(torch.uint8))
-    # normal numbers in, normal numbers out: the hardware's atomic add rounds like an add in the type
+    # normal numbers in, normal numbers out: the atomic units round like an add in the type,
+    # and so does the plain read-modify-write of the exclusive form
     assert _ulps(got[dsl], want[dsl], dtype) == 0
     torch.testing.assert_close(got.float(), want.float(), atol=1e-2, rtol=1e-2)
 

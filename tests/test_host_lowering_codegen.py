@@ -461,3 +461,32 @@ def test_attention_producer_tables_by_hand():
     assert t.signal_offsets == [0, 1]
     assert t.cum_wave_sizes == [3 * 2 * 256, 2 * 3 * 2 * 256]
     assert t.cum_tiles == 3 * 2 * 512
+
+
+def test_accumulating_box_copies_with_a_single_writer_are_found():
+    """Pull form of reduce-scatter by direct reduction: every sum into a rank's result sits in
+    that rank's own op list, so none needs atomics; push form: every rank adds into every
+    result, all of them do."""
+    from syncopate_amd.communication.comm_runtime.communication_context import CommContext
+    from syncopate_amd.communication.common_descriptors import build_reduce_scatter_direct_reduce_plan
+
+    world = 4
+    for kind, expect in (("pull", 16), ("push", 0)):
+        plans = {r: build_reduce_scatter_direct_reduce_plan(shape=(1024, 512), dtype=torch.float16, axis=0,
+                                                            mesh_size=world, rank=r, src_buffer="src",
+                                                            dst_buffer="dst", transfer_kind=kind)
+                 for r in range(world)}
+        gen = CommGenerator(plans)
+        gen.plan_signals()
+        info = gen.generate_code_for_plan(options=CodeGenOptions(copy_engine=False, use_tma=False))
+        ctx = CommContext.__new__(CommContext)        # the analysis needs no device
+        ctx.info = info
+        sole = ctx._find_sole_writer_ops()
+        boxes = [op for lists in info.operations for ops in lists for op in ops if isinstance(op, SMCopyOp)]
+        assert len(boxes) == 16 and len(sole) == expect
+        # two lists writing overlapping boxes of one destination: neither is a sole writer
+        if kind == "pull":
+            info.operations[0].append(list(info.operations[0][0]))
+            sole = ctx._find_sole_writer_ops()
+            assert not any(id(op) in sole for op in info.operations[0][0] if isinstance(op, SMCopyOp))
+            assert all(id(op) in sole for op in info.operations[1][0] if isinstance(op, SMCopyOp))
