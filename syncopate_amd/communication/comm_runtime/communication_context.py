@@ -28,7 +28,7 @@ from typing import Dict, List, Optional
 import torch
 
 from ... import _lib
-from ..descriptor import ReduceOp, SignalType
+from ..descriptor import CollectiveOp, ReduceOp, SignalType
 from .operations import (
     CollectiveComm,
     CommInfo,
@@ -199,7 +199,9 @@ class CommContext:
         (ring, double ring) only deliver this rank's data when the whole mesh is replayed; on one
         GPU that is one stream doing all the mesh's copies in turn.  Waits for another rank's
         COMPUTE_DONE flags are taken as satisfied (only this rank's compute kernel runs); this
-        rank's own are real waits on the flags its kernel writes."""
+        rank's own are real waits on the flags its kernel writes.  A library collective
+        (CollectiveComm) is carried out once for the mesh, at the point where every rank's list
+        has arrived at it."""
         if not self.streams:
             return
         stream = self.streams[0]
@@ -213,6 +215,12 @@ class CommContext:
             if r != self.rank and self.compute_signal_bufs:
                 self.compute_signal_bufs[r].fill_(1)
         remaining = sum(len(ops) for _, ops in lists)
+        # the k-th library collective of every list is one collective of the mesh: it is carried
+        # out once, when every list that has a k-th collective has arrived at it
+        nth = [0] * len(lists)                           # collectives passed, per list
+        counts = [sum(isinstance(op, CollectiveComm) for op in ops) for _, ops in lists]
+        arrived: Dict[int, Dict[int, CollectiveComm]] = {}
+        done_collectives = set()
         while remaining:
             progressed = False
             for idx, (owner, ops) in enumerate(lists):
@@ -221,6 +229,22 @@ class CommContext:
                     if isinstance(op, WaitIntraNodeSignal) and op.signal_type != SignalType.COMPUTE_DONE:
                         if (op.signal_type, op.rank % world, op.offset) not in written:
                             break            # its writer has not been enqueued yet
+                    if isinstance(op, CollectiveComm):
+                        k = nth[idx]
+                        if k not in done_collectives:
+                            here = arrived.setdefault(k, {})
+                            if owner not in here:
+                                here[owner] = op
+                                progressed = True
+                            if len(here) < sum(1 for c in counts if c > k):
+                                break        # the other ranks have not reached it yet
+                            self._mesh_collective(here, stream)
+                            done_collectives.add(k)
+                        nth[idx] += 1
+                        cursor[idx] += 1
+                        remaining -= 1
+                        progressed = True
+                        continue
                     self._issue(op, owner, stream, handle, neglect_local)
                     if isinstance(op, IntraNodeSignal):
                         written.add((op.signal_type, op.rank % world, op.offset))
@@ -230,6 +254,60 @@ class CommContext:
             if not progressed:
                 raise RuntimeError("the op lists wait for flags nobody writes: the plan cannot be replayed")
         self._zero_stale_set()
+
+    def _mesh_collective(self, per_rank: Dict[int, CollectiveComm], stream: torch.cuda.Stream) -> None:
+        """One library collective of the simulated mesh, carried out on `stream` over the ranks'
+        buffers of this process with the box copy / accumulate kernel (sums in rank order, one
+        rounding in the element type per addition, the way a ring adds them up).  The reference
+        hands these records to NCCL / NVSHMEM (communication_context.py:190-236), which needs one
+        process per rank; here they exist so that plans with collectives replay end to end."""
+        ranks = sorted(per_rank)
+        first = per_rank[ranks[0]]
+        for r in ranks:
+            o = per_rank[r]
+            if (o.op, o.src, o.dst, tuple(o.src_slice), tuple(o.dst_slice)) != \
+                    (first.op, first.src, first.dst, tuple(first.src_slice), tuple(first.dst_slice)):
+                raise ValueError(f"ranks disagree about a collective: {first} against {o}")
+        world = self.info.local_world_size
+        if ranks != list(range(world)):
+            raise ValueError(f"collective {first} is issued by ranks {ranks} of {world}")
+        units = self.info.num_copy_sms if self.info.num_copy_sms > 0 else 64
+        src_idx = tuple(slice(ax.start, ax.end) for ax in first.src_slice)
+        dst_idx = tuple(slice(ax.start, ax.end) for ax in first.dst_slice)
+        srcs = [self.comm_buffers[first.src][r][src_idx] for r in ranks]
+        dsts = [self.comm_buffers[first.dst][r][dst_idx] for r in ranks]
+
+        def total_into(out: torch.Tensor, parts: List[torch.Tensor]) -> None:
+            persistent_copy_last_contig(parts[0], out, num_sms=units, stream=stream)
+            for part in parts[1:]:
+                persistent_copy_last_contig(part, out, num_sms=units, reduce_op=ReduceOp.SUM, stream=stream,
+                                            exclusive=True)
+
+        if first.op == CollectiveOp.REDUCE_SCATTER:
+            # the scattered axis: the one where the source is `world` times the destination
+            axes = [a for a, (s, d) in enumerate(zip(srcs[0].shape, dsts[0].shape)) if s != d]
+            if len(axes) != 1 or srcs[0].shape[axes[0]] != world * dsts[0].shape[axes[0]]:
+                raise ValueError(f"{first}: source {tuple(srcs[0].shape)} is not {world} destination blocks "
+                                 f"{tuple(dsts[0].shape)} along one axis")
+            axis, width = axes[0], dsts[0].shape[axes[0]]
+            for q in ranks:
+                total_into(dsts[q], [s.narrow(axis, q * width, width) for s in srcs])
+        elif first.op == CollectiveOp.ALL_REDUCE:
+            if first.src != first.dst or src_idx != dst_idx:
+                raise ValueError("the in-place all-reduce needs one buffer and one slice for source and result")
+            with torch.cuda.stream(stream):
+                total = torch.empty(srcs[0].shape, dtype=srcs[0].dtype, device=self.device)
+            total_into(total, srcs)
+            for q in ranks:
+                persistent_copy_last_contig(total, dsts[q], num_sms=units, stream=stream)
+        elif first.op == CollectiveOp.ALL_REDUCE_NVSHARP:
+            if first.src == first.dst:
+                raise ValueError("the two-buffer all-reduce needs different source and result buffers")
+            total_into(dsts[0], srcs)
+            for q in ranks[1:]:
+                persistent_copy_last_contig(dsts[0], dsts[q], num_sms=units, stream=stream)
+        else:
+            raise NotImplementedError(f"collective {first.op} in the single-GPU executor")
 
     def _find_sole_writer_ops(self) -> set:
         """Accumulating box copies whose destination box nobody outside their own op list writes
@@ -320,8 +398,7 @@ class CommContext:
                                         exclusive=id(op) in self._sole_writer_ops)
         elif isinstance(op, CollectiveComm):
             raise NotImplementedError(
-                "library collectives need the other ranks to be real processes; "
-                "the single-GPU executor replays copy/flag op lists only")
+                "a library collective involves every rank: replay the whole mesh with execute_mesh()")
         else:
             raise TypeError(f"unknown op record {type(op).__name__}")
 

@@ -105,6 +105,25 @@ CASES = {
                                          dict(shape=(8192, 1024), dtype="bfloat16", src_buffer="src",
                                               dst_buffer="dst", src_split_axis=1, dst_split_axis=0, num_waves=4,
                                               transfer_kind="push", compute_producer=True), 8, [True]),
+    "rs_collective_split2_producer": ("build_reduce_scatter_collective_plan",
+                                      dict(shape=(64, 32), dtype="float16", axis=0, split_axis=1,
+                                           src_buffer="src", dst_buffer="dst", num_reduce_scatters=2,
+                                           compute_producer=True), 4, [True]),
+    "rs_collective_single_3d": ("build_reduce_scatter_collective_plan",
+                                dict(shape=(2, 8, 6), dtype="float32", axis=1, src_buffer="src",
+                                     dst_buffer="dst"), 4, [True]),
+    "rs_collective_rows_w8": ("build_reduce_scatter_collective_plan",
+                              dict(shape=(8192, 1024), dtype="bfloat16", axis=0, split_axis=-1,
+                                   src_buffer="src", dst_buffer="dst", num_reduce_scatters=4,
+                                   compute_producer=True), 8, [True]),
+    "ar_inplace_split4_producer": ("build_all_reduce_plan",
+                                   dict(shape=(8192, 1024), dtype="bfloat16", buffer_name="c", num_all_reduces=4,
+                                        split_axis=0, compute_producer=True), 8, [True]),
+    "ar_inplace_single": ("build_all_reduce_plan",
+                          dict(shape=(16, 8), dtype="float16", buffer_name="c"), 4, [True]),
+    "ar_two_buffers_split2_producer": ("build_all_reduce_nvsharp_plan",
+                                       dict(shape=(64, 32), dtype="float16", src_name="src", dst_name="dst",
+                                            num_all_reduces=2, split_axis=1, compute_producer=True), 4, [True]),
     "rs_direct_push": ("build_reduce_scatter_direct_reduce_plan",
                        dict(shape=(64, 32), dtype="float16", axis=0, src_buffer="src", dst_buffer="dst",
                             transfer_kind="push"), 4, [False]),

@@ -554,3 +554,92 @@ def test_gemm_rs_sm_reduce_iteration(hip, kind, rank):
             want = add_once(start[peer], partial[rank][peer * rows:(peer + 1) * rows], fragile)
             same(ctx.comm_buffers["dst"][peer].cpu(), want, fragile)
             assert ctx.recv_signal_bufs[peer].tolist() == [1 if i == rank else 0 for i in range(world)]
+
+
+@pytest.mark.parametrize("form", ["reduce_scatter", "all_reduce", "all_reduce_two_buffers"])
+def test_gemm_then_library_collective_whole_mesh(hip, form):
+    """Producer GEMM -> per slab: wait for its COMPUTE_DONE flag, one collective of the mesh, one
+    RECEIVE flag (tests/test_gemm_rs_collective.py:90-165, tests/test_gemm_ar_collective.py).  The
+    other ranks' partial products are computed beforehand; this rank's kernel runs beside the
+    replay of the mesh, which carries each collective out over the ranks' buffers."""
+    from syncopate_amd.communication.code_gen import CommGenerator
+    from syncopate_amd.communication.comm_runtime.communication_context import CommContext
+    from syncopate_amd.communication.common_descriptors import (
+        build_all_reduce_nvsharp_plan,
+        build_all_reduce_plan,
+        build_reduce_scatter_collective_plan,
+    )
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.gemm import gemm_producer
+    from syncopate_amd.interface import lower_comm_plan_to_raw_schedules
+    from syncopate_amd.interface.wave_tables import gemm_producer_tables
+
+    world, rank, M, N, K, BM, BN, programs, slabs = 4, 2, 1024, 512, 256, 128, 128, 24, 2
+    dtype = torch.bfloat16
+    if form == "reduce_scatter":
+        build = lambda r: build_reduce_scatter_collective_plan(
+            shape=(M, N), dtype=dtype, axis=0, split_axis=1, mesh_size=world, rank=r, src_buffer="src",
+            dst_buffer="dst", num_reduce_scatters=slabs, compute_producer=True)
+        produced, result = "src", "dst"
+    elif form == "all_reduce":
+        build = lambda r: build_all_reduce_plan(
+            shape=(M, N), dtype=dtype, mesh_size=world, rank=r, buffer_name="c", num_all_reduces=slabs,
+            split_axis=0, compute_producer=True)
+        produced, result = "c", "c"
+    else:
+        build = lambda r: build_all_reduce_nvsharp_plan(
+            shape=(M, N), dtype=dtype, mesh_size=world, rank=r, src_name="src", dst_name="dst",
+            num_all_reduces=slabs, split_axis=1, compute_producer=True)
+        produced, result = "src", "dst"
+    gen = CommGenerator({r: build(r) for r in range(world)})
+    gen.plan_signals()
+    schedules = lower_comm_plan_to_raw_schedules(gen)
+    info = gen.generate_code_for_plan()
+    info.local_world_size = info.world_size
+    ctx = CommContext(rank, info)
+    with pytest.raises(NotImplementedError):
+        ctx.execute()                       # one rank's list alone cannot carry out a collective
+
+    g = torch.Generator().manual_seed(31)
+    a = [(0.1 * torch.randn(M, K, generator=g)).to(dtype) for _ in range(world)]
+    b = [(0.1 * torch.randn(N, K, generator=g)).to(dtype) for _ in range(world)]
+    for r in range(world):
+        ctx.comm_buffers[produced][r].fill_(float("nan"))
+    ctx.reset_signals(whole_mesh=True)
+
+    def produce(r):
+        tables = gemm_producer_tables(schedules[r][produced])
+        shapes, offsets, signals = tables.block_shapes, tables.block_offsets, tables.signal_offsets
+        if form == "all_reduce":
+            # source and result in one buffer: the lowering puts the resident whole tensor in front
+            # as a wave without a flag, and the caller drops it (tests/test_gemm_ar_collective.py:120-122)
+            assert shapes[0] == [M, N] and signals[0] == -1
+            shapes, offsets, signals = shapes[1:], offsets[1:], signals[1:]
+        assert len(shapes) == slabs and sorted(signals) == list(range(slabs))
+        gemm_producer(a[r].cuda(), b[r].cuda(), ctx.comm_buffers[produced][r], ctx.compute_signal_bufs[r],
+                      shapes, offsets, signals, programs, BM, BN, 64, 8,
+                      cum_tiles=sum(h * w for h, w in shapes))
+
+    for r in range(world):
+        if r != rank:
+            produce(r)
+    ctx.start_after()
+    ctx.execute_mesh()
+    produce(rank)
+    ctx.end_before()
+    check_status()
+    ctx.check_status()
+
+    partial = [numerics.gemm_fp32(a[r], b[r]) for r in range(world)]
+    total = sum(p.double() for p in partial)
+    rows = M // world
+    for r in range(world):
+        got = ctx.comm_buffers[result][r].cpu()
+        want = total[r * rows:(r + 1) * rows] if form == "reduce_scatter" else total
+        assert got.shape == want.shape
+        # W roundings to 16 bits on top of the GEMMs'; the reference bounds the path by 1e-2 too
+        torch.testing.assert_close(got.double(), want, atol=2e-2, rtol=2e-2)
+        assert ctx.recv_signal_bufs[r].tolist() == [1] * slabs
+    if form != "all_reduce":
+        # the partial products were only read
+        assert _rel(ctx.comm_buffers["src"][rank], partial[rank]) <= REL_TOL

@@ -490,3 +490,109 @@ def test_accumulating_box_copies_with_a_single_writer_are_found():
             sole = ctx._find_sole_writer_ops()
             assert not any(id(op) in sole for op in info.operations[0][0] if isinstance(op, SMCopyOp))
             assert all(id(op) in sole for op in info.operations[1][0] if isinstance(op, SMCopyOp))
+
+
+# ---- library-collective plans (reference: tests/test_all_reduce_descriptor.py, tests/test_reduce_scatter_codegen.py)
+
+def _collective_info(builder, mesh, **kwargs):
+    gen = CommGenerator({r: builder(mesh_size=mesh, rank=r, **kwargs) for r in range(mesh)})
+    gen.plan_signals()
+    return gen, gen.generate_code_for_plan()
+
+
+def test_all_reduce_slabs_become_collective_then_flag():
+    from syncopate_amd.communication.comm_runtime.operations import CollectiveComm
+    from syncopate_amd.communication.common_descriptors import build_all_reduce_plan
+    from syncopate_amd.communication.descriptor import AxisSlice, CollectiveOp
+
+    _, info = _collective_info(build_all_reduce_plan, 2, shape=(4, 4), dtype=torch.float32, buffer_name="buf",
+                               num_all_reduces=2, split_axis=1)
+    assert info.world_size == 2 and info.recv_signal_num == 2
+    for rank in range(2):
+        (ops,) = info.operations[rank]
+        assert len(ops) == 4
+        for idx in range(2):
+            coll, flag = ops[2 * idx], ops[2 * idx + 1]
+            assert isinstance(coll, CollectiveComm) and coll.op == CollectiveOp.ALL_REDUCE
+            assert (coll.src, coll.dst) == ("buf", "buf")
+            want = (AxisSlice(0, 4), AxisSlice(2 * idx, 2 * idx + 2))
+            assert tuple(coll.src_slice) == want and tuple(coll.dst_slice) == want
+            assert isinstance(flag, IntraNodeSignal) and (flag.offset, flag.rank) == (idx, rank)
+
+    _, gated = _collective_info(build_all_reduce_plan, 2, shape=(4, 4), dtype=torch.float32, buffer_name="buf",
+                                compute_producer=True)
+    assert gated.compute_signal_num == 1
+    for rank in range(2):
+        wait, coll, flag = gated.operations[rank][0]
+        assert isinstance(wait, WaitIntraNodeSignal) and wait.signal_type == SignalType.COMPUTE_DONE
+        assert isinstance(coll, CollectiveComm) and isinstance(flag, IntraNodeSignal)
+
+
+def test_reduce_scatter_collective_slabs_and_destination_schedule():
+    from syncopate_amd.communication.comm_runtime.operations import CollectiveComm
+    from syncopate_amd.communication.common_descriptors import build_reduce_scatter_collective_plan
+    from syncopate_amd.communication.descriptor import AxisSlice, CollectiveOp
+
+    kw = dict(shape=(4, 4), dtype=torch.float32, axis=0, split_axis=1, src_buffer="src", dst_buffer="dst")
+    gen, info = _collective_info(build_reduce_scatter_collective_plan, 2, num_reduce_scatters=2, **kw)
+    assert info.world_size == 2 and info.recv_signal_num == 2
+    for rank in range(2):
+        (ops,) = info.operations[rank]
+        assert len(ops) == 4
+        for idx in range(2):
+            coll, flag = ops[2 * idx], ops[2 * idx + 1]
+            assert isinstance(coll, CollectiveComm) and coll.op == CollectiveOp.REDUCE_SCATTER
+            assert (coll.src, coll.dst) == ("src", "dst")
+            assert tuple(coll.src_slice) == (AxisSlice(0, 4), AxisSlice(2 * idx, 2 * idx + 2))
+            assert tuple(coll.dst_slice) == (AxisSlice(0, 2), AxisSlice(2 * idx, 2 * idx + 2))
+            assert isinstance(flag, IntraNodeSignal) and (flag.offset, flag.rank) == (idx, rank)
+    # the consumer of the result sees one wave per collective, one tile each
+    fresh = CommGenerator({r: build_reduce_scatter_collective_plan(mesh_size=2, rank=r, num_reduce_scatters=2, **kw)
+                           for r in range(2)})
+    fresh.plan_signals()
+    lowered = lower_comm_plan_to_raw_schedules(fresh)
+    for rank in range(2):
+        schedule = lowered[rank]["dst"]
+        assert schedule.global_shape == (2, 4) and schedule.num_waves == 2
+        assert all(len(wave) == 1 for wave in schedule.block_infos)
+
+    _, gated = _collective_info(build_reduce_scatter_collective_plan, 2, compute_producer=True, **kw)
+    assert gated.compute_signal_num == 1
+    for rank in range(2):
+        wait, coll, flag = gated.operations[rank][0]
+        assert isinstance(wait, WaitIntraNodeSignal) and wait.signal_type == SignalType.COMPUTE_DONE
+        assert isinstance(coll, CollectiveComm) and isinstance(flag, IntraNodeSignal)
+
+
+def test_collective_plan_argument_errors():
+    from syncopate_amd.communication.common_descriptors import (
+        build_all_reduce_nvsharp_plan,
+        build_all_reduce_plan,
+        build_reduce_scatter_collective_plan,
+    )
+
+    ar = dict(dtype=torch.float16, mesh_size=2, rank=0, buffer_name="b")
+    with pytest.raises(ValueError):
+        build_all_reduce_plan((4, 4), num_all_reduces=2, **ar)                  # which axis to cut?
+    with pytest.raises(ValueError):
+        build_all_reduce_plan((4, 6), num_all_reduces=4, split_axis=1, **ar)    # 6 % 4
+    with pytest.raises(IndexError):
+        build_all_reduce_plan((4, 4), num_all_reduces=2, split_axis=2, **ar)
+    with pytest.raises(ValueError):
+        build_all_reduce_plan((), **ar)
+    with pytest.raises(ValueError):
+        build_all_reduce_plan((4, 4), num_all_reduces=0, split_axis=0, **ar)
+    two = build_all_reduce_nvsharp_plan((4, 4), dtype=torch.float16, mesh_size=2, rank=1, src_name="s", dst_name="d",
+                                        num_all_reduces=2, split_axis=-1)
+    assert set(two.tensors_involved) == {"s", "d"} and not two.local_regions
+    rs = dict(dtype=torch.float16, mesh_size=2, rank=0, src_buffer="s", dst_buffer="d")
+    with pytest.raises(ValueError):
+        build_reduce_scatter_collective_plan((4, 4), axis=0, split_axis=0, **rs)     # cut along the scattered axis
+    with pytest.raises(ValueError):
+        build_reduce_scatter_collective_plan((4,), axis=0, **rs)                      # no other axis to cut
+    with pytest.raises(ValueError):
+        build_reduce_scatter_collective_plan((3, 4), axis=0, **rs)                    # 3 % 2
+    with pytest.raises(ValueError):
+        build_reduce_scatter_collective_plan((4, 4), axis=0, num_reduce_scatters=2, **rs)
+    plan = build_reduce_scatter_collective_plan((4, 4, 6), axis=2, **rs)              # default: wraps to axis 0
+    assert plan.tensors_involved["d"][0] == torch.Size((4, 4, 3))
