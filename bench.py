@@ -45,7 +45,7 @@ def _events(n):
     return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
 
 
-def build_ag_gemm(device, copy_blocks=0):
+def build_ag_gemm(device, copy_blocks=0, split_units=0):
     from syncopate_amd.communication.code_gen import CommGenerator
     from syncopate_amd.communication.comm_runtime.communication_context import CommContext
     from syncopate_amd.communication.common_descriptors import build_all_gather_plan_1d_swizzle
@@ -61,6 +61,10 @@ def build_ag_gemm(device, copy_blocks=0):
     info = gen.generate_code_for_plan()
     compile_ms = (time.perf_counter() - t0) * 1e3
     info.local_world_size = info.world_size
+    if split_units:
+        # the device split in two: `split_units` compute units for the producer's copy kernels, the
+        # consumer on the stream that owns the rest
+        info.need_green_ctx, info.num_copy_sms = True, split_units
     tables = gemm_consumer_tables(schedule, N)
 
     torch.manual_seed(0)
@@ -383,6 +387,9 @@ def main():
                          "streaming copy kernel with N workgroups")
     ap.add_argument("--tile", default=f"{BM}x{BN}", help="output tile of the consumer, e.g. 256x256 or 256x224")
     ap.add_argument("--programs", type=int, default=NUM_SMS, help="persistent programs of the consumer")
+    ap.add_argument("--split-device", type=int, default=0, metavar="N",
+                    help="give N compute units (a multiple of 8) to the producer's stream and the rest to the "
+                         "consumer's, by compute-unit masks")
     ap.add_argument("--lead-ops", type=int, default=LEAD_OPS,
                     help="the consumer launch waits for this many leading ops of the side stream (0: none)")
     args = ap.parse_args()
@@ -400,9 +407,14 @@ def main():
     device = torch.device("cuda", 0)
     torch.cuda.set_device(device)
 
-    state = build_ag_gemm(device, args.copy_blocks)
-    wall_ms, gated_ms, resident_ms = run_ag_gemm(state, args.steps, args.warmup, args.resident_only,
-                                                 not args.no_graph)
+    if args.split_device and (args.copy_blocks == 0 or not args.no_graph):
+        sys.exit("--split-device splits the compute units between two streams: it needs the copy kernel "
+                 "(--copy-blocks N) and launches from the host (--no-graph; a graph's kernel nodes carry no mask)")
+    state = build_ag_gemm(device, args.copy_blocks, args.split_device)
+    with torch.cuda.stream(state["ctx"].compute_stream):
+        wall_ms, gated_ms, resident_ms = run_ag_gemm(state, args.steps, args.warmup, args.resident_only,
+                                                     not args.no_graph)
+    torch.cuda.synchronize()
     traffic_calibration(device)
     err, gathered = check_ag_gemm(state)
     reduce_ms, reduce_bytes = run_reduce(device, max(args.steps, 30), args.warmup)
@@ -437,6 +449,7 @@ def main():
                                            f"copy kernel of {args.copy_blocks} workgroups")
                         + " + flag-set kernel per chunk",
             "launch": "eager" if args.no_graph else "one hip graph replay of all timed steps",
+            "split_device": state["ctx"].cu_split,
         },
         "pct_bf16_mfma_peak": 100.0 * value / MFMA_BF16_PEAK_TFLOPS,
         "flag_wait_overhead_pct": 100.0 * (gated_ms - resident_ms) / resident_ms,

@@ -276,6 +276,21 @@ int syn_flag_wait(const uint64_t* flag, uint64_t value, int64_t spin_timeout_us,
  * (models a slow link in front of a chunk copy). */
 int syn_delay_us(int64_t us, syn_stream_t stream);
 
+/* A stream whose kernels run only on the compute units whose bits are set in `mask` (`words`
+ * 32-bit words, bit i of the device: XCD i % 8, and within the XCD the compute units in turn over
+ * its shader engines), with a hardware queue of its own.  Two streams with disjoint masks split
+ * the device between communication and compute kernels: the counterpart of the reference's green
+ * contexts (comm_runtime/split_green_ctx.py:121-215, used when CommInfo.need_green_ctx is set,
+ * communication_context.py:66-72).  Destroy the stream with syn_stream_destroy when its work is
+ * done. */
+int syn_stream_create_cu_mask(const uint32_t* mask, uint32_t words, syn_stream_t* stream);
+int syn_stream_destroy(syn_stream_t stream);
+/* Launch `workgroups` workgroups that each record where they ran: out[2 b] = hardware id word
+ * (compute unit, shader array, shader engine in bits 8..15), out[2 b + 1] = XCD id, and stay for
+ * `dwell` short sleeps so that the grid spreads over every compute unit the stream may use.
+ * No counterpart in the reference; it is how a partition of the device is checked. */
+int syn_where_async(uint32_t* out, int32_t workgroups, int32_t dwell, syn_stream_t stream);
+
 /* Library/ABI version: major*10000 + minor*100 + patch. */
 int syn_version(void);
 

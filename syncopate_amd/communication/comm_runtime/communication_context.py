@@ -37,6 +37,7 @@ from .operations import (
     SMCopyOp,
     WaitIntraNodeSignal,
 )
+from .cu_partition import split_device_cu_mask
 from .persistent_copy import persistent_copy_last_contig
 from .streams import pick_side_streams
 
@@ -106,9 +107,22 @@ class CommContext:
         # one stream per op list, none of them on the hardware queue of the stream the compute
         # kernels are launched on (the current stream unless `compute_stream` names it): a flag
         # wait spinning on a shared queue would hold back the very kernel that sets the flag
-        self.compute_stream = (torch.cuda.current_stream(self.device) if compute_stream is None
-                               else compute_stream)
-        self.streams = pick_side_streams(len(info.operations[self.rank]), self.compute_stream, self.device)
+        if info.need_green_ctx:
+            # the device split in two (communication_context.py:66-72): `num_copy_sms` compute
+            # units (rounded up to a whole number per XCD) for the one communication stream, the
+            # rest for `self.compute_stream`, on which the caller launches its kernels
+            if len(info.operations[self.rank]) != 1:
+                raise ValueError("a split device carries one communication stream")
+            if info.num_copy_sms <= 0:
+                raise ValueError("a split device needs CommInfo.num_copy_sms compute units for communication")
+            (comm, rest), self.cu_split = split_device_cu_mask(self.device, 1, info.num_copy_sms)
+            self.streams = [comm]
+            self.compute_stream = rest
+        else:
+            self.cu_split = None
+            self.compute_stream = (torch.cuda.current_stream(self.device) if compute_stream is None
+                                   else compute_stream)
+            self.streams = pick_side_streams(len(info.operations[self.rank]), self.compute_stream, self.device)
 
     # ---- flags and stream ordering -------------------------------------------
 

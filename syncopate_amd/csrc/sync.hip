@@ -256,6 +256,21 @@ static void launch_box_add_any(const BoxParams& p, int unit, int blocks, bool na
     }
 }
 
+// Where did each workgroup run?  out[2 b] = the hardware id word of workgroup b's first
+// wavefront (compute unit, shader array and shader engine in bits 8..15), out[2 b + 1] = the id
+// of its XCD.  The workgroups stay for `dwell` short sleeps so that a grid spreads over every
+// compute unit its stream may use.
+__global__ void __launch_bounds__(256) where_kernel(uint32_t* out, int dwell) {
+    uint32_t hw, xcd;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw));
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcd));
+    for (int i = 0; i < dwell; ++i) __builtin_amdgcn_s_sleep(16);
+    if (threadIdx.x == 0) {
+        out[2 * blockIdx.x] = hw;
+        out[2 * blockIdx.x + 1] = xcd;
+    }
+}
+
 __global__ void __launch_bounds__(64) delay_kernel(int64_t ticks) {
     if (threadIdx.x == 0) {
         const uint64_t t0 = wall_clock64();
@@ -383,6 +398,30 @@ int syn_delay_us(int64_t us, syn_stream_t stream) {
         khz = 100000;
     hipLaunchKernelGGL(syn::delay_kernel, dim3(1), dim3(64), 0,
                        reinterpret_cast<hipStream_t>(stream), us * (int64_t)khz / 1000);
+    return (int)hipGetLastError();
+}
+
+int syn_stream_create_cu_mask(const uint32_t* mask, uint32_t words, syn_stream_t* stream) {
+    if (!mask || !stream || words == 0 || words > 32) return SYN_EINVAL;
+    uint32_t any = 0;
+    for (uint32_t i = 0; i < words; ++i) any |= mask[i];
+    if (!any) return SYN_EINVAL;                       // a stream without compute units never runs a kernel
+    hipStream_t s = nullptr;
+    const hipError_t err = hipExtStreamCreateWithCUMask(&s, words, mask);
+    if (err != hipSuccess) return (int)err;
+    *stream = reinterpret_cast<syn_stream_t>(s);
+    return 0;
+}
+
+int syn_stream_destroy(syn_stream_t stream) {
+    if (!stream) return SYN_EINVAL;
+    return (int)hipStreamDestroy(reinterpret_cast<hipStream_t>(stream));
+}
+
+int syn_where_async(uint32_t* out, int32_t workgroups, int32_t dwell, syn_stream_t stream) {
+    if (!out || workgroups <= 0 || workgroups > 65536 || dwell < 0 || dwell > 4096) return SYN_EINVAL;
+    hipLaunchKernelGGL(syn::where_kernel, dim3(workgroups), dim3(256), 0,
+                       reinterpret_cast<hipStream_t>(stream), out, dwell);
     return (int)hipGetLastError();
 }
 

@@ -465,8 +465,9 @@ def test_attention_to_all2all_iteration(hip, rank, dtype, causal):
             assert ctx.recv_signal_bufs[peer].sum().item() == 1
 
 
-@pytest.mark.parametrize("kind,rank", [("pull", 1), ("pull", 3), ("push", 2)])
-def test_gemm_rs_sm_reduce_iteration(hip, kind, rank):
+@pytest.mark.parametrize("kind,rank,split", [("pull", 1, False), ("pull", 3, False), ("push", 2, False),
+                                             ("pull", 0, True)])
+def test_gemm_rs_sm_reduce_iteration(hip, kind, rank, split):
     """Reduce-scatter by direct reduction with box copies on compute units
     (tests/test_gemm_rs_sm_reduce.py:95-175): every rank's producer GEMM writes its partial product
     and one COMPUTE_DONE flag per chunk; `pull`: this rank's side stream waits for each peer's
@@ -490,11 +491,19 @@ def test_gemm_rs_sm_reduce_iteration(hip, kind, rank):
     schedules = lower_comm_plan_to_raw_schedules(gen)
     info = gen.generate_code_for_plan(options=CodeGenOptions(copy_engine=False, use_tma=False))
     info.local_world_size = info.world_size
-    ctx = CommContext(rank, info)
-    with pytest.raises(ValueError):
-        ctx.execute()                     # box copies need compute units: num_copy_sms is still 0
-    torch.cuda.synchronize()
-    info.num_copy_sms = 10
+    if split:
+        # the device split in two like the reference's green contexts (tests/test_gemm_rs_collective.py:124-126):
+        # 16 compute units for the box copies, the GEMMs on the stream that owns the other 240
+        info.num_copy_sms, info.need_green_ctx, programs = 10, True, 240
+        ctx = CommContext(rank, info)
+        assert ctx.cu_split == [16, 240]
+    else:
+        ctx = CommContext(rank, info)
+        with pytest.raises(ValueError):
+            ctx.execute()                     # box copies need compute units: num_copy_sms is still 0
+        torch.cuda.synchronize()
+        info.num_copy_sms = 10
+    compute = ctx.compute_stream
 
     g = torch.Generator().manual_seed(23)
     a = [(0.1 * torch.randn(M, K, generator=g)).to(dtype) for _ in range(world)]
@@ -504,14 +513,18 @@ def test_gemm_rs_sm_reduce_iteration(hip, kind, rank):
         ctx.comm_buffers["src"][r].fill_(float("nan"))     # a chunk added before it was stored shows
         ctx.comm_buffers["dst"][r].copy_(start[r].cuda())
     ctx.reset_signals(whole_mesh=True)
+    operands = {r: (a[r].cuda(), b[r].cuda()) for r in range(world)}
+    compute.wait_stream(torch.cuda.current_stream())
     ctx.start_after()
     ctx.execute()                                          # the side stream waits for the flags
     runs = range(world) if kind == "pull" else [rank]
-    for r in runs:
-        tables = gemm_producer_tables(schedules[r]["src"])
-        gemm_producer(a[r].cuda(), b[r].cuda(), ctx.comm_buffers["src"][r], ctx.compute_signal_bufs[r],
-                      tables.block_shapes, tables.block_offsets, tables.signal_offsets, programs, BM, BN, 64, 8,
-                      cum_tiles=tables.cum_tiles)
+    with torch.cuda.stream(compute):
+        for r in runs:
+            tables = gemm_producer_tables(schedules[r]["src"])
+            gemm_producer(*operands[r], ctx.comm_buffers["src"][r], ctx.compute_signal_bufs[r],
+                          tables.block_shapes, tables.block_offsets, tables.signal_offsets, programs, BM, BN, 64, 8,
+                          cum_tiles=tables.cum_tiles)
+    torch.cuda.current_stream().wait_stream(compute)
     ctx.end_before()
     check_status()
     ctx.check_status()

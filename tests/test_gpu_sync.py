@@ -26,3 +26,39 @@ def test_side_streams_avoid_the_compute_streams_hardware_queue(hip):
     other = picked[0]
     for s in pick_side_streams(2, compute_stream=other):
         assert not shares_hardware_queue(s, other)
+
+
+def test_device_split_by_compute_unit_masks(hip):
+    """Streams on disjoint sets of compute units (the reference splits the device into green
+    contexts, comm_runtime/split_green_ctx.py:161-215): a grid on each stream stays inside its
+    set, the sets are disjoint, and every XCD gives the same number of units to the small group."""
+    from syncopate_amd.communication.comm_runtime.cu_partition import (
+        cu_mask_words,
+        group_sizes,
+        split_device_cu_mask,
+        where_workgroups_ran,
+    )
+
+    dev = torch.device("cuda", 0)
+    total = torch.cuda.get_device_properties(dev).multi_processor_count
+    everywhere = where_workgroups_ran(torch.cuda.current_stream())
+    assert len(everywhere) == total
+    streams, sizes = split_device_cu_mask(dev, 1, 20)
+    assert sizes == [24, total - 24] and len(streams) == 2
+    small, rest = (where_workgroups_ran(s) for s in streams)
+    assert len(small) == 24 and len(rest) == total - 24
+    assert not (small & rest) and (small | rest) == everywhere
+    per_xcd = {}
+    for xcd, _ in small:
+        per_xcd[xcd] = per_xcd.get(xcd, 0) + 1
+    assert sorted(per_xcd.values()) == [3] * 8
+    # kernels on the two streams run side by side and both finish
+    a, b = (torch.zeros(1 << 20, device=dev) for _ in range(2))
+    for s, t in zip(streams, (a, b)):
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            t.add_(1.0)
+    torch.cuda.synchronize()
+    assert a.sum().item() == b.sum().item() == float(1 << 20)
+    assert cu_mask_words(8, 24, 64) == [0xFFFFFF00, 0]
+    assert group_sizes(256, 2, 9) == [16, 16, 224]

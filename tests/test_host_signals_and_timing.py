@@ -200,3 +200,20 @@ def test_plan_pretty_with_signals():
         "    Stream 0:",
         "      op[0] pull -> signals: receive_data@1[0]",
     ])
+
+
+def test_compute_unit_groups_and_mask_words():
+    from syncopate_amd.communication.comm_runtime.cu_partition import cu_mask_words, group_sizes
+
+    assert group_sizes(256, 1, 10) == [16, 240]          # a whole number of units per XCD
+    assert group_sizes(256, 1, 32) == [32, 224]
+    assert group_sizes(256, 3, 8) == [8, 8, 8, 232]
+    with pytest.raises(RuntimeError):
+        group_sizes(256, 1, 250)                         # nothing would be left for compute
+    with pytest.raises(ValueError):
+        group_sizes(256, 0, 8)
+    assert cu_mask_words(0, 32, 256) == [0xFFFFFFFF] + [0] * 7
+    assert cu_mask_words(32, 224, 256) == [0] + [0xFFFFFFFF] * 7
+    assert cu_mask_words(30, 4, 64) == [0xC0000000, 0x3]
+    with pytest.raises(ValueError):
+        cu_mask_words(250, 10, 256)
