@@ -45,7 +45,7 @@ def _events(n):
     return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
 
 
-def build_ag_gemm(device, copy_blocks=0, split_units=0):
+def build_ag_gemm(device, copy_blocks=0, split_units=0, fuse_flags=False):
     from syncopate_amd.communication.code_gen import CommGenerator
     from syncopate_amd.communication.comm_runtime.communication_context import CommContext
     from syncopate_amd.communication.common_descriptors import build_all_gather_plan_1d_swizzle
@@ -71,7 +71,7 @@ def build_ag_gemm(device, copy_blocks=0, split_units=0):
     a = (0.02 * torch.randn(M, K, device=device)).bfloat16()
     b = (0.02 * torch.randn(N, K, device=device)).bfloat16()
     # two flag sets: the reset of one iteration's flags happens behind the next one's copies
-    ctx = CommContext(RANK, info, device=device, copy_blocks=copy_blocks, flag_sets=2)
+    ctx = CommContext(RANK, info, device=device, copy_blocks=copy_blocks, flag_sets=2, fuse_flags=fuse_flags)
     rows = M // WORLD
     for r in range(WORLD):     # every rank's symmetric buffer holds its own shard
         ctx.comm_buffers["a"][r][r * rows:(r + 1) * rows].copy_(a[r * rows:(r + 1) * rows])
@@ -387,6 +387,8 @@ def main():
                          "streaming copy kernel with N workgroups")
     ap.add_argument("--tile", default=f"{BM}x{BN}", help="output tile of the consumer, e.g. 256x256 or 256x224")
     ap.add_argument("--programs", type=int, default=NUM_SMS, help="persistent programs of the consumer")
+    ap.add_argument("--fuse-flags", action="store_true",
+                    help="with --copy-blocks N: one kernel per chunk that copies and then sets the flag")
     ap.add_argument("--split-device", type=int, default=0, metavar="N",
                     help="give N compute units (a multiple of 8) to the producer's stream and the rest to the "
                          "consumer's, by compute-unit masks")
@@ -410,7 +412,7 @@ def main():
     if args.split_device and (args.copy_blocks == 0 or not args.no_graph):
         sys.exit("--split-device splits the compute units between two streams: it needs the copy kernel "
                  "(--copy-blocks N) and launches from the host (--no-graph; a graph's kernel nodes carry no mask)")
-    state = build_ag_gemm(device, args.copy_blocks, args.split_device)
+    state = build_ag_gemm(device, args.copy_blocks, args.split_device, args.fuse_flags)
     with torch.cuda.stream(state["ctx"].compute_stream):
         wall_ms, gated_ms, resident_ms = run_ag_gemm(state, args.steps, args.warmup, args.resident_only,
                                                      not args.no_graph)
@@ -445,9 +447,11 @@ def main():
                         "fp32 accumulate",
             "tile": [BM, BN, BK],
             "programs": NUM_SMS,
-            "producer": "side stream: " + ("hipMemcpyAsync" if args.copy_blocks == 0 else
-                                           f"copy kernel of {args.copy_blocks} workgroups")
-                        + " + flag-set kernel per chunk",
+            "producer": "side stream: " + (
+                f"one kernel of {args.copy_blocks} workgroups per chunk that copies, then sets the flag"
+                if args.fuse_flags else
+                ("hipMemcpyAsync" if args.copy_blocks == 0 else f"copy kernel of {args.copy_blocks} workgroups")
+                + " + flag-set kernel per chunk"),
             "launch": "eager" if args.no_graph else "one hip graph replay of all timed steps",
             "split_device": state["ctx"].cu_split,
         },

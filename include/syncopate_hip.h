@@ -252,6 +252,14 @@ int syn_copy_kernel_async(void* dst, const void* src, int64_t nbytes, int32_t nu
 #define SYN_ELEM_2B 4
 #define SYN_ELEM_4B 5
 #define SYN_ELEM_8B 6
+/* A chunk copy that sets the chunk's flag itself (`*flag = value` once every byte has landed):
+ * one kernel where the reference issues a copy and a stream write
+ * (communication_context.py:129-150), with at most `num_blocks` workgroups of 1024 threads.
+ * `ticket` is one zeroed 32-bit word of device memory that the copies of ONE stream share: the
+ * kernel counts its workgroups in it and leaves it zero again.  16-byte alignment as for
+ * syn_copy_kernel_async. */
+int syn_copy_flag_async(void* dst, const void* src, int64_t nbytes, uint64_t* flag, uint64_t value,
+                        uint32_t* ticket, int32_t num_blocks, syn_stream_t stream);
 /* What syn_box_copy_async does with the destination */
 #define SYN_BOX_COPY 0            /* dst = src */
 #define SYN_BOX_ADD_ATOMIC 1      /* dst += src by atomic adds: several senders may add into one

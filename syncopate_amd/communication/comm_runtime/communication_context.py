@@ -56,7 +56,7 @@ class CommContext:
     def __init__(self, rank: int, info: CommInfo, multi_info: bool = False, *,
                  device: Optional[torch.device] = None, link_delay_us: int = 0,
                  wait_timeout_us: int = 2_000_000, copy_blocks: int = 0, flag_sets: int = 1,
-                 compute_stream: Optional[torch.cuda.Stream] = None) -> None:
+                 compute_stream: Optional[torch.cuda.Stream] = None, fuse_flags: bool = False) -> None:
         if info.local_world_size <= 0:
             info.local_world_size = info.world_size
         if info.local_world_size != info.world_size:
@@ -74,6 +74,11 @@ class CommContext:
         # 0: contiguous copies go through hipMemcpyAsync; > 0: through a streaming copy kernel of
         # that many 256-thread workgroups (16-byte aligned copies only)
         self.copy_blocks = int(copy_blocks)
+        # with copy_blocks > 0: a copy that is followed by its flag write in the op list becomes
+        # ONE kernel that copies and then sets the flag (execute() only)
+        self.fuse_flags = bool(fuse_flags)
+        if self.fuse_flags and self.copy_blocks <= 0:
+            raise ValueError("fuse_flags needs the copy kernel: copy_blocks > 0")
         self._lib = _lib.load()
         world = info.local_world_size
 
@@ -104,6 +109,8 @@ class CommContext:
         }
         self.status = torch.zeros(_lib.SYN_STATUS_WORDS, dtype=torch.int32, device=self.device)
         self._sole_writer_ops = self._find_sole_writer_ops()
+        # one workgroup counter per communication stream for the fused copy + flag kernel
+        self._tickets = torch.zeros(max(1, len(info.operations[self.rank])), dtype=torch.int32, device=self.device)
         # one stream per op list, none of them on the hardware queue of the stream the compute
         # kernels are launched on (the current stream unless `compute_stream` names it): a flag
         # wait spinning on a shared queue would hold back the very kernel that sets the flag
@@ -190,14 +197,23 @@ class CommContext:
         takes the compute units, and every chunk of the iteration arrives later."""
         self._lead_events = []
         self._check_copy_units(self.info.operations[self.rank])
-        for stream, ops in zip(self.streams, self.info.operations[self.rank]):
+        for lane, (stream, ops) in enumerate(zip(self.streams, self.info.operations[self.rank])):
             handle = int(stream.cuda_stream)
-            for index, op in enumerate(ops):
-                self._issue(op, self.rank, stream, handle, neglect_local)
-                if lead_ops > 0 and index + 1 == min(lead_ops, len(ops)):
+            lead = min(lead_ops, len(ops))
+            index = 0
+            while index < len(ops):
+                op, done = ops[index], 1
+                if (self.fuse_flags and isinstance(op, CopyEngineOp) and index + 1 < len(ops)
+                        and isinstance(ops[index + 1], IntraNodeSignal)
+                        and self._issue_copy_with_flag(op, ops[index + 1], lane, handle, neglect_local)):
+                    done = 2
+                else:
+                    self._issue(op, self.rank, stream, handle, neglect_local)
+                if lead_ops > 0 and index < lead <= index + done:
                     event = torch.cuda.Event()
                     event.record(stream)
                     self._lead_events.append(event)
+                index += done
         self._zero_stale_set()
 
     def wait_lead(self, stream: Optional[torch.cuda.Stream] = None) -> None:
@@ -357,6 +373,34 @@ class CommContext:
         # before anything is enqueued (communication_context.py:164 asserts it per op)
         if self.info.num_copy_sms <= 0 and any(isinstance(op, SMCopyOp) for ops in op_lists for op in ops):
             raise ValueError("box copies run on compute units: set CommInfo.num_copy_sms first")
+
+    def _issue_copy_with_flag(self, op: CopyEngineOp, flag_op: IntraNodeSignal, lane: int, handle: int,
+                              neglect_local: bool) -> bool:
+        """A copy and the flag write behind it as one kernel; False if the pair does not qualify
+        (then both are issued on their own)."""
+        world = self.info.local_world_size
+        if op.src_rank == op.dst_rank and neglect_local:
+            return False
+        if flag_op.signal_type != SignalType.RECEIVE_DATA:
+            return False
+        src = self.comm_buffers[op.src][op.src_rank % world]
+        dst = self.comm_buffers[op.dst][op.dst_rank % world]
+        if op.src_offset + op.size > src.numel() * src.element_size() or \
+                op.dst_offset + op.size > dst.numel() * dst.element_size():
+            raise ValueError(f"{op} runs past the end of its buffer")
+        dst_ptr, src_ptr = dst.data_ptr() + op.dst_offset, src.data_ptr() + op.src_offset
+        if op.size <= 0 or op.size % 16 or dst_ptr % 16 or src_ptr % 16:
+            return False
+        flags = self.recv_signal_bufs[flag_op.rank % world]
+        if not 0 <= flag_op.offset < flags.numel():
+            raise ValueError(f"{flag_op} is outside the flag array")
+        lib = self._lib
+        if self.link_delay_us and op.src_rank != op.dst_rank:
+            _lib.check("syn_delay_us", lib.syn_delay_us(self.link_delay_us, handle))
+        _lib.check("syn_copy_flag_async",
+                   lib.syn_copy_flag_async(dst_ptr, src_ptr, op.size, flags.data_ptr() + 8 * flag_op.offset, 1,
+                                           self._tickets.data_ptr() + 4 * lane, self.copy_blocks, handle))
+        return True
 
     def _issue(self, op, owner: int, stream: torch.cuda.Stream, handle: int, neglect_local: bool) -> None:
         """Enqueue one op of rank `owner`'s list on `stream`."""

@@ -242,8 +242,8 @@ def test_copy_kernel_producer_matches_copy_engine(hip):
     g = torch.Generator().manual_seed(2)
     a = torch.randn(M, K, generator=g).half()
     rows = M // world
-    for blocks in (0, 8):
-        ctx = CommContext(rank, info, copy_blocks=blocks)
+    for blocks, fused in ((0, False), (8, False), (8, True), (3, True)):
+        ctx = CommContext(rank, info, copy_blocks=blocks, fuse_flags=fused)
         for r in range(world):
             ctx.comm_buffers["a"][r][r * rows:(r + 1) * rows].copy_(a[r * rows:(r + 1) * rows])
         ctx.reset_signals()
@@ -253,6 +253,53 @@ def test_copy_kernel_producer_matches_copy_engine(hip):
         ctx.check_status()
         assert torch.equal(ctx.comm_buffers["a"][rank].cpu(), a)
         assert ctx.recv_signal_bufs[rank].tolist() == [1] * (world - 1)
+        assert ctx._tickets.tolist() == [0]          # the fused kernel leaves its workgroup counter at zero
+    with pytest.raises(ValueError):
+        CommContext(rank, info, fuse_flags=True)     # needs the copy kernel
+
+
+def test_fused_copy_and_flag_gates_the_consumer(hip):
+    """The consumer GEMM polls flags that the fused copy + flag kernels of a side stream set: a
+    flag seen means the chunk's bytes are there (NaN poison otherwise), over several iterations."""
+    from syncopate_amd.communication.comm_runtime.communication_context import CommContext
+    from syncopate_amd.communication.common_descriptors import build_all_gather_plan_1d_swizzle
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.gemm import gemm_consumer
+    from syncopate_amd.interface.wave_tables import gemm_consumer_tables
+
+    world, rank, M, N, K, BM, BN = 8, 5, 4096, 1024, 1024, 128, 256
+    plans = {r: build_all_gather_plan_1d_swizzle((M, K), torch.bfloat16, 0, world, r, "a", "pull")
+             for r in range(world)}
+    schedules, info = _compile(plans)
+    tables = gemm_consumer_tables(schedules[rank]["a"], N)
+    g = torch.Generator().manual_seed(8)
+    a = (0.05 * torch.randn(M, K, generator=g)).bfloat16()
+    b = (0.05 * torch.randn(N, K, generator=g)).bfloat16().cuda()
+    ref = numerics.gemm_fp32(a, b.cpu())
+    rows = M // world
+    ctx = CommContext(rank, info, copy_blocks=24, fuse_flags=True, flag_sets=2, link_delay_us=30)
+    for r in range(world):
+        ctx.comm_buffers["a"][r][r * rows:(r + 1) * rows].copy_(a[r * rows:(r + 1) * rows])
+    symm = ctx.comm_buffers["a"][rank]
+    c = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    first = None
+    for it in range(3):
+        for r in range(world):
+            if r != rank:
+                symm[r * rows:(r + 1) * rows].fill_(float("nan"))
+        c.zero_()
+        ctx.reset_signals()
+        ctx.start_after()
+        gemm_consumer(symm, b, c, ctx.recv_signal_bufs[rank], tables.block_shapes, tables.block_offsets,
+                      tables.signal_offsets, world, 200, BM, BN, cum_tiles=tables.cum_tiles)
+        ctx.execute()
+        ctx.end_before()
+        check_status()
+        ctx.check_status()
+        assert torch.equal(symm.cpu(), a)
+        assert _rel(c, ref) <= REL_TOL
+        first = c.clone() if first is None else first
+        assert torch.equal(c, first)
 
 
 def test_copy_kernel_rejects_misaligned(hip):
@@ -263,6 +310,12 @@ def test_copy_kernel_rejects_misaligned(hip):
     assert hip.syn_copy_kernel_async(buf.data_ptr() + 8, buf.data_ptr() + 128, 64, 4, s) == _lib.SYN_EALIGN
     assert hip.syn_copy_kernel_async(buf.data_ptr(), buf.data_ptr() + 128, 60, 4, s) == _lib.SYN_EALIGN
     assert hip.syn_copy_kernel_async(buf.data_ptr(), buf.data_ptr() + 128, 64, 0, s) == _lib.SYN_EINVAL
+    words = torch.zeros(4, dtype=torch.int64, device="cuda")
+    flag, ticket = words.data_ptr(), words.data_ptr() + 8
+    assert hip.syn_copy_flag_async(buf.data_ptr() + 8, buf.data_ptr() + 128, 64, flag, 1, ticket, 4, s) == _lib.SYN_EALIGN
+    assert hip.syn_copy_flag_async(buf.data_ptr(), buf.data_ptr() + 128, 64, None, 1, ticket, 4, s) == _lib.SYN_EINVAL
+    assert hip.syn_copy_flag_async(buf.data_ptr(), buf.data_ptr() + 128, 0, flag, 1, ticket, 4, s) == _lib.SYN_EINVAL
+    assert words.tolist() == [0, 0, 0, 0]
     torch.cuda.synchronize()
 
 
