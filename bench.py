@@ -37,6 +37,7 @@ M, K, N, WORLD, RANK = 8192, 8192, 3584, 8, 0
 BM, BN, BK, GROUP_M = 256, 256, 64, 8
 NUM_SMS = 224                        # 448 tiles = 2 per program; 32 of the 256 CUs stay free for the
                                      # copy kernels of the producer
+XCD_REMAP = False                    # consecutive tile ids on one XCD (see --xcd-remap)
 LEAD_OPS = 1                         # ops of the side stream the consumer launch waits for (see fused_step)
 EIGHT_WAVES = False                  # 256-thread workgroups: one wavefront per SIMD, 128x128 of C each
 
@@ -94,7 +95,7 @@ def run_ag_gemm(state, steps, warmup, resident_only=False, use_graph=True):
     stream = torch.cuda.current_stream()
 
     def consumer(flag_words):
-        gemm(symm, b, c, WORLD, NUM_SMS, BM, BN, BK, GROUP_M, signal_ptr=flag_words, xcd_remap=False,
+        gemm(symm, b, c, WORLD, NUM_SMS, BM, BN, BK, GROUP_M, signal_ptr=flag_words, xcd_remap=XCD_REMAP,
              eight_waves=EIGHT_WAVES, **tables)
 
     def fused_step():
@@ -371,7 +372,7 @@ def cpu_baseline(state):
 
 
 def main():
-    global BM, BN, NUM_SMS, LEAD_OPS
+    global BM, BN, NUM_SMS, LEAD_OPS, XCD_REMAP
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
@@ -387,6 +388,8 @@ def main():
                          "streaming copy kernel with N workgroups")
     ap.add_argument("--tile", default=f"{BM}x{BN}", help="output tile of the consumer, e.g. 256x256 or 256x224")
     ap.add_argument("--programs", type=int, default=NUM_SMS, help="persistent programs of the consumer")
+    ap.add_argument("--xcd-remap", action="store_true",
+                    help="each XCD works on a contiguous range of tile ids (one chunk's tiles at a time)")
     ap.add_argument("--fuse-flags", action="store_true",
                     help="with --copy-blocks N: one kernel per chunk that copies and then sets the flag")
     ap.add_argument("--split-device", type=int, default=0, metavar="N",
@@ -406,6 +409,7 @@ def main():
     BM, BN = (int(x) for x in args.tile.lower().split("x"))
     NUM_SMS = args.programs
     LEAD_OPS = args.lead_ops
+    XCD_REMAP = args.xcd_remap
     device = torch.device("cuda", 0)
     torch.cuda.set_device(device)
 
