@@ -273,7 +273,8 @@ def run_box_copies(device, steps, warmup):
 
 def run_attention(device, steps, warmup):
     """All-gather attention at the headline ring / all-gather configuration: 4096 local q rows, 32 heads, against 32768
-    kv rows as 8 chunks of 4096 in double-ring arrival order (every chunk resident), head dim 128."""
+    kv rows as 8 chunks of 4096 in double-ring arrival order (every chunk resident), head dim 128; two q
+    blocks per workgroup in opposite phases (pair_q_blocks)."""
     from syncopate_amd.computation._launch import check_status
     from syncopate_amd.computation.attn import attention_forward
 
@@ -291,12 +292,12 @@ def run_attention(device, steps, warmup):
                   signal_ptr=torch.ones(chunks, dtype=torch.int64, device=device))
     out = torch.empty_like(q)
     for _ in range(warmup):
-        attention_forward(q, k, v, D ** -0.5, out=out, **tables)
+        attention_forward(q, k, v, D ** -0.5, out=out, pair_q_blocks=True, **tables)
     torch.cuda.synchronize()
     begin, end = _events(1)[0], _events(1)[0]
     begin.record()
     for _ in range(steps):
-        attention_forward(q, k, v, D ** -0.5, out=out, **tables)
+        attention_forward(q, k, v, D ** -0.5, out=out, pair_q_blocks=True, **tables)
     end.record()
     torch.cuda.synchronize()
     check_status()

@@ -37,6 +37,8 @@ extern "C" {
 #define SYN_STATUS_WORDS 4
 #define SYN_STATUS_OK 0
 #define SYN_STATUS_SPIN_TIMEOUT 1   /* [1]=wave index, [2]=program id, [3]=signal offset */
+#define SYN_STATUS_BAD_PAIRING 2    /* SYN_ATTN_PAIR_Q_BLOCKS on a wave with an odd number of q blocks:
+                                       [1]=wave index, [2]=program id, [3]=q blocks of the wave */
 
 /* gemm option bits */
 #define SYN_GEMM_XCD_REMAP 1u       /* permute hardware workgroup ids so that consecutive
@@ -221,8 +223,20 @@ typedef struct syn_attn_desc {
                                        880-901, 1125-1137): no flag is waited for; every finished
                                        tile bumps counters[wave] and the tile that completes a wave
                                        (Z*H*Q blocks of it) sets flags[signal_offsets[wave]] to 1   */
+    int32_t options;                /* SYN_ATTN_* bits                                                */
 } syn_attn_desc;
 
+/* syn_attn_desc.options: one workgroup of eight wavefronts takes two consecutive q blocks (tiles
+ * 2i and 2i + 1) and runs them half a kv block apart, so that the softmax of one overlaps the
+ * matrix products of the other and both read K and V from the same LDS blocks.  No counterpart in
+ * the reference (one program per tile there); results and merge protocol are the same.  The
+ * caller vouches that every wave holds an even number of q blocks; not with `causal` or
+ * `counters`. */
+#define SYN_ATTN_PAIR_Q_BLOCKS 1u
+/* workgroup b takes tile (b % 8) * (grid / 8) + b / 8 instead of tile b: the workgroups of one XCD
+ * then work on consecutive tiles - the q blocks of one head - and that head's K and V pass through
+ * one L2 instead of eight.  The visit log records the program each tile ran on either way. */
+#define SYN_ATTN_XCD_REMAP 2u
 int syn_attn_fwd(const syn_attn_desc* desc, syn_stream_t stream);
 
 /* Host-only check of an attention wave table (HOST pointers). */

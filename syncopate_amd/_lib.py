@@ -28,6 +28,9 @@ SYN_GEMM_EIGHT_WAVES = 2
 SYN_GEMM_RING_PIPE = 4
 SYN_GEMM_NO_K_STAGGER = 8
 SYN_GEMM_TWO_STAGE = 16
+SYN_ATTN_PAIR_Q_BLOCKS = 1
+SYN_ATTN_XCD_REMAP = 2
+SYN_STATUS_BAD_PAIRING = 2
 SYN_BOX_COPY, SYN_BOX_ADD_ATOMIC, SYN_BOX_ADD_EXCLUSIVE = range(3)
 SYN_ELEM_BF16, SYN_ELEM_FP16, SYN_ELEM_FP32, SYN_ELEM_1B, SYN_ELEM_2B, SYN_ELEM_4B, SYN_ELEM_8B = range(7)
 
@@ -121,6 +124,7 @@ class AttnDesc(ctypes.Structure):
         ("v_strides", c_int64 * 3),
         ("o_strides", c_int64 * 3),
         ("counters", c_void_p),
+        ("options", c_int32),
     ]
 
 

@@ -61,6 +61,8 @@ def attention_forward(
     num_programs: int = 0,
     counter_ptr: Optional[torch.Tensor] = None,
     output_buffer: Optional[torch.Tensor] = None,
+    pair_q_blocks: bool = False,
+    xcd_remap: bool = False,
     out: Optional[torch.Tensor] = None,
     return_lse: bool = False,
     visit_log: Optional[torch.Tensor] = None,
@@ -79,6 +81,12 @@ def attention_forward(
     bumps its wave's counter and the tile that completes a wave sets the wave's flag in
     `signal_ptr`.  `output_buffer` (alias of `out`) is the reference's name for the comm buffer
     the result is written into.
+    `pair_q_blocks` (an extension): one workgroup of eight wavefronts takes two consecutive q
+    blocks and runs them half a kv block apart, the softmax of one beside the matrix products of
+    the other, both reading K and V from the same LDS blocks.  Every wave must hold an even
+    number of q blocks; not with `causal` or `counter_ptr`.
+    `xcd_remap` (an extension): the workgroups of one XCD take consecutive tiles (the q blocks of
+    one head), so that a head's K and V are fetched into one L2 instead of eight.
     """
     dev = require_cuda(q, k, v, signal_ptr)
     if not (q.dtype == k.dtype == v.dtype):
@@ -116,18 +124,22 @@ def attention_forward(
     tables = (wave_offsets, wave_sizes, cum_wave_sizes, signal_offsets)   # the caller's objects
     caller_owned = all(isinstance(t, torch.Tensor) and t.is_cuda
                        for t in (wave_offsets, wave_sizes, cum_wave_sizes, signal_offsets))
-    params = (num_waves, Z, H, Sq, Skv, cum_tiles, flags.numel())
+    if pair_q_blocks and (causal or counter_ptr is not None):
+        raise ValueError("pair_q_blocks goes with neither causal nor counter_ptr")
+    params = (num_waves, Z, H, Sq, Skv, cum_tiles, flags.numel(), bool(pair_q_blocks))
     if cum_tiles is None or not (caller_owned and already_checked(tables, params)):
         ho, hs, hc, hg = host_copy(offs), host_copy(sizes), host_copy(cums), host_copy(sigs)
         if cum_tiles is None:
             cum_tiles = int(hc[:num_waves].max().item())
+        if pair_q_blocks and any(int(hs[i, 2]) % (2 * BLOCK_M) for i in range(num_waves) if int(hc[i]) > 0):
+            raise ValueError("pair_q_blocks needs an even number of q blocks in every wave")
         _lib.check(
             "syn_attn_check_waves",
             lib.syn_attn_check_waves(host_ptr(ho), host_ptr(hs), host_ptr(hc), host_ptr(hg), num_waves,
                                      Z, H, Sq, Skv, BLOCK_M, BLOCK_N, int(cum_tiles), flags.numel()),
         )
         if caller_owned:
-            remember_checked(tables, (num_waves, Z, H, Sq, Skv, cum_tiles, flags.numel()))
+            remember_checked(tables, (num_waves, Z, H, Sq, Skv, cum_tiles, flags.numel(), bool(pair_q_blocks)))
 
     if output_buffer is not None:
         if out is not None and out is not output_buffer:
@@ -161,6 +173,7 @@ def attention_forward(
         sm_scale=float(sm_scale), cum_tiles=int(cum_tiles), spin_timeout_us=int(spin_timeout_us),
         q_strides=strides(q), k_strides=strides(k), v_strides=strides(v), o_strides=strides(o),
         counters=None if counter_ptr is None else counter_ptr.data_ptr(),
+        options=(_lib.SYN_ATTN_PAIR_Q_BLOCKS if pair_q_blocks else 0) | (_lib.SYN_ATTN_XCD_REMAP if xcd_remap else 0),
     )
     with torch.cuda.device(dev):
         _lib.check("syn_attn_fwd", lib.syn_attn_fwd(ctypes.byref(desc), _lib.stream_handle(stream)))

@@ -53,6 +53,7 @@ struct AttnParams {
     int32_t Z, H, Sq, Skv;
     int32_t causal;
     int32_t num_tiles;
+    int32_t xcd_remap;    // workgroups of one XCD take consecutive tiles (see logical_program_id)
     float qk_scale;       // sm_scale * 1.44269504 (template.py:178-179)
     // element strides {batch, head, row}
     int64_t q_st[3], k_st[3], v_st[3], o_st[3];
@@ -168,7 +169,11 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
     const unsigned char* __restrict__ V = reinterpret_cast<const unsigned char*>(p.v);
     T* __restrict__ O = reinterpret_cast<T*>(p.o);
 
-    for (int tile_id = blockIdx.x; tile_id < p.num_tiles; tile_id += gridDim.x) {
+    // Workgroups are dealt to the 8 XCDs in turn.  Consecutive tiles are the q blocks of one head and
+    // read the same K and V: with the remap an XCD's workgroups take consecutive tiles, so a head's
+    // K and V pass through one L2 instead of eight.
+    const int first_tile = logical_program_id((int)blockIdx.x, (int)gridDim.x, p.xcd_remap != 0);
+    for (int tile_id = first_tile; tile_id < p.num_tiles; tile_id += gridDim.x) {
         // ---- tile id -> wave -> (z, h, q block, kv range) ----
         int w = 0;
         while (w < p.num_waves && p.cum_wave_sizes[w] / kBlockM <= tile_id) ++w;
@@ -467,6 +472,400 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Two q blocks per workgroup, in opposite phases.
+//
+// A kv block costs a wavefront about as many cycles on the vector ALU (the softmax: 64 scores per
+// lane, one quarter-rate exponential each) as on the matrix pipe (64 MFMAs), and two independent
+// workgroups on a compute unit drift into step, so that both pipes idle half of the time.  Here
+// one workgroup of eight wavefronts holds two q blocks that read the same kv range - group 0
+// (wavefronts 0-3) tile 2i, group 1 (wavefronts 4-7) tile 2i + 1 - and runs them one slot apart:
+//
+//   slot         0      1      2          3          4          ...   2N         2N+1
+//   group 0      S0     sm0    PV0,S1     sm1        PV1,S2           PV(N-1)    -
+//   group 1      -      S0     sm0        PV0,S1     sm1              sm(N-1)    PV(N-1)
+//
+// so in every slot the two wavefronts of a SIMD use different pipes.  Both groups read K and V
+// from the same LDS blocks (half the fills per q row); K and V are double buffered: V(n) and
+// K(n+1) are fetched at slot 2n by all eight wavefronts, into the buffers whose last readers
+// (V(n-2), K(n-1)) finished in slot 2n-1, and have landed by the end of slot 2n+1.  One barrier
+// per slot, i.e. two per kv block and wavefront instead of four.
+// ---------------------------------------------------------------------------------------------
+constexpr int kPairThreads = 512;
+constexpr int kPairFills = kBlockBytes / 1024 / 8;      // 4 fills of 1 KB per wavefront and block
+
+__device__ __forceinline__ void dma_kv_block8(unsigned char* lds, const unsigned char* src, size_t pitch,
+                                              unsigned lane_off, int wave8) {
+#pragma unroll
+    for (int i = 0; i < kPairFills; ++i) {
+        const int blk = i * 8 + wave8;                  // blk % 4 == wave8 % 4: the swizzle of the 4-wave form holds
+        __builtin_amdgcn_global_load_lds((global_void_ptr)(src + (size_t)(blk * 4) * pitch + lane_off),
+                                         (lds_void_ptr)(lds + blk * 1024), 16, 0, 0);
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnParams p) {
+    typedef typename AttnMfma<T>::frag_t frag_t;
+    typedef T vec4_t __attribute__((ext_vector_type(4)));
+
+    __shared__ __attribute__((aligned(1024))) unsigned char k_lds[2 * kBlockBytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char v_lds[2 * kBlockBytes];
+    __shared__ int s_abort;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave8 = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int grp = wave8 >> 2;          // which of the two q blocks
+    const int wave = wave8 & 3;          // 32-row slice of the q block
+    const int r = lane & 31;
+    const int half = lane >> 5;
+
+    if (tid == 0) s_abort = 0;
+    __syncthreads();
+
+    // per-lane offsets exactly as in attn_fwd_kernel (the fill swizzle depends on wave8 % 4 only)
+    const int f_row = lane >> 4, f_c = lane & 15;
+    const size_t k_pitch = (size_t)p.k_st[2] * sizeof(T), v_pitch = (size_t)p.v_st[2] * sizeof(T);
+    const unsigned k_fill_off = (unsigned)(f_row * k_pitch + ((f_c ^ (4 * wave + f_row)) << 4));
+    const unsigned v_fill_off = (unsigned)(f_row * v_pitch + ((f_c ^ (f_row << 2)) << 4));
+    const int k_rd = r * kRowBytes;
+    const int i16 = lane & 15;
+    const int v_row = 4 * half + (i16 >> 2);
+    const int v_col_bytes = (16 * ((lane >> 4) & 1) + 4 * (i16 & 3)) * 2;
+    const int v_swz = (i16 >> 2) << 2;
+    int v_rd[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        v_rd[i] = v_row * kRowBytes + ((((4 * i + (v_col_bytes >> 4)) ^ v_swz) << 4) | (v_col_bytes & 15));
+    int k_chunk[8];
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) k_chunk[ks] = ((2 * ks + half) ^ (r & 15)) << 4;
+
+    const T* __restrict__ Q = reinterpret_cast<const T*>(p.q);
+    const unsigned char* __restrict__ K = reinterpret_cast<const unsigned char*>(p.k);
+    const unsigned char* __restrict__ V = reinterpret_cast<const unsigned char*>(p.v);
+    T* __restrict__ O = reinterpret_cast<T*>(p.o);
+
+    const int num_pairs = p.num_tiles / 2;
+    const int first_pair = logical_program_id((int)blockIdx.x, (int)gridDim.x, p.xcd_remap != 0);
+    for (int pair = first_pair; pair < num_pairs; pair += gridDim.x) {
+        // ---- tile id -> wave -> (z, h, q block, kv range); the two tiles of a pair differ in the q block only ----
+        const int tile_id = 2 * pair + grp;
+        int w = 0;
+        while (w < p.num_waves && p.cum_wave_sizes[w] / kBlockM <= tile_id) ++w;
+        if (w >= p.num_waves) return;
+        const int prev = w == 0 ? 0 : p.cum_wave_sizes[w - 1] / kBlockM;
+        const int t = tile_id - prev;
+        const int size_h = p.wave_sizes[w * 4 + 1];
+        const int nq = p.wave_sizes[w * 4 + 2] / kBlockM;
+        const int nkv = p.wave_sizes[w * 4 + 3] / kBlockN;
+        const int z = t / (nq * size_h) + p.wave_offsets[w * 4 + 0];
+        const int h = (t / nq) % size_h + p.wave_offsets[w * 4 + 1];
+        const int qb = t % nq + p.wave_offsets[w * 4 + 2] / kBlockM;
+        const int kv_lo = p.wave_offsets[w * 4 + 3] / kBlockN;
+        const int sig = p.signal_offsets[w];
+        if ((nq & 1) || (prev & 1)) {
+            // the caller promised an even number of q blocks per wave; leave a note instead of wrong results
+            if (lane == 0 && wave8 == 0) report_status(p.status, SYN_STATUS_BAD_PAIRING, w, (int)blockIdx.x, nq);
+            return;
+        }
+
+        if (p.visit_log != nullptr && lane == 0 && wave == 0) {
+            int4* rec = reinterpret_cast<int4*>(p.visit_log) + 2 * (size_t)tile_id;
+            rec[0] = make_int4(w, z, h, qb);
+            rec[1] = make_int4(kv_lo, kv_lo + nkv, sig, (int)blockIdx.x);
+        }
+
+        if (sig >= 0) {
+            if (tid == 0) {
+                const bool ok = spin_until_equal(p.flags + sig, 1ull, p.timeout_ticks);
+                if (!ok) {
+                    report_status(p.status, SYN_STATUS_SPIN_TIMEOUT, w, (int)blockIdx.x, sig);
+                    s_abort = 1;
+                }
+            }
+            __syncthreads();
+            acquire_fence_agent();
+            if (s_abort) return;
+        }
+
+        const size_t head = (size_t)z * p.H + h;
+        const int q_row = qb * kBlockM + wave * 32 + r;
+        const T* q_src = Q + z * p.q_st[0] + h * p.q_st[1] + q_row * p.q_st[2] + 8 * half;
+        const unsigned char* k_base = K + (z * p.k_st[0] + h * p.k_st[1]) * (int64_t)sizeof(T) +
+                                      (size_t)kv_lo * kBlockN * k_pitch;
+        const unsigned char* v_base = V + (z * p.v_st[0] + h * p.v_st[1]) * (int64_t)sizeof(T) +
+                                      (size_t)kv_lo * kBlockN * v_pitch;
+
+        // every wavefront has passed the barrier that ended the previous pair: all four buffers are free
+        dma_kv_block8(k_lds, k_base, k_pitch, k_fill_off, wave8);
+
+        frag_t qf[8];
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) qf[ks] = *reinterpret_cast<const frag_t*>(q_src + 16 * ks);
+        f32x16_t o_acc[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) o_acc[i][e] = 0.f;
+        float m_i = -INFINITY;
+        float l_i = 0.f;
+        f32x16_t s[4];
+        frag_t pf[8];
+
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(attn_vmcnt(0));       // K block 0 (and Q) have landed
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+
+        // V(m) and K(m+1) are fetched at the start of slot 2m by every wavefront and are first read in
+        // slot 2m + 2; their buffers were last read in slot 2m - 1.  (Spreading the fills between the
+        // products or the exponentials, or leaving them all to the group that is in its softmax,
+        // measured 1-6 % slower: a wavefront stalls at every fill wherever it is placed.)
+        auto fetch = [&](const int m) {
+            __builtin_amdgcn_sched_barrier(0);
+            dma_kv_block8(v_lds + (m & 1) * kBlockBytes, v_base + (size_t)m * kBlockN * v_pitch, v_pitch, v_fill_off,
+                          wave8);
+            if (m + 1 < nkv)
+                dma_kv_block8(k_lds + ((m + 1) & 1) * kBlockBytes, k_base + (size_t)(m + 1) * kBlockN * k_pitch,
+                              k_pitch, k_fill_off, wave8);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+
+        // S^T = K(n) . Q^T
+        auto scores = [&](const int n) {
+            const f32x16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            // fragments of steps ks and ks + 1 are in registers; the register a product has just
+            // consumed is refilled with the fragment of step ks + 2, so a read has almost two steps
+            // (256 MFMA cycles) to come back
+            frag_t kf[2][4];
+            const unsigned char* k_row = k_lds + (n & 1) * kBlockBytes + k_rd;
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    kf[b][j] = *reinterpret_cast<const frag_t*>(k_row + 32 * j * kRowBytes + k_chunk[b]);
+            __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    s[j] = AttnMfma<T>::run(kf[ks & 1][j], qf[ks], ks == 0 ? zero : s[j]);
+                    if (ks + 2 < 8)
+                        kf[ks & 1][j] = *reinterpret_cast<const frag_t*>(k_row + 32 * j * kRowBytes + k_chunk[ks + 2]);
+                }
+                if (ks + 2 < 8) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    }
+                } else {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+                }
+            }
+        };
+
+        // online softmax in base 2 over the scores in s; leaves P^T in pf
+        auto softmax = [&]() {
+            float mx = -INFINITY;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s[j][e]);
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            const float m_new = fmaxf(m_i, mx * p.qk_scale);
+            const float alpha = fast_exp2(m_i - m_new);
+            if (__builtin_amdgcn_ballot_w64(m_new != m_i) != 0) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) o_acc[i][e] *= alpha;
+            }
+            float row_sum = 0.f;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const float pe = fast_exp2(s[j][e] * p.qk_scale - m_new);
+                    row_sum += pe;
+                    pf[2 * j + (e >> 3)][e & 7] = (T)pe;
+                }
+            l_i = l_i * alpha + row_sum;
+            m_i = m_new;
+        };
+
+        // O^T += V(n)^T . P^T
+        auto weighted_values = [&](const int n) {
+            typedef short s16x8_t __attribute__((ext_vector_type(8)));
+            const unsigned char* v_blk = v_lds + (n & 1) * kBlockBytes;
+            s16x4_t vlo[2][4], vhi[2][4];
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const unsigned char* src = v_blk + 16 * b * kRowBytes + v_rd[i];
+                    vlo[b][i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)src);
+                    vhi[b][i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(src + 8 * kRowBytes));
+                }
+            __builtin_amdgcn_sched_group_barrier(0x100, 16, 0);
+#pragma unroll
+            for (int t2 = 0; t2 < 8; ++t2) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const s16x4_t lo = vlo[t2 & 1][i], hi = vhi[t2 & 1][i];
+                    const s16x8_t both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    o_acc[i] = AttnMfma<T>::run(__builtin_bit_cast(frag_t, both), pf[t2], o_acc[i]);
+                    if (t2 + 2 < 8) {
+                        const unsigned char* src = v_blk + 16 * (t2 + 2) * kRowBytes + v_rd[i];
+                        vlo[t2 & 1][i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)src);
+                        vhi[t2 & 1][i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(src + 8 * kRowBytes));
+                    }
+                }
+                if (t2 + 2 < 8) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                    }
+                } else {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+                }
+            }
+        };
+
+
+        // a slot ends when every wavefront's LDS reads have returned; at the end of an odd slot the
+        // blocks fetched one slot earlier have landed as well
+        auto end_even = [&]() {
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_waitcnt(0xc07f);
+            __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        auto end_odd = [&]() {
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_waitcnt(0x0070);
+            __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+        };
+
+        // the two groups run the same phases one slot apart; written out per group so that the scores
+        // (group 0) or the probabilities (group 1) are the only block-sized values that live across
+        // an iteration
+        if (grp == 0) {
+            fetch(0);                                    // slot 0
+            scores(0);
+            end_even();
+            for (int n = 0; n + 1 < nkv; ++n) {
+                softmax();                               // slot 2n + 1
+                end_odd();
+                fetch(n + 1);                            // slot 2n + 2
+                weighted_values(n);
+                scores(n + 1);
+                end_even();
+            }
+            softmax();                                   // slot 2N - 1
+            end_odd();
+            weighted_values(nkv - 1);                    // slot 2N
+            end_even();
+            end_odd();                                   // slot 2N + 1: group 1 finishes
+        } else {
+            fetch(0);                                    // slot 0: group 0 starts
+            end_even();
+            scores(0);                                   // slot 1
+            end_odd();
+            for (int n = 0; n + 1 < nkv; ++n) {
+                fetch(n + 1);                            // slot 2n + 2
+                softmax();
+                end_even();
+                weighted_values(n);                      // slot 2n + 3
+                scores(n + 1);
+                end_odd();
+            }
+            softmax();                                   // slot 2N
+            end_even();
+            weighted_values(nkv - 1);                    // slot 2N + 1
+            end_odd();
+        }
+
+        // ---- epilogue: lse2 = m + log2(l), O = acc / l, merged into the output under the q blocks' locks ----
+        const float l_tot = l_i + __shfl_xor(l_i, 32);
+        const float lse2 = m_i + fast_log2(l_tot);
+        const float inv_l = 1.0f / l_tot;
+        const int lock_idx = (int)(head * (p.Sq / kBlockM)) + qb;
+        if (tid == 0) {
+            // one thread takes both locks, lower q block first: every workgroup that wants this
+            // pair of q blocks takes them in the same order
+            const uint64_t t0 = wall_clock64();
+            bool ok = true;
+            for (int which = 0; which < 2 && ok; ++which) {
+                while (atomicCAS(p.lock + lock_idx + which, 0, 1) != 0) {
+                    __builtin_amdgcn_s_sleep(4);
+                    if ((int64_t)(wall_clock64() - t0) > p.timeout_ticks) { ok = false; break; }
+                }
+                if (!ok && which == 1) __hip_atomic_store(p.lock + lock_idx, 0, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            if (!ok) {
+                report_status(p.status, SYN_STATUS_SPIN_TIMEOUT, w, (int)blockIdx.x, -2);
+                s_abort = 1;
+            }
+        }
+        __syncthreads();
+        acquire_fence_agent();
+        if (s_abort) return;
+
+        const bool is_first = __hip_atomic_load(p.first + lock_idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0;
+        float w_old = 0.f, w_new = 1.f, lse_out = lse2;
+        float* lse_ptr = p.lse + head * p.Sq + q_row;
+        if (!is_first) {
+            const float m_old = *lse_ptr;
+            const float delta = m_old - lse2;
+            const float mmax = fmaxf(m_old, lse2);
+            lse_out = mmax + fast_log2(1.0f + fast_exp2(-fabsf(delta)));
+            w_old = fast_exp2(m_old - lse_out);
+            w_new = fast_exp2(lse2 - lse_out);
+        }
+        T* o_row = O + z * p.o_st[0] + h * p.o_st[1] + q_row * p.o_st[2] + 4 * half;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                float x[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) x[c] = o_acc[i][4 * g + c] * inv_l * w_new;
+                T* dst = o_row + 32 * i + 8 * g;
+                if (!is_first) {
+                    const vec4_t old = *reinterpret_cast<const vec4_t*>(dst);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) x[c] += (float)old[c] * w_old;
+                }
+                vec4_t out;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) out[c] = (T)x[c];
+                *reinterpret_cast<vec4_t*>(dst) = out;
+            }
+        if (half == 0) *lse_ptr = lse_out;
+
+        __threadfence();
+        __syncthreads();
+        if (tid == 0) {
+            // tid 0 is in group 0: its lock_idx is the lower q block of the pair
+            for (int which = 1; which >= 0; --which) {
+                __hip_atomic_store(p.first + lock_idx + which, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(p.lock + lock_idx + which, 0, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+    }
+}
+
+template <typename T>
+static int launch_attn_pairs(const AttnParams& p, int grid, hipStream_t stream) {
+    hipLaunchKernelGGL((attn_pair_kernel<T>), dim3(grid), dim3(kPairThreads), 0, stream, p);
+    return (int)hipGetLastError();
+}
+
 template <typename T>
 static int launch_attn(const AttnParams& p, int grid, hipStream_t stream) {
     hipLaunchKernelGGL((attn_fwd_kernel<T>), dim3(grid), dim3(kAttnThreads), 0, stream, p);
@@ -551,6 +950,7 @@ int syn_attn_fwd(const syn_attn_desc* d, syn_stream_t stream) {
     p.Skv = d->Skv;
     p.causal = d->causal ? 1 : 0;
     p.num_tiles = (int)tiles;
+    p.xcd_remap = (d->options & SYN_ATTN_XCD_REMAP) ? 1 : 0;
     p.qk_scale = d->sm_scale * 1.44269504f;
     {
         // all-zero strides: contiguous [Z, H, S, D]
@@ -570,9 +970,17 @@ int syn_attn_fwd(const syn_attn_desc* d, syn_stream_t stream) {
         }
     }
 
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (d->options & SYN_ATTN_PAIR_Q_BLOCKS) {
+        // two q blocks per workgroup: the caller vouches for an even number of q blocks in every wave
+        if (d->causal || d->counters || tiles % 2) return SYN_EINVAL;
+        int grid = d->num_programs > 0 ? d->num_programs : (int)(tiles / 2);
+        if (grid > tiles / 2) grid = (int)(tiles / 2);
+        return d->dtype == SYN_DTYPE_BF16 ? launch_attn_pairs<__bf16>(p, grid, s)
+                                          : launch_attn_pairs<_Float16>(p, grid, s);
+    }
     int grid = d->num_programs > 0 ? d->num_programs : (int)tiles;
     if (grid > tiles) grid = (int)tiles;
-    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     return d->dtype == SYN_DTYPE_BF16 ? launch_attn<__bf16>(p, grid, s)
                                       : launch_attn<_Float16>(p, grid, s);
 }

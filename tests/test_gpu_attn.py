@@ -137,3 +137,69 @@ def test_bshd_layout_and_strided_views(hip, causal):
     o2 = attention_forward(wide[:, 1:], kv[0, :, :, 64:64 + S], kv[1, :, :, 64:64 + S], sm_scale, **tables)
     check_status()
     assert _rel(o2, ref) <= REL_TOL
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("num_programs,xcd_remap", [(0, False), (3, False), (0, True), (16, True)])
+def test_paired_q_blocks_match_sdpa_and_oracle(hip, dtype, num_programs, xcd_remap):
+    """Two q blocks per workgroup in opposite phases (an extension: one program per tile in the
+    reference): same tiles, same merge under the q blocks' locks, results to the same tolerance."""
+    from syncopate_amd.computation.attn import attention_forward
+    from syncopate_amd.computation._launch import check_status
+
+    Z, H, Sq, Skv = 2, 3, 512, 1024
+    q, k, v = _qkv(Z, H, Sq, Skv, dtype, seed=4)
+    chunks = [(512, 768), (0, 256), (768, 1024), (256, 512)]          # arrival order
+    offsets, sizes, cums, signals, total = _kv_waves(Z, H, Sq, chunks, [-1, 0, 1, 2])
+    flags = torch.ones(3, dtype=torch.int64, device="cuda")
+    sm_scale = 128 ** -0.5
+    tiles = total // 128
+    log = torch.full((tiles, 8), -1, dtype=torch.int32, device="cuda")
+    o, lse = attention_forward(q.cuda(), k.cuda(), v.cuda(), sm_scale, wave_offsets=offsets,
+                               wave_sizes=sizes, cum_wave_sizes=cums, signal_ptr=flags,
+                               signal_offsets=signals, NUM_WAVES=4, cum_tiles=total,
+                               num_programs=num_programs, return_lse=True, visit_log=log,
+                               pair_q_blocks=True, xcd_remap=xcd_remap)
+    check_status()
+    assert _rel(o, numerics.sdpa_fp32(q, k, v, sm_scale)) <= REL_TOL
+    want_o, want_lse = numerics.chunked_attention(q, k, v, sm_scale, chunks)
+    assert _rel(o, want_o.float()) <= REL_TOL
+    assert (lse.cpu() - want_lse).abs().max().item() <= 2e-2
+
+    # every tile was visited once, with the kv range and flag of its wave; tiles 2i and 2i + 1 by one program
+    got = log.cpu().tolist()
+    grid = min(num_programs, tiles // 2) if num_programs else tiles // 2
+    for tile_id, rec in enumerate(got):
+        exp = visit_order.attn_tile_work(tile_id, offsets, sizes, cums, signals)
+        assert rec[:7] == [exp["wave"], exp["z"], exp["h"], exp["q_block"], exp["kv_lo"], exp["kv_hi"], exp["signal"]]
+        assert 0 <= rec[7] < grid
+        assert rec[7] == got[tile_id ^ 1][7]
+    if not xcd_remap:
+        assert [rec[7] for rec in got[0::2]] == [pair % grid for pair in range(tiles // 2)]
+    else:
+        # a bijection between workgroups and first pairs: every program took its share
+        first = {}
+        for pair in range(tiles // 2):
+            first.setdefault(got[2 * pair][7], pair)
+        assert sorted(first) == list(range(grid)) and sorted(first.values()) == list(range(grid))
+
+
+def test_paired_q_blocks_argument_errors(hip):
+    from syncopate_amd.computation.attn import attention_forward
+
+    q, k, v = (t.cuda() for t in _qkv(1, 1, 384, 256, torch.bfloat16))
+    offsets, sizes, cums, signals, total = _kv_waves(1, 1, 384, [(0, 256)], [-1])
+    flags = torch.ones(1, dtype=torch.int64, device="cuda")
+    kw = dict(wave_offsets=offsets, wave_sizes=sizes, cum_wave_sizes=cums, signal_ptr=flags, signal_offsets=signals,
+              cum_tiles=total)
+    with pytest.raises(ValueError, match="even number of q blocks"):
+        attention_forward(q, k, v, 0.1, pair_q_blocks=True, **kw)            # three q blocks
+    q2, k2, v2 = (t.cuda() for t in _qkv(1, 1, 256, 256, torch.bfloat16))
+    offsets, sizes, cums, signals, total = _kv_waves(1, 1, 256, [(0, 256)], [-1])
+    kw = dict(wave_offsets=offsets, wave_sizes=sizes, cum_wave_sizes=cums, signal_ptr=flags, signal_offsets=signals,
+              cum_tiles=total)
+    with pytest.raises(ValueError):
+        attention_forward(q2, k2, v2, 0.1, pair_q_blocks=True, causal=True, **kw)
+    with pytest.raises(ValueError):
+        attention_forward(q2, k2, v2, 0.1, pair_q_blocks=True,
+                          counter_ptr=torch.zeros(1, dtype=torch.int32, device="cuda"), **kw)
