@@ -128,6 +128,12 @@ typedef struct syn_gemm_remote {
     int32_t c_ld;                   /* row length of a peer C buffer (multiple of 4)           */
     int32_t c_atomic_add;           /* 1: add into the peer C (packed 16-bit float atomics),
                                        0: store                                                */
+    const int32_t* k_ranges;        /* device int32[num_waves, 2] or NULL: {first k, count} of
+                                       the part of K a wave contracts over, multiples of 64
+                                       (split-K waves: the generated GEMM with a K range axis,
+                                       tests/computation/transform/examples/example_splitk_gemm.py:
+                                       36-112, consumer of tests/test_all2all_gemm.py:113-160);
+                                       needs c_atomic_add and a zeroed C                       */
 } syn_gemm_remote;
 
 /*

@@ -86,6 +86,7 @@ class GemmRemote(ctypes.Structure):
         ("c_dst_offsets", c_void_p),
         ("c_ld", c_int32),
         ("c_atomic_add", c_int32),
+        ("k_ranges", c_void_p),
     ]
 
 

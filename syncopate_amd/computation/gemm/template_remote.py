@@ -69,6 +69,7 @@ def gemm_remote(
     target_rank: Optional[TableLike] = None,
     dst_offsets: Optional[TableLike] = None,
     atomic_add: bool = False,
+    k_ranges: Optional[TableLike] = None,
     signal_ptr: Optional[torch.Tensor] = None,
     signal_offsets: Optional[TableLike] = None,
     cum_tiles: int = 0,
@@ -83,7 +84,9 @@ def gemm_remote(
     `a_target_rank` (then the A rows of wave w are rows `tile row inside the wave` of shard
     a_target_rank[w]).  `c` is a tensor [M, N], or a list of per-rank buffers [rows, ldc]
     together with `target_rank` and `dst_offsets` ([num_waves, 2] element offsets of the wave's
-    region in the peer buffer); `atomic_add` adds instead of storing.
+    region in the peer buffer); `atomic_add` adds instead of storing.  `k_ranges` ([num_waves, 2]:
+    first k and count, multiples of 64) makes a wave contract over part of K only; its partial
+    product has to be added (`atomic_add`) into a C that starts at zero.
     """
     a_list = list(a) if isinstance(a, (list, tuple)) else None
     c_list = list(c) if isinstance(c, (list, tuple)) else None
@@ -163,6 +166,20 @@ def gemm_remote(
         remote.c_atomic_add = 1 if atomic_add else 0
     elif atomic_add:
         raise ValueError("atomic_add needs c bound to peers")
+    if k_ranges is not None:
+        if c_list is None or not atomic_add:
+            raise ValueError("k_ranges produce partial products: c must be bound and added into (atomic_add)")
+        ranges = as_device_table(k_ranges, dev, 2)
+        hk = host_copy(ranges)
+        if ranges.shape[0] < num_waves:
+            raise ValueError("k_ranges is shorter than the wave tables")
+        k0, kn = hk[:num_waves, 0], hk[:num_waves, 1]
+        if int(k0.min()) < 0 or int(kn.min()) <= 0 or int((k0 % 64).max()) or int((kn % 64).max()):
+            raise ValueError("k ranges must start at and span positive multiples of 64")
+        if int((k0 + kn).max()) > K:
+            raise ValueError("a k range runs past K")
+        keep.append(ranges)
+        remote.k_ranges = ranges.data_ptr()
 
     if visit_log is not None:
         tiles = (int(cum_tiles) if cum_tiles else M * N) // (BLOCK_SIZE_M * BLOCK_SIZE_N)
@@ -253,3 +270,42 @@ def gemm_rs_producer_persistent(
     gemm_remote(a, b, bufs, num_gemm_sms, BLOCK_SIZE_M, BLOCK_SIZE_N, BLOCK_SIZE_K, GROUP_SIZE_M, STAGES,
                 cur_wave_sizes=cur_wave_size, wave_offsets=wave_offset, M=m, target_rank=target_rank,
                 dst_offsets=dst, atomic_add=True, cum_tiles=m * b.shape[0], **kwargs)
+
+
+def gemm_splitk(
+    a: torch.Tensor,
+    b: torch.Tensor,
+    c: torch.Tensor,
+    world_size: int,
+    num_gemm_sms: int,
+    BLOCK_SIZE_M: int = 128,
+    BLOCK_SIZE_N: int = 256,
+    BLOCK_SIZE_K: int = 64,
+    GROUP_SIZE_M: int = 8,
+    STAGES: int = 3,
+    *,
+    cur_wave_sizes: TableLike,
+    wave_offsets: TableLike,
+    signal_ptr: Optional[torch.Tensor] = None,
+    signal_offsets: Optional[TableLike] = None,
+    cum_tiles: int = 0,
+    **kwargs,
+) -> None:
+    """c += a @ b.T, wave by wave, where a wave is a box [rows, cols, k count] at [row, col, first k]
+    of the (M, N, K) iteration space: the call form of the reference's transformed split-K GEMM
+    (tests/computation/transform/examples/example_splitk_gemm.py:117-175, called with three-column
+    tables at tests/test_all2all_gemm.py:142-160 and tests/test_gemm_all2all_gemm.py:183-196).
+    Each (tile, wave) pair is one work item whose partial product is atomically added into `c`,
+    which the caller zeroes; a wave with a flag is waited for before its part of A is read."""
+    dev = require_cuda(a, b, c)
+    sizes3 = as_device_table(cur_wave_sizes, dev, 3)
+    offsets3 = as_device_table(wave_offsets, dev, 3)
+    num_waves = sizes3.shape[0]
+    if offsets3.shape[0] != num_waves:
+        raise ValueError("wave size and offset tables disagree on the number of waves")
+    gemm_remote(a, b, [c], num_gemm_sms, BLOCK_SIZE_M, BLOCK_SIZE_N, BLOCK_SIZE_K, GROUP_SIZE_M, STAGES,
+                cur_wave_sizes=sizes3[:, :2].contiguous(), wave_offsets=offsets3[:, :2].contiguous(), M=a.shape[0],
+                target_rank=torch.zeros(num_waves, dtype=torch.int32, device=dev),
+                dst_offsets=offsets3[:, :2].contiguous(), atomic_add=True,
+                k_ranges=torch.stack([offsets3[:, 2], sizes3[:, 2]], dim=1).contiguous(),
+                signal_ptr=signal_ptr, signal_offsets=signal_offsets, cum_tiles=cum_tiles, **kwargs)

@@ -8,8 +8,8 @@ that already contain the wave walk, the flag waits and the producer epilogue, so
 annotations select a template and fix its call form instead: `transform(source)` returns a
 `KernelBinding` that knows
 
-  * which template the annotated tiling is (GEMM: single axes M, N; attention: single axes Z, H, Q
-    and a range axis KV),
+  * which template the annotated tiling is (GEMM: single axes M, N; split-K GEMM: the same with a
+    range axis K; attention: single axes Z, H, Q and a range axis KV),
   * the keyword arguments the reference would have appended to the kernel (same names, same
     order, same defaults: transformer.py:1125-1178), which are the keywords `launch()` takes,
   * per bound descriptor, whether the compute kernel reads it from a peer or writes / atomically
@@ -48,7 +48,7 @@ class RemoteSlot:
 
 @dataclass
 class KernelBinding:
-    template: str                               # "gemm" or "attention"
+    template: str                               # "gemm", "gemm_splitk" or "attention"
     persistent: bool
     annotations: ParsedAnnotations
     consumer: bool
@@ -96,7 +96,20 @@ class KernelBinding:
             raise TypeError("counter_ptr given to a kernel bound without enable_producer")
         if self.template == "gemm":
             return self._launch_gemm(args, kwargs, tables, flags, flag_offsets, counters)
+        if self.template == "gemm_splitk":
+            return self._launch_gemm_splitk(args, kwargs, tables, flags, flag_offsets, counters)
         return self._launch_attention(args, kwargs, tables, flags, flag_offsets, counters)
+
+    def _launch_gemm_splitk(self, args, kwargs, tables, flags, flag_offsets, counters):
+        from ..gemm import gemm_splitk
+
+        if self.remote or counters is not None:
+            raise NotImplementedError("the split-K template is a consumer that adds into a local result")
+        if not self.persistent:
+            raise NotImplementedError("the split-K template takes the persistent kernel's tables (cur_wave_sizes)")
+        return gemm_splitk(*args, cur_wave_sizes=self._wave_sizes(tables), wave_offsets=tables["wave_offsets"],
+                           signal_ptr=flags, signal_offsets=flag_offsets, cum_tiles=tables.get("cum_tiles", 0),
+                           **kwargs)
 
     def _wave_sizes(self, tables: Mapping[str, Any]):
         name = "cur_wave_sizes" if self.persistent else "wave_sizes"
@@ -159,11 +172,13 @@ def _template_for(parsed: ParsedAnnotations) -> str:
     ranges = [a.axis.lower() for a in parsed.axis_counts if a.kind == "range"]
     if singles == ["m", "n"] and not ranges:
         return "gemm"
+    if singles == ["m", "n"] and ranges == ["k"]:
+        return "gemm_splitk"
     if singles == ["z", "h", "q"] and ranges == ["kv"]:
         return "attention"
     raise AnnotationError(
-        f"no HIP template tiles single axes {singles} with range axes {ranges}: "
-        "there is a GEMM over (M, N) and an attention over (Z, H, Q) with a KV range")
+        f"no HIP template tiles single axes {singles} with range axes {ranges}: there is a GEMM over "
+        "(M, N), the same with a K range per wave, and an attention over (Z, H, Q) with a KV range")
 
 
 class AnnotationTransformer:

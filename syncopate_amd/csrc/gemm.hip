@@ -56,6 +56,9 @@ struct GemmParams {
     const int32_t* c_dst_offsets;
     int32_t c_ld;
     int32_t c_atomic;
+    // per-wave K range {first k, count}: a wave contracts over part of K only (split-K waves,
+    // whose partial products are added into C); null: every wave takes all of K
+    const int32_t* wave_k;
 };
 
 // kernel modes
@@ -732,6 +735,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
     const T* a_base = nullptr;
     T* c_base = nullptr;
     int dst_m = 0, dst_n = 0;
+    int cur_k0 = 0, cur_klen = p.K;
     auto enter_wave = [&](int w) {
         cur_wave = w;
         if (w < kLdsWaves) {
@@ -756,6 +760,10 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
                 c_base = reinterpret_cast<T*>(p.c_peers[p.c_target[w]]);
                 dst_m = p.c_dst_offsets[2 * w];
                 dst_n = p.c_dst_offsets[2 * w + 1];
+            }
+            if (p.wave_k) {
+                cur_k0 = p.wave_k[2 * w];
+                cur_klen = p.wave_k[2 * w + 1];
             }
         }
     };
@@ -807,6 +815,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
         T* c_tile;                       // element (0, 0) of the tile in its C buffer
         size_t ldc;
         int k_rot, wave, sig, wave_tiles;
+        int k_len;                       // elements of K the tile contracts over (the panels start at its first k)
     };
     // get_pid_mn (template.py:10-18) on the wave-local tile id, and the tile's K phase
     auto locate = [&](int tile_id) -> Tile {
@@ -840,6 +849,12 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
         // same few memory channels; four phases spread them while tiles that share a panel of A
         // or B still stay within 512 elements of each other (L2 reuse).
         t.k_rot = p.k_stagger ? ((pid_m + pid_n) & 3) * (128 / Pipe::BK) : 0;
+        t.k_len = K;
+        if (REMOTE) {
+            t.a_panel += (size_t)cur_k0 * sizeof(T);
+            t.b_panel += (size_t)cur_k0 * sizeof(T);
+            t.k_len = cur_klen;
+        }
         t.wave = cur_wave;
         t.sig = cur_sig;
         t.wave_tiles = cur_tiles;
@@ -854,7 +869,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
     }
     if (cur_wave < 0) return;
     Tile tile = locate(pid);
-    Pipe::prologue(panel_a(tile), panel_b(tile), row_bytes, K, tile.k_rot, lane, wave);
+    Pipe::prologue(panel_a(tile), panel_b(tile), row_bytes, tile.k_len, tile.k_rot, lane, wave);
 
     for (int it = 0; it < tiles_here; ++it) {
         f32x16_t acc[TM][TN];
@@ -865,7 +880,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
 #pragma unroll
                 for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-        Pipe::main(acc, panel_a(tile), panel_b(tile), row_bytes, K, tile.k_rot, lane, wave);
+        Pipe::main(acc, panel_a(tile), panel_b(tile), row_bytes, tile.k_len, tile.k_rot, lane, wave);
 
         // The stages are free: start the next tile's fills before this tile's C is stored, unless
         // the next tile opens a wave whose flag is still to be waited for (nothing of a chunk may
@@ -879,7 +894,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
             if (cur_wave < 0) return;
             if (!gated) {
                 next = locate(next_id);
-                Pipe::prologue(panel_a(next), panel_b(next), row_bytes, K, next.k_rot, lane, wave);
+                Pipe::prologue(panel_a(next), panel_b(next), row_bytes, next.k_len, next.k_rot, lane, wave);
             }
         }
 
@@ -966,7 +981,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
         if (has_next && gated) {
             if (!wait_flag(cur_sig)) return;
             next = locate(next_id);
-            Pipe::prologue(panel_a(next), panel_b(next), row_bytes, K, next.k_rot, lane, wave);
+            Pipe::prologue(panel_a(next), panel_b(next), row_bytes, next.k_len, next.k_rot, lane, wave);
         }
         tile = next;
     }
@@ -1031,6 +1046,7 @@ static int gemm_entry(const syn_gemm_desc* d, hipStream_t stream, int mode,
         if (c_remote && (!remote->c_target_rank || !remote->c_dst_offsets || remote->c_ld <= 0)) return SYN_EINVAL;
         if (c_remote && remote->c_ld % 4) return SYN_EALIGN;
         if (remote->c_atomic_add && !c_remote) return SYN_EINVAL;
+        if (remote->k_ranges && !(c_remote && remote->c_atomic_add)) return SYN_EINVAL;   // partial products are added
     }
     if ((!d->a && !a_remote) || !d->b || (!d->c && !c_remote) || !d->wave_sizes || !d->wave_offsets ||
         !d->signal_offsets)
@@ -1080,6 +1096,7 @@ static int gemm_entry(const syn_gemm_desc* d, hipStream_t stream, int mode,
     p.c_dst_offsets = c_remote ? remote->c_dst_offsets : nullptr;
     p.c_ld = c_remote ? remote->c_ld : 0;
     p.c_atomic = (remote && remote->c_atomic_add) ? 1 : 0;
+    p.wave_k = remote ? remote->k_ranges : nullptr;
     const bool eight = (d->options & SYN_GEMM_EIGHT_WAVES) != 0;
     // the ring needs whole groups of four 32-deep slabs (and does not exist for 224-wide tiles)
     const bool ring = (d->options & SYN_GEMM_RING_PIPE) && d->K % 128 == 0 && d->block_n != 224;

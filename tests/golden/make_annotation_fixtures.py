@@ -64,16 +64,33 @@ def flash_forward(q, k, v, o, Z, H, SQ, SKV, BQ: tl.constexpr, BKV: tl.constexpr
     # @sy.dispatch end
     attend(pid_z, pid_h, pid_q, kv_lo, kv_hi)
 """,
-    "split_k_has_no_template": """
-def split_k(a, b, c, M, N, K, BM: tl.constexpr, BN: tl.constexpr, BK: tl.constexpr):
+    "batched_rows_have_no_template": """
+def rowwise(x, y, B, R, BR: tl.constexpr):
     pid = tl.program_id(0)      # @sy.tile_id
+    nb = B                      # @sy.axis_count B
+    nr = tl.cdiv(R, BR)         # @sy.axis_count R block=BR
+    # @sy.dispatch begin
+    pid_b, pid_r = divmod(pid, nr)
+    # @sy.pid_map B=pid_b R=pid_r
+    # @sy.dispatch end
+""",
+    "gemm_split_k_persistent": """
+def split_k(a, b, c, M, N, K, BM: tl.constexpr, BN: tl.constexpr, BK: tl.constexpr, PROGRAMS: tl.constexpr):
+    first = tl.program_id(0)
     tm = tl.cdiv(M, BM)         # @sy.axis_count M block=BM
     tn = tl.cdiv(N, BN)         # @sy.axis_count N block=BN
     tk = tl.cdiv(K, BK)         # @sy.axis_count K=range block=BK
-    # @sy.dispatch begin
-    pid_m, pid_n, k_lo, k_hi = split(pid, tm, tn, tk)
-    # @sy.pid_map M=pid_m N=pid_n K=k_lo..k_hi
-    # @sy.dispatch end
+    tile = first - PROGRAMS     # @sy.tile_id persistent
+    # @sy.persistent_init begin
+    # @sy.persistent_init end
+    for _ in range(first, tm * tn, PROGRAMS):
+        tile += PROGRAMS
+        # @sy.dispatch begin
+        pid_m, pid_n, k_lo, k_hi = split(tile, tm, tn, tk)
+        # @sy.pid_map M=pid_m N=pid_n K=k_lo..k_hi
+        # @sy.dispatch end
+        add_into(c, pid_m, pid_n, contract(a, b, pid_m, pid_n, k_lo, k_hi))
+        # @sy.producer_epilogue
 """,
 }
 

@@ -709,3 +709,80 @@ def test_gemm_then_library_collective_whole_mesh(hip, form):
     if form != "all_reduce":
         # the partial products were only read
         assert _rel(ctx.comm_buffers["src"][rank], partial[rank]) <= REL_TOL
+
+
+@pytest.mark.parametrize("rank", [1, 2])
+def test_gemm_all2all_gemm_chain(hip, rank):
+    """An MLP with its hidden layer sharded by columns and its output by rows
+    (tests/test_gemm_all2all_gemm.py:126-200, 257-318): producer GEMM x @ w1_shard^T with a flag per
+    row block -> all-to-all by box copies on compute units (every rank sends each owner its rows)
+    -> split-K consumer GEMM over the gathered columns, which starts on a source rank's columns
+    as soon as that rank's block has arrived.  The other ranks' first GEMMs are computed
+    beforehand; the whole mesh's op lists are replayed beside this rank's two kernels."""
+    from syncopate_amd.communication.code_gen import CodeGenOptions, CommGenerator
+    from syncopate_amd.communication.comm_runtime.communication_context import CommContext
+    from syncopate_amd.communication.common_descriptors import build_all_to_all_plan_dim
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.gemm import gemm_producer, gemm_splitk
+    from syncopate_amd.interface import lower_comm_plan_to_raw_schedules
+    from syncopate_amd.interface.wave_tables import gemm_producer_tables
+
+    world, seq, hidden, ffn, BM, BN = 4, 1024, 256, 1024, 128, 128
+    seq_local, ffn_local = seq // world, ffn // world
+    dtype = torch.float16
+    gen = CommGenerator({r: build_all_to_all_plan_dim(
+        shape=(seq, ffn_local), dtype=dtype, mesh_size=world, rank=r, src_buffer="src", dst_buffer="dst",
+        src_split_axis=1, dst_split_axis=0, transfer_kind="push", compute_producer=True) for r in range(world)})
+    gen.plan_signals()
+    schedules = lower_comm_plan_to_raw_schedules(gen)
+    info = gen.generate_code_for_plan(CodeGenOptions(copy_engine=False))
+    info.local_world_size = info.world_size
+    info.num_copy_sms = 12
+    ctx = CommContext(rank, info)
+
+    g = torch.Generator().manual_seed(41)
+    x = (0.1 * torch.randn(seq, hidden, generator=g)).to(dtype)
+    w1 = [(0.1 * torch.randn(ffn_local, hidden, generator=g)).to(dtype) for _ in range(world)]
+    w2 = (0.1 * torch.randn(hidden, ffn, generator=g)).to(dtype)
+    xd, w2d = x.cuda(), w2.cuda()
+
+    def first_gemm(r):
+        tables = gemm_producer_tables(schedules[r]["src"])
+        gemm_producer(xd, w1[r].cuda(), ctx.comm_buffers["src"][r], ctx.compute_signal_bufs[r], tables.block_shapes,
+                      tables.block_offsets, tables.signal_offsets, 24, BM, BN, 64, 8, cum_tiles=tables.cum_tiles)
+
+    # the consumer's tables: a wave per source rank, [rows, hidden, that rank's columns] at [0, 0, first column]
+    dst = schedules[rank]["dst"]
+    shapes = [[rows, hidden, cols] for rows, cols in dst.gen_block_shape_lists()]
+    offsets = [[r0, 0, c0] for r0, c0 in dst.gen_block_offset_lists()]
+    signals = dst.gen_signal_lists()
+    assert sorted(c0 for _, _, c0 in offsets) == [q * ffn_local for q in range(world)] and sorted(signals) == [0, 1, 2, 3]
+
+    out = torch.zeros(seq_local, hidden, dtype=dtype, device="cuda")
+    ctx.comm_buffers["dst"][rank].fill_(float("nan"))       # columns read before their flag would show
+    ctx.reset_signals(whole_mesh=True)
+    for r in range(world):
+        if r != rank:
+            first_gemm(r)
+    ctx.start_after()
+    ctx.execute_mesh()
+    first_gemm(rank)
+    gemm_splitk(ctx.comm_buffers["dst"][rank], w2d, out, world, 24, BM, BN, 64, 8, cur_wave_sizes=shapes,
+                wave_offsets=offsets, signal_ptr=ctx.recv_signal_bufs[rank], signal_offsets=signals,
+                cum_tiles=sum(s[0] * s[1] for s in shapes))
+    ctx.end_before()
+    check_status()
+    ctx.check_status()
+
+    hidden_act = torch.cat([numerics.gemm_fp32(x, w1[r]) for r in range(world)], dim=1)       # [seq, ffn]
+    mine = hidden_act[rank * seq_local:(rank + 1) * seq_local]
+    gathered = ctx.comm_buffers["dst"][rank].float().cpu()
+    assert _rel(gathered, mine) <= REL_TOL
+    for q in range(world):
+        # what rank q sent is bit for bit what its GEMM produced
+        sent = ctx.comm_buffers["src"][q][rank * seq_local:(rank + 1) * seq_local]
+        assert torch.equal(ctx.comm_buffers["dst"][rank][:, q * ffn_local:(q + 1) * ffn_local], sent)
+    want = mine.to(dtype).float() @ w2.float().t()
+    # four partial products rounded to fp16 and added; the reference bounds the chain by 5e-1
+    assert _rel(out, want) <= 4 * REL_TOL
+    assert ctx.recv_signal_bufs[rank].tolist() == [1] * world

@@ -136,3 +136,56 @@ def test_remote_argument_errors(hip):
         gemm_remote(a, b, [c], 8, 128, 128, target_rank=[0], dst_offsets=[[128, 0]], **kw)  # does not fit
     with pytest.raises(ValueError):
         gemm_remote([a[:128]], b, c, 8, 128, 128, a_target_rank=[0], **kw)   # wave taller than the shard
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("BM,BN,chunks", [(128, 256, [(256, 128), (0, 64), (64, 192), (384, 128)]),
+                                          (256, 256, [(0, 256), (256, 256)]),
+                                          (128, 128, [(448, 64), (0, 448)])])
+def test_split_k_waves_add_up_to_the_product(hip, dtype, BM, BN, chunks):
+    """Waves that each contract over part of K (first k, count) and add their partial product into
+    C: the transformed split-K GEMM of the reference (tests/computation/transform/examples/
+    example_splitk_gemm.py:36-112), whose K chunks arrive one by one (tests/test_all2all_gemm.py:
+    94-103 builds the three-column tables)."""
+    from syncopate_amd.computation.gemm import gemm_splitk
+    from syncopate_amd.computation._launch import check_status
+
+    M, N, K = 512, 512, 512
+    g = torch.Generator().manual_seed(21)
+    a = (0.05 * torch.randn(M, K, generator=g)).to(dtype)
+    b = (0.05 * torch.randn(N, K, generator=g)).to(dtype)
+    ref = numerics.gemm_fp32(a, b)
+    sizes = [[M, N, count] for _, count in chunks]
+    offsets = [[0, 0, first] for first, _ in chunks]
+    flags = torch.ones(len(chunks), dtype=torch.int64, device="cuda")
+    c = torch.zeros(M, N, dtype=dtype, device="cuda")
+    gemm_splitk(a.cuda(), b.cuda(), c, 1, 37, BM, BN, 64, 8, cur_wave_sizes=sizes, wave_offsets=offsets,
+                signal_ptr=flags, signal_offsets=list(range(len(chunks))), cum_tiles=len(chunks) * M * N)
+    check_status()
+    # one rounding to 16 bits per chunk on top of the product's
+    assert _max_rel_err(c, ref) <= len(chunks) * REL_TOL
+    torch.testing.assert_close(c.float().cpu(), ref, atol=2e-2, rtol=2e-2)
+    # each chunk alone is the product over its columns
+    for (first, count), size, off in zip(chunks, sizes, offsets):
+        part = torch.zeros(M, N, dtype=dtype, device="cuda")
+        gemm_splitk(a.cuda(), b.cuda(), part, 1, 16, BM, BN, 64, 8, cur_wave_sizes=[size], wave_offsets=[off],
+                    cum_tiles=M * N)
+        want = numerics.gemm_fp32(a[:, first:first + count], b[:, first:first + count])
+        assert ((part.float().cpu() - want).abs().max() / ref.abs().max()).item() <= REL_TOL
+    check_status()
+
+
+def test_split_k_argument_errors(hip):
+    from syncopate_amd.computation.gemm import gemm_remote, gemm_splitk
+
+    a = torch.zeros(256, 256, dtype=torch.bfloat16, device="cuda")
+    b = torch.zeros(256, 256, dtype=torch.bfloat16, device="cuda")
+    c = torch.zeros(256, 256, dtype=torch.bfloat16, device="cuda")
+    kw = dict(cum_tiles=256 * 256)
+    with pytest.raises(ValueError, match="multiples of 64"):
+        gemm_splitk(a, b, c, 1, 8, 128, 128, cur_wave_sizes=[[256, 256, 96]], wave_offsets=[[0, 0, 0]], **kw)
+    with pytest.raises(ValueError, match="past K"):
+        gemm_splitk(a, b, c, 1, 8, 128, 128, cur_wave_sizes=[[256, 256, 128]], wave_offsets=[[0, 0, 192]], **kw)
+    with pytest.raises(ValueError, match="added into"):
+        gemm_remote(a, b, [c], 8, 128, 128, cur_wave_sizes=[[256, 256]], wave_offsets=[[0, 0]], M=256,
+                    target_rank=[0], dst_offsets=[[0, 0]], k_ranges=[[0, 128]], **kw)      # plain stores

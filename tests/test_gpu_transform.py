@@ -135,3 +135,22 @@ def test_attention_binding_matches_the_template_call(hip):
     # agree to rounding, not bit for bit
     torch.testing.assert_close(got.float(), want.float(), atol=2e-3, rtol=2e-3)
     assert _rel(got, numerics.sdpa_fp32(q.cpu(), k.cpu(), v.cpu(), D ** -0.5)) <= 2e-2
+
+
+def test_split_k_binding(hip):
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.transform import AnnotationTransformer
+
+    M, N, K, BM, BN = 256, 512, 384, 128, 256
+    g = torch.Generator().manual_seed(13)
+    a = (0.05 * torch.randn(M, K, generator=g)).bfloat16()
+    b = (0.05 * torch.randn(N, K, generator=g)).bfloat16()
+    binding = AnnotationTransformer(enable_consumer=True).transform(SNIPPETS["gemm_split_k_persistent"])
+    assert binding.template == "gemm_splitk"
+    c = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
+    flags = torch.ones(3, dtype=torch.int64, device="cuda")
+    binding.launch(a.cuda(), b.cuda(), c, 1, 20, BM, BN, 64, 8,
+                   cur_wave_sizes=_table([[M, N, 128]] * 3), wave_offsets=_table([[0, 0, 256], [0, 0, 0], [0, 0, 128]]),
+                   signal_ptr=flags, signal_offsets=_table([0, 1, 2]), cum_tiles=3 * M * N)
+    check_status()
+    assert _rel(c, numerics.gemm_fp32(a, b)) <= 3 * REL_TOL

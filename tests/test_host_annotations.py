@@ -115,8 +115,11 @@ def test_template_choice():
     assert attention.tile_shape == ("1", "1", "BQ")
     assert [n for n, _ in attention.extra_args] == ["wave_offsets", "wave_sizes", "cum_wave_sizes", "signal_ptr",
                                                     "signal_offsets", "cum_tiles", "NUM_WAVES"]
+    split_k = AnnotationTransformer(enable_consumer=True).transform(snippets["gemm_split_k_persistent"])
+    assert split_k.template == "gemm_splitk" and split_k.persistent and split_k.tile_shape == ("BM", "BN")
+    assert [a.kind for a in split_k.annotations.axis_counts] == ["single", "single", "range"]
     with pytest.raises(AnnotationError, match="no HIP template"):
-        AnnotationTransformer().transform(snippets["split_k_has_no_template"])
+        AnnotationTransformer().transform(snippets["batched_rows_have_no_template"])
     with pytest.raises(AnnotationError, match="producer_epilogue"):
         AnnotationTransformer(enable_producer=True).transform(snippets["attention_with_kv_range"])
     with pytest.raises(ValueError):
