@@ -230,6 +230,13 @@ typedef struct syn_attn_desc {
                                        tile bumps counters[wave] and the tile that completes a wave
                                        (Z*H*Q blocks of it) sets flags[signal_offsets[wave]] to 1   */
     int32_t options;                /* SYN_ATTN_* bits                                                */
+    const uint64_t* wait_flags;     /* with counters only, both or neither: a second flag array and the   */
+    const int32_t* wait_signal_offsets; /* index per wave (-1: none) this launch WAITS for before it reads
+                                       a wave's K and V, while it sets `flags` as a producer - the
+                                       transform pass with enable_consumer and enable_producer
+                                       (consumer_signal_ptr / consumer_signal_offsets beside the
+                                       producer's, transformer.py:1077-1123,
+                                       tests/test_all2all_attn_all2all.py:192-210)                    */
 } syn_attn_desc;
 
 /* syn_attn_desc.options: one workgroup of eight wavefronts takes two consecutive q blocks (tiles

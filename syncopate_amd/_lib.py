@@ -126,6 +126,8 @@ class AttnDesc(ctypes.Structure):
         ("o_strides", c_int64 * 3),
         ("counters", c_void_p),
         ("options", c_int32),
+        ("wait_flags", c_void_p),
+        ("wait_signal_offsets", c_void_p),
     ]
 
 

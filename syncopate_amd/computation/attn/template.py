@@ -61,6 +61,8 @@ def attention_forward(
     num_programs: int = 0,
     counter_ptr: Optional[torch.Tensor] = None,
     output_buffer: Optional[torch.Tensor] = None,
+    consumer_signal_ptr: Optional[torch.Tensor] = None,
+    consumer_signal_offsets: Optional[TableLike] = None,
     pair_q_blocks: bool = False,
     xcd_remap: bool = False,
     out: Optional[torch.Tensor] = None,
@@ -81,6 +83,9 @@ def attention_forward(
     bumps its wave's counter and the tile that completes a wave sets the wave's flag in
     `signal_ptr`.  `output_buffer` (alias of `out`) is the reference's name for the comm buffer
     the result is written into.
+    `consumer_signal_ptr` / `consumer_signal_offsets` (with `counter_ptr`): a second flag array
+    and the index per wave (-1: none) that the producer form waits for before it reads a wave's K
+    and V - the transform pass with both roles enabled (tests/test_all2all_attn_all2all.py:192-210).
     `pair_q_blocks` (an extension): one workgroup of eight wavefronts takes two consecutive q
     blocks and runs them half a kv block apart, the softmax of one beside the matrix products of
     the other, both reading K and V from the same LDS blocks.  Every wave must hold an even
@@ -149,6 +154,18 @@ def attention_forward(
         if counter_ptr.dtype != torch.int32 or counter_ptr.device != dev or not counter_ptr.is_contiguous() \
                 or counter_ptr.numel() < num_waves:
             raise ValueError("counter_ptr must be a contiguous int32 tensor with one word per wave on q's device")
+    wait_flags = wait_sigs = None
+    if (consumer_signal_ptr is None) != (consumer_signal_offsets is None):
+        raise ValueError("consumer_signal_ptr and consumer_signal_offsets go together")
+    if consumer_signal_ptr is not None:
+        if counter_ptr is None:
+            raise ValueError("without counter_ptr, signal_ptr itself is what the kernel waits for")
+        wait_flags = flag_buffer(consumer_signal_ptr)
+        wait_sigs = as_device_table(consumer_signal_offsets, dev, None)
+        hw = host_copy(wait_sigs)
+        if wait_sigs.numel() < num_waves or int(hw[:num_waves].min()) < -1 or \
+                int(hw[:num_waves].max()) >= wait_flags.numel():
+            raise ValueError("consumer_signal_offsets must hold one index into consumer_signal_ptr (or -1) per wave")
     o = torch.empty(q.shape, dtype=q.dtype, device=dev) if out is None else out
     if o.shape != q.shape or o.dtype != q.dtype:
         raise ValueError("out must match q")
@@ -174,6 +191,8 @@ def attention_forward(
         q_strides=strides(q), k_strides=strides(k), v_strides=strides(v), o_strides=strides(o),
         counters=None if counter_ptr is None else counter_ptr.data_ptr(),
         options=(_lib.SYN_ATTN_PAIR_Q_BLOCKS if pair_q_blocks else 0) | (_lib.SYN_ATTN_XCD_REMAP if xcd_remap else 0),
+        wait_flags=None if wait_flags is None else wait_flags.data_ptr(),
+        wait_signal_offsets=None if wait_sigs is None else wait_sigs.data_ptr(),
     )
     with torch.cuda.device(dev):
         _lib.check("syn_attn_fwd", lib.syn_attn_fwd(ctypes.byref(desc), _lib.stream_handle(stream)))

@@ -76,12 +76,15 @@ class KernelBinding:
         return tables
 
     def _signal_tables(self, tables: Mapping[str, Any]) -> Tuple[Any, Any, Any]:
-        """(flag words, per-wave flag offsets, tile counters) under whichever names the roles gave them."""
-        both = self.consumer and self.producer
-        if both:
-            raise NotImplementedError(
-                "a kernel that is consumer and producer at once waits on one flag array and reports "
-                "into another: neither HIP template takes two flag arrays")
+        """(flag words, per-wave flag offsets, tile counters) under whichever names the roles gave them;
+        with both roles these are the producer's, and the consumer's travel as a second pair."""
+        if self.consumer and self.producer:
+            if self.template != "attention":
+                raise NotImplementedError(
+                    "a GEMM that is consumer and producer at once waits on one flag array and reports "
+                    "into another: the GEMM templates take one flag array")
+            return (tables.get("producer_signal_ptr"), tables.get("producer_signal_offsets"),
+                    tables.get("producer_counter_ptr"))
         return tables.get("signal_ptr"), tables.get("signal_offsets"), tables.get("counter_ptr")
 
     def launch(self, *args, **kwargs):
@@ -161,6 +164,9 @@ class KernelBinding:
         if flags is None or flag_offsets is None:
             raise ValueError("signal_ptr and signal_offsets are required")
         waves = tables.get("NUM_WAVES") or None
+        if self.consumer and self.producer:
+            kwargs = dict(kwargs, consumer_signal_ptr=tables.get("consumer_signal_ptr"),
+                          consumer_signal_offsets=tables.get("consumer_signal_offsets"))
         return attention_forward(*args, wave_offsets=tables["wave_offsets"], wave_sizes=sizes,
                                  cum_wave_sizes=tables["cum_wave_sizes"], signal_ptr=flags,
                                  signal_offsets=flag_offsets, NUM_WAVES=waves,

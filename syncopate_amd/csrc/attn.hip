@@ -48,6 +48,8 @@ struct AttnParams {
     int32_t* visit_log;
     int32_t* status;
     int32_t* counters;
+    const uint64_t* wait_flags;          // producer form that is a consumer as well: flags to wait for ...
+    const int32_t* wait_offsets;         // ... and the index per wave (-1: none)
     int64_t timeout_ticks;
     int32_t num_waves;
     int32_t Z, H, Sq, Skv;
@@ -200,12 +202,15 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
         const int kv_end = p.causal ? min(kv_hi, qb + 1) : kv_hi;
         if (kv_lo >= kv_end) continue;
 
-        // producer form (counters given): the wave's flag is one this kernel SETS, nothing to wait for
-        if (sig >= 0 && p.counters == nullptr) {
+        // producer form (counters given): the wave's flag is one this kernel SETS; it waits only if a
+        // second flag array says what for (a kernel that consumes one exchange and feeds another)
+        const int wait_sig = p.wait_offsets != nullptr ? p.wait_offsets[w] : (p.counters == nullptr ? sig : -1);
+        if (wait_sig >= 0) {
             if (tid == 0) {
-                const bool ok = spin_until_equal(p.flags + sig, 1ull, p.timeout_ticks);
+                const uint64_t* wait_flags = p.wait_flags != nullptr ? p.wait_flags : p.flags;
+                const bool ok = spin_until_equal(wait_flags + wait_sig, 1ull, p.timeout_ticks);
                 if (!ok) {
-                    report_status(p.status, SYN_STATUS_SPIN_TIMEOUT, w, (int)blockIdx.x, sig);
+                    report_status(p.status, SYN_STATUS_SPIN_TIMEOUT, w, (int)blockIdx.x, wait_sig);
                     s_abort = 1;
                 }
             }
@@ -920,6 +925,8 @@ int syn_attn_fwd(const syn_attn_desc* d, syn_stream_t stream) {
     if (d->dtype != SYN_DTYPE_BF16 && d->dtype != SYN_DTYPE_FP16) return SYN_EINVAL;
     if (d->causal && d->Sq != d->Skv) return SYN_EINVAL;
     if (d->cum_tiles <= 0 || d->cum_tiles % kBlockM) return SYN_EINVAL;
+    if ((d->wait_flags == nullptr) != (d->wait_signal_offsets == nullptr)) return SYN_EINVAL;
+    if (d->wait_flags && !d->counters) return SYN_EINVAL;     // without counters `flags` is what is waited for
     if (!(d->sm_scale > 0.f)) return SYN_EINVAL;
     if (!aligned16(d->q) || !aligned16(d->k) || !aligned16(d->v) || !aligned16(d->o)) return SYN_EALIGN;
     if (d->visit_log && !aligned16(d->visit_log)) return SYN_EALIGN;
@@ -942,6 +949,8 @@ int syn_attn_fwd(const syn_attn_desc* d, syn_stream_t stream) {
     p.visit_log = d->visit_log;
     p.status = d->status;
     p.counters = d->counters;
+    p.wait_flags = d->wait_flags;
+    p.wait_offsets = d->wait_signal_offsets;
     p.timeout_ticks = timeout_ticks(d->spin_timeout_us);
     p.num_waves = d->num_waves;
     p.Z = d->Z;
@@ -973,7 +982,7 @@ int syn_attn_fwd(const syn_attn_desc* d, syn_stream_t stream) {
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     if (d->options & SYN_ATTN_PAIR_Q_BLOCKS) {
         // two q blocks per workgroup: the caller vouches for an even number of q blocks in every wave
-        if (d->causal || d->counters || tiles % 2) return SYN_EINVAL;
+        if (d->causal || d->counters || d->wait_flags || d->wait_signal_offsets || tiles % 2) return SYN_EINVAL;
         int grid = d->num_programs > 0 ? d->num_programs : (int)(tiles / 2);
         if (grid > tiles / 2) grid = (int)(tiles / 2);
         return d->dtype == SYN_DTYPE_BF16 ? launch_attn_pairs<__bf16>(p, grid, s)

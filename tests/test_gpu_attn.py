@@ -29,6 +29,15 @@ def _kv_waves(Z, H, Sq, chunks, signals):
     return offsets, sizes, cums, list(signals), total
 
 
+def _attention_snippet():
+    """The annotated attention kernel of the annotation fixture (a producer needs an epilogue mark on top)."""
+    import json
+    import os
+
+    path = os.path.join(os.path.dirname(__file__), "golden", "annotation_cases.json")
+    return json.load(open(path))["snippets"]["attention_with_kv_range"]
+
+
 def _rel(out, ref):
     return ((out.float().cpu() - ref).abs().max() / ref.abs().max()).item()
 
@@ -203,3 +212,58 @@ def test_paired_q_blocks_argument_errors(hip):
     with pytest.raises(ValueError):
         attention_forward(q2, k2, v2, 0.1, pair_q_blocks=True,
                           counter_ptr=torch.zeros(1, dtype=torch.int32, device="cuda"), **kw)
+
+
+def test_producer_form_that_also_waits(hip):
+    """Both roles at once (tests/test_all2all_attn_all2all.py:192-245: consumer_signal_* beside the
+    producer's): the kernel waits for a wave's consumer flag before it reads that wave's K and V,
+    and counts finished tiles into the producer's flags."""
+    from syncopate_amd import _lib
+    from syncopate_amd.communication.comm_runtime.streams import pick_side_streams
+    from syncopate_amd.computation.attn import attention_forward
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.transform import AnnotationTransformer
+
+    Z, H, Sq, Skv = 1, 2, 256, 1024
+    q, k, v = _qkv(Z, H, Sq, Skv, torch.float16, seed=9)
+    chunks = [(0, 256), (256, 512), (512, 768), (768, 1024)]
+    offsets, sizes, cums, _, total = _kv_waves(Z, H, Sq, chunks, [0, 1, 2, 3])
+    sm_scale = 128 ** -0.5
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    staged_k, staged_v = kd.clone(), vd.clone()
+    kd[:, :, 512:].fill_(float("nan"))        # the last two chunks arrive late
+    vd[:, :, 512:].fill_(float("nan"))
+    wait_flags = torch.zeros(2, dtype=torch.int64, device="cuda")
+    done_flags = torch.zeros(4, dtype=torch.int64, device="cuda")
+    counters = torch.zeros(4, dtype=torch.int32, device="cuda")
+    side = pick_side_streams(1)[0]
+    main = torch.cuda.current_stream()
+    side.wait_stream(main)
+    binding = AnnotationTransformer(enable_consumer=True, enable_producer=True, consumer_descriptors=("desc_q",)) \
+        .transform(_attention_snippet().replace("    attend(", "    # @sy.producer_epilogue\n    attend("))
+    assert binding.template == "attention"
+    out = binding.launch(qd, kd, vd, sm_scale, wave_offsets=offsets, wave_sizes=sizes, cum_wave_sizes=cums,
+                         NUM_WAVES=4, cum_tiles=total, producer_signal_ptr=done_flags,
+                         producer_signal_offsets=[0, 1, 2, 3], producer_counter_ptr=counters,
+                         consumer_signal_ptr=wait_flags, consumer_signal_offsets=[-1, -1, 0, 1],
+                         spin_timeout_us=3_000_000)
+    lib = _lib.load()
+    for i, (lo, hi) in enumerate(chunks[2:]):
+        _lib.check("syn_delay_us", lib.syn_delay_us(300, _lib.stream_handle(side)))
+        with torch.cuda.stream(side):
+            kd[:, :, lo:hi].copy_(staged_k[:, :, lo:hi])
+            vd[:, :, lo:hi].copy_(staged_v[:, :, lo:hi])
+        _lib.check("syn_flag_set", lib.syn_flag_set(wait_flags.data_ptr() + 8 * i, 1, _lib.stream_handle(side)))
+    main.wait_stream(side)
+    check_status()
+    assert _rel(out, numerics.sdpa_fp32(q, k, v, sm_scale)) <= REL_TOL
+    assert done_flags.tolist() == [1, 1, 1, 1] and counters.tolist() == [Z * H * Sq // 128] * 4
+    # argument errors of the second flag pair
+    with pytest.raises(ValueError):
+        attention_forward(qd, kd, vd, sm_scale, wave_offsets=offsets, wave_sizes=sizes, cum_wave_sizes=cums,
+                          signal_ptr=done_flags, signal_offsets=[0, 1, 2, 3], cum_tiles=total,
+                          consumer_signal_ptr=wait_flags, consumer_signal_offsets=[-1, -1, 0, 1])     # no counters
+    with pytest.raises(ValueError):
+        attention_forward(qd, kd, vd, sm_scale, wave_offsets=offsets, wave_sizes=sizes, cum_wave_sizes=cums,
+                          signal_ptr=done_flags, signal_offsets=[0, 1, 2, 3], cum_tiles=total, counter_ptr=counters,
+                          consumer_signal_ptr=wait_flags, consumer_signal_offsets=[-1, -1, 0, 2])     # beyond the array
