@@ -786,3 +786,61 @@ def test_gemm_all2all_gemm_chain(hip, rank):
     # four partial products rounded to fp16 and added; the reference bounds the chain by 5e-1
     assert _rel(out, want) <= 4 * REL_TOL
     assert ctx.recv_signal_bufs[rank].tolist() == [1] * world
+
+
+def test_all2all_then_split_k_gemm(hip):
+    """Attention output [B, S, H/W, D] per rank -> all-to-all (heads gathered, sequence scattered,
+    4-D boxes copied on compute units) -> output projection over the gathered heads, a source
+    rank's heads at a time (tests/test_all2all_gemm.py:80-160, 222-275)."""
+    from syncopate_amd.communication.code_gen import CodeGenOptions, CommGenerator
+    from syncopate_amd.communication.comm_runtime.communication_context import CommContext
+    from syncopate_amd.communication.common_descriptors import build_all_to_all_plan_dim
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.gemm import gemm_splitk
+    from syncopate_amd.interface import lower_comm_plan_to_raw_schedules
+
+    world, rank, B, S, H, D, BM, BN = 4, 3, 2, 512, 8, 128, 128, 256
+    s_local, h_local, hidden = S // world, H // world, H * D
+    dtype = torch.float16
+    gen = CommGenerator({r: build_all_to_all_plan_dim(
+        shape=(B, S, h_local, D), dtype=dtype, mesh_size=world, rank=r, src_buffer="src", dst_buffer="dst",
+        src_split_axis=2, dst_split_axis=1, transfer_kind="push") for r in range(world)})
+    gen.plan_signals()
+    schedules = lower_comm_plan_to_raw_schedules(gen)
+    info = gen.generate_code_for_plan(CodeGenOptions(copy_engine=False))
+    info.local_world_size = info.world_size
+    info.num_copy_sms = 12
+    ctx = CommContext(rank, info)
+    assert tuple(ctx.comm_buffers["dst"][rank].shape) == (B, s_local, H, D)
+
+    g = torch.Generator().manual_seed(43)
+    attn_out = [(0.1 * torch.randn(B, S, h_local, D, generator=g)).to(dtype) for _ in range(world)]
+    w = (0.1 * torch.randn(hidden, hidden, generator=g)).to(dtype)
+    for r in range(world):
+        ctx.comm_buffers["src"][r].copy_(attn_out[r].cuda())
+    ctx.comm_buffers["dst"][rank].fill_(float("nan"))
+
+    dst = schedules[rank]["dst"]
+    shapes = [[b * s, hidden, h * d] for b, s, h, d in dst.gen_block_shape_lists()]
+    offsets = [[0, 0, oh * D + od] for _, _, oh, od in dst.gen_block_offset_lists()]
+    signals = dst.gen_signal_lists()
+    assert sorted(o[2] for o in offsets) == [q * h_local * D for q in range(world)]
+
+    gemm_input = ctx.comm_buffers["dst"][rank].reshape(-1, hidden)          # [B * S/W, H * D]
+    out = torch.zeros(gemm_input.shape[0], hidden, dtype=dtype, device="cuda")
+    ctx.reset_signals(whole_mesh=True)
+    ctx.start_after()
+    ctx.execute_mesh()
+    gemm_splitk(gemm_input, w.cuda(), out, world, 40, BM, BN, 64, 8, cur_wave_sizes=shapes, wave_offsets=offsets,
+                signal_ptr=ctx.recv_signal_bufs[rank], signal_offsets=signals,
+                cum_tiles=sum(s[0] * s[1] for s in shapes))
+    ctx.end_before()
+    check_status()
+    ctx.check_status()
+
+    # the exchange, restated: rank r keeps its sequence slice of every rank's heads
+    want_in = torch.cat([attn_out[q][:, rank * s_local:(rank + 1) * s_local] for q in range(world)], dim=2)
+    assert torch.equal(ctx.comm_buffers["dst"][rank].cpu(), want_in)
+    want = want_in.reshape(-1, hidden).float() @ w.float().t()
+    assert _rel(out, want) <= 4 * REL_TOL
+    assert ctx.recv_signal_bufs[rank].tolist() == [1] * world
