@@ -38,7 +38,7 @@ BM, BN, BK, GROUP_M = 256, 256, 64, 8
 NUM_SMS = 224                        # 448 tiles = 2 per program; 32 of the 256 CUs stay free for the
                                      # copy kernels of the producer
 XCD_REMAP = False                    # consecutive tile ids on one XCD (see --xcd-remap)
-LEAD_OPS = 1                         # ops of the side stream the consumer launch waits for (see fused_step)
+LEAD_OPS = 4                         # ops of the side stream the consumer launch waits for: two chunks and their flags
 EIGHT_WAVES = False                  # 256-thread workgroups: one wavefront per SIMD, 128x128 of C each
 
 
@@ -103,7 +103,7 @@ def run_ag_gemm(state, steps, warmup, resident_only=False, use_graph=True):
         ctx.reset_signals()               # switches to the zeroed flag set
         ctx.start_after(cur)
         ctx.execute(lead_ops=LEAD_OPS)
-        ctx.wait_lead(cur)                # the kernel starts behind the first chunk's copy
+        ctx.wait_lead(cur)                # the kernel starts behind the first two chunks (copies are 3x faster before it does)
         consumer(ctx.recv_signal_bufs[RANK])
         ctx.end_before(cur)
 
