@@ -7,7 +7,8 @@ A step is one fused all-gather+GEMM iteration of rank 0 of a simulated mesh of 8
 copied into the symmetric buffer on a side stream in the order the lowered schedule
 prescribes (copy, then flag), the consumer GEMM (8192 x 8192 x 3584) on the compute stream
 waiting on each chunk's flag.  All operands are resident in HBM before the timed region.
-Prints ONE JSON line.
+The W warm-up steps follow SETTLE_STEPS further untimed steps (an idle device's clocks settle
+over the first ~10 ms of work); the timed region is exactly K steps.  Prints ONE JSON line.
 """
 
 from __future__ import annotations
@@ -37,6 +38,9 @@ M, K, N, WORLD, RANK = 8192, 8192, 3584, 8, 0
 BM, BN, BK, GROUP_M = 256, 256, 64, 8
 NUM_SMS = 224                        # 448 tiles = 2 per program; 32 of the 256 CUs stay free for the
                                      # copy kernels of the producer
+SETTLE_STEPS = 40                    # untimed steps ahead of the W warm-up steps: the clocks of an idle device
+                                     # take some ten milliseconds of this work to settle (20 steps behind 5
+                                     # warm-up steps measure 0.49 ms per step, behind 40 of them 0.43 ms)
 XCD_REMAP = False                    # consecutive tile ids on one XCD (see --xcd-remap)
 LEAD_OPS = 4                         # ops of the side stream the consumer launch waits for: two chunks and their flags
 EIGHT_WAVES = False                  # 256-thread workgroups: one wavefront per SIMD, 128x128 of C each
@@ -108,10 +112,12 @@ def run_ag_gemm(state, steps, warmup, resident_only=False, use_graph=True):
         ctx.end_before(cur)
 
     # One step is ~25 launches (7 copies, 7 flag writes, flag reset, stream joins, the GEMM):
-    # replayed as HIP graphs so that the host's launch rate is not what gets measured (kernels
-    # and memcpy nodes only).  A graph holds an even number of steps, since consecutive steps
-    # use alternate flag sets: two for the warm-up, all timed steps in one; an odd step count
-    # ends with one step launched from the host.
+    # replayed as a HIP graph so that the host's launch rate is not what gets measured (kernels
+    # and memcpy nodes only).  The graph holds two steps, since consecutive steps use alternate
+    # flag sets; the warm-up replays it, the timed region replays it steps/2 times (the first
+    # replay of a graph pays for its instantiation on the device: ~1.5 ms for 20 steps' nodes,
+    # which a graph of all timed steps replayed once would book as 60 us per step); an odd step
+    # count ends with one step launched from the host.
     def capture(n):
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
@@ -131,23 +137,22 @@ def run_ag_gemm(state, steps, warmup, resident_only=False, use_graph=True):
         fused_step()
         fused_step()
     torch.cuda.synchronize()
-    timed_in_graph = steps - steps % 2
-    warm_graph = capture(2) if use_graph else None
-    timed_graph = capture(timed_in_graph) if use_graph and timed_in_graph else None
+    pair_graph = capture(2) if use_graph else None
 
     # ---- gated run: the step the metric is quoted on ----
-    wall_ms = gated_kernel_ms = None
+    wall_ms = gated_kernel_ms = no_lead_kernel_ms = None
     if not resident_only:
-        for _ in range((warmup + 1) // 2):
+        for _ in range(SETTLE_STEPS // 2 + (warmup + 1) // 2):
             if use_graph:
-                warm_graph.replay()
+                pair_graph.replay()
             else:
                 fused_step()
                 fused_step()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        if timed_graph is not None:          # EXACTLY `steps` fused steps, nothing else on the streams
-            timed_graph.replay()
+        if pair_graph is not None:           # EXACTLY `steps` fused steps, nothing else on the streams
+            for _ in range(steps // 2):
+                pair_graph.replay()
             if steps % 2:
                 fused_step()
         else:
@@ -155,19 +160,26 @@ def run_ag_gemm(state, steps, warmup, resident_only=False, use_graph=True):
                 fused_step()
         torch.cuda.synchronize()
         wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-        # the same steps once more with HIP events around the consumer launch (event markers
-        # perturb the overlap slightly, so they stay out of the timed region above)
-        begin, end = _events(steps), _events(steps)
-        for i in range(steps):
-            ctx.reset_signals()
-            ctx.start_after(stream)
-            ctx.execute()
-            begin[i].record(stream)
-            consumer(ctx.recv_signal_bufs[RANK])
-            end[i].record(stream)
-            ctx.end_before(stream)
-        torch.cuda.synchronize()
-        gated_kernel_ms = sum(s.elapsed_time(e) for s, e in zip(begin, end)) / steps
+        # the same steps once more, launched from the host, with HIP events around the consumer
+        # launch (event markers perturb the overlap slightly, so they stay out of the timed region
+        # above); then a few with the kernel launched together with the first copy instead of
+        # behind the leading chunks
+        def kernel_ms(count, lead):
+            begin, end = _events(count), _events(count)
+            for i in range(count):
+                ctx.reset_signals()
+                ctx.start_after(stream)
+                ctx.execute(lead_ops=lead)
+                if lead:
+                    ctx.wait_lead(stream)
+                begin[i].record(stream)
+                consumer(ctx.recv_signal_bufs[RANK])
+                end[i].record(stream)
+                ctx.end_before(stream)
+            torch.cuda.synchronize()
+            return sum(s.elapsed_time(e) for s, e in zip(begin, end)) / count
+        gated_kernel_ms = kernel_ms(steps, LEAD_OPS)
+        no_lead_kernel_ms = kernel_ms(min(steps, 20), 0) if LEAD_OPS else gated_kernel_ms
     check_status()
     ctx.check_status()
 
@@ -185,8 +197,8 @@ def run_ag_gemm(state, steps, warmup, resident_only=False, use_graph=True):
     resident_kernel_ms = sum(s.elapsed_time(e) for s, e in zip(begin, end)) / steps
     check_status()
     if resident_only:
-        wall_ms = gated_kernel_ms = resident_kernel_ms
-    return wall_ms, gated_kernel_ms, resident_kernel_ms
+        wall_ms = gated_kernel_ms = no_lead_kernel_ms = resident_kernel_ms
+    return wall_ms, gated_kernel_ms, no_lead_kernel_ms, resident_kernel_ms
 
 
 def traffic_calibration(device):
@@ -376,8 +388,9 @@ def main():
     global BM, BN, NUM_SMS, LEAD_OPS, XCD_REMAP
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    # a step is ~0.45 ms: the defaults time a few hundred of them (the whole run still takes well under a minute)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="launch every step's operations from the host "
                     "instead of replaying them as one HIP graph")
@@ -419,7 +432,7 @@ def main():
                  "(--copy-blocks N) and launches from the host (--no-graph; a graph's kernel nodes carry no mask)")
     state = build_ag_gemm(device, args.copy_blocks, args.split_device, args.fuse_flags)
     with torch.cuda.stream(state["ctx"].compute_stream):
-        wall_ms, gated_ms, resident_ms = run_ag_gemm(state, args.steps, args.warmup, args.resident_only,
+        wall_ms, gated_ms, no_lead_ms, resident_ms = run_ag_gemm(state, args.steps, args.warmup, args.resident_only,
                                                      not args.no_graph)
     torch.cuda.synchronize()
     traffic_calibration(device)
@@ -439,6 +452,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "settle_steps": SETTLE_STEPS,
         "ms_per_step": wall_ms,
         "higher_is_better": True,
         "scaling": "weak",
@@ -457,12 +471,14 @@ def main():
                 if args.fuse_flags else
                 ("hipMemcpyAsync" if args.copy_blocks == 0 else f"copy kernel of {args.copy_blocks} workgroups")
                 + " + flag-set kernel per chunk"),
-            "launch": "eager" if args.no_graph else "one hip graph replay of all timed steps",
+            "launch": "eager" if args.no_graph else "a hip graph of two steps, replayed steps/2 times",
             "split_device": state["ctx"].cu_split,
         },
         "pct_bf16_mfma_peak": 100.0 * value / MFMA_BF16_PEAK_TFLOPS,
         "flag_wait_overhead_pct": 100.0 * (gated_ms - resident_ms) / resident_ms,
+        "step_over_resident_kernel_pct": 100.0 * (wall_ms - resident_ms) / resident_ms,
         "kernel_ms_gated": gated_ms,
+        "kernel_ms_gated_launched_with_first_copy": no_lead_ms,
         "kernel_ms_resident": resident_ms,
         "resident_tflops": flop / (resident_ms * 1e-3) / 1e12,
         "rs_reduce_GBps": reduce_bytes / (reduce_ms * 1e-3) / 1e9,
