@@ -107,6 +107,18 @@ int syn_gemm_consumer(const syn_gemm_desc* desc, syn_stream_t stream);
 int syn_gemm_producer(const syn_gemm_desc* desc, syn_stream_t stream);
 
 /*
+ * A GEMM in both roles: the producer above that, before the first tile of a wave, also waits
+ * (acquire) until wait_flags[wait_signal_offsets[wave]] == 1 where that index is >= 0 - e.g. the
+ * GEMM of a tensor-parallel layer whose A arrives by all-gather and whose C leaves by
+ * reduce-scatter.  `wait_flags` (device, 8-byte words) is a flag array of its own: `desc->flags`
+ * stays what the launch SETS.  Replaces the kernel the reference's transformer generates when a
+ * source carries consumer and producer annotations at once
+ * (syncopate/computation/transform/transformer.py:759-901, both passes applied).
+ */
+int syn_gemm_consumer_producer(const syn_gemm_desc* desc, const uint64_t* wait_flags,
+                               const int32_t* wait_signal_offsets, syn_stream_t stream);
+
+/*
  * Remote bindings of a GEMM launch: per wave, A is read from a peer's shard and / or the C
  * tile goes into a peer's buffer instead of the local one.  Counterpart of the reference's
  * dl.symm_at(ptr, target_rank) rebinding: kernel_gemm_ag_read_remote

@@ -135,6 +135,7 @@ class AttnDesc(ctypes.Structure):
 _SIGNATURES = {
     "syn_gemm_consumer": (c_int32, [POINTER(GemmDesc), c_void_p]),
     "syn_gemm_producer": (c_int32, [POINTER(GemmDesc), c_void_p]),
+    "syn_gemm_consumer_producer": (c_int32, [POINTER(GemmDesc), c_void_p, c_void_p, c_void_p]),
     "syn_gemm_remote_binding": (c_int32, [POINTER(GemmDesc), POINTER(GemmRemote), c_void_p]),
     "syn_gemm_check_waves": (
         c_int32,

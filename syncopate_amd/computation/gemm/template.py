@@ -58,6 +58,8 @@ def _launch(
     two_stage: bool,
     spin_timeout_us: int,
     stream: Optional[torch.cuda.Stream],
+    wait_signal_buffer: Optional[torch.Tensor] = None,
+    wait_signal_offsets: Optional[TableLike] = None,
 ) -> None:
     # shape/dtype contract of the reference launchers (template.py:177-185)
     assert a.shape[1] == b.shape[1], "Incompatible dimensions"  # b is [N, K]
@@ -95,6 +97,20 @@ def _launch(
         )
         if caller_owned:
             remember_checked(tables, params)
+
+    wait_flags = wait_sigs = None
+    if (wait_signal_buffer is None) != (wait_signal_offsets is None):
+        raise ValueError("the flags to wait for and their per-wave indices come together")
+    if wait_signal_buffer is not None:
+        if not producer:
+            raise ValueError("a consumer waits on its signal buffer: a second flag array is for a producer that also waits")
+        wait_flags = flag_buffer(wait_signal_buffer)
+        wait_sigs = as_device_table(wait_signal_offsets, dev, None)
+        if wait_sigs.numel() != num_waves:
+            raise ValueError("one index to wait for per wave (-1: none)")
+        hw = host_copy(wait_sigs)
+        if int(hw.min()) < -1 or int(hw.max()) >= wait_flags.numel():
+            raise ValueError("an index to wait for is outside its flag array")
 
     if producer:
         if counter_buffer is None:
@@ -139,6 +155,11 @@ def _launch(
         | (_lib.SYN_GEMM_TWO_STAGE if two_stage else 0),
     )
     with torch.cuda.device(dev):
+        if wait_flags is not None:
+            _lib.check("syn_gemm_consumer_producer",
+                       lib.syn_gemm_consumer_producer(ctypes.byref(desc), wait_flags.data_ptr(), wait_sigs.data_ptr(),
+                                                      _lib.stream_handle(stream)))
+            return
         fn = lib.syn_gemm_producer if producer else lib.syn_gemm_consumer
         name = "syn_gemm_producer" if producer else "syn_gemm_consumer"
         _lib.check(name, fn(ctypes.byref(desc), _lib.stream_handle(stream)))
@@ -237,6 +258,8 @@ def gemm(
     signal_ptr,
     signal_offsets,
     counter_ptr=None,
+    consumer_signal_ptr=None,
+    consumer_signal_offsets=None,
     cum_tiles=0,
     visit_log=None,
     xcd_remap=True,
@@ -250,8 +273,12 @@ def gemm(
     """Call form of the launcher the reference's transform pass emits for the
     annotated persistent GEMM (tests/computation/transform/examples/
     example_persistent_gemm.py:125-181; extra arguments transformer.py:1139-1149):
-    a consumer when `counter_ptr` is None, a producer otherwise.
+    a consumer when `counter_ptr` is None, a producer otherwise.  A producer given
+    `consumer_signal_ptr` and `consumer_signal_offsets` (one index per wave, -1: none) is a
+    consumer as well: it waits for those flags wave by wave and sets `signal_ptr`'s - both
+    passes of the transform applied to one kernel.
     """
     _launch(counter_ptr is not None, a, b, c, signal_ptr, cur_wave_sizes, wave_offsets, signal_offsets,
             num_gemm_sms, BLOCK_SIZE_M, BLOCK_SIZE_N, BLOCK_SIZE_K, GROUP_SIZE_M, cum_tiles,
-            counter_ptr, visit_log, xcd_remap, eight_waves, ring_pipe, k_stagger, two_stage, spin_timeout_us, stream)
+            counter_ptr, visit_log, xcd_remap, eight_waves, ring_pipe, k_stagger, two_stage, spin_timeout_us, stream,
+            consumer_signal_ptr, consumer_signal_offsets)

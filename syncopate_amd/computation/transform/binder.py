@@ -79,10 +79,10 @@ class KernelBinding:
         """(flag words, per-wave flag offsets, tile counters) under whichever names the roles gave them;
         with both roles these are the producer's, and the consumer's travel as a second pair."""
         if self.consumer and self.producer:
-            if self.template != "attention":
+            if self.template == "gemm_splitk" or self.remote:
                 raise NotImplementedError(
-                    "a GEMM that is consumer and producer at once waits on one flag array and reports "
-                    "into another: the GEMM templates take one flag array")
+                    "both roles at once are bound for the GEMM template without peer descriptors and for "
+                    "the attention template")
             return (tables.get("producer_signal_ptr"), tables.get("producer_signal_offsets"),
                     tables.get("producer_counter_ptr"))
         return tables.get("signal_ptr"), tables.get("signal_offsets"), tables.get("counter_ptr")
@@ -127,6 +127,9 @@ class KernelBinding:
         if not self.remote:
             if flags is None or flag_offsets is None:
                 raise ValueError("signal_ptr and signal_offsets are required")
+            if self.consumer and self.producer:
+                kwargs = dict(kwargs, consumer_signal_ptr=tables.get("consumer_signal_ptr"),
+                              consumer_signal_offsets=tables.get("consumer_signal_offsets"))
             return gemm(*args, cur_wave_sizes=sizes, wave_offsets=tables["wave_offsets"], signal_ptr=flags,
                         signal_offsets=flag_offsets, counter_ptr=counters, cum_tiles=tables.get("cum_tiles", 0),
                         **kwargs)

@@ -34,6 +34,8 @@ struct GemmParams {
     const void* b;
     void* c;
     uint64_t* flags;
+    const uint64_t* wait_flags;          // producer that is a consumer as well: flags to wait for ...
+    const int32_t* wait_offsets;         // ... and the index per wave (-1: none)
     const int32_t* wave_sizes;
     const int32_t* wave_offsets;
     const int32_t* signal_offsets;
@@ -732,6 +734,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
     // --- wave walk state (uniform across the workgroup) ---
     int cur_wave = -1, past_tiles = 0, cur_tiles = 0;
     int cur_m = 0, cur_n = 0, off_m = 0, off_n = 0, cur_sig = -1;
+    int cur_wait = -1;            // flag index the wave waits for: its own signal (consumer), the second table's (producer)
     const T* a_base = nullptr;
     T* c_base = nullptr;
     int dst_m = 0, dst_n = 0;
@@ -751,6 +754,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
             off_n = p.wave_offsets[w * 2 + 1] / BN;
             cur_sig = p.signal_offsets[w];
         }
+        cur_wait = PRODUCER ? (p.wait_offsets != nullptr ? p.wait_offsets[w] : -1) : cur_sig;
         cur_tiles = cur_m * cur_n;
         if (REMOTE) {
             // the wave's peer: A rows are read from its shard and / or C tiles go into its buffer,
@@ -771,7 +775,8 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
 
     auto wait_flag = [&](int sig) -> bool {
         if (tid == 0) {
-            const bool ok = spin_until_equal(p.flags + sig, 1ull, p.timeout_ticks);
+            const uint64_t* flags = PRODUCER ? p.wait_flags : p.flags;
+            const bool ok = spin_until_equal(flags + sig, 1ull, p.timeout_ticks);
             if (!ok) {
                 report_status(p.status, SYN_STATUS_SPIN_TIMEOUT, cur_wave, pid, sig);
                 s_abort = 1;
@@ -783,10 +788,8 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
     };
 
     // the reference's consumer waits for wave 0 before it looks at its first tile (template.py:92-97)
-    if (!PRODUCER) {
-        if (cur_sig >= 0) {
-            if (!wait_flag(cur_sig)) return;
-        }
+    if (cur_wait >= 0) {
+        if (!wait_flag(cur_wait)) return;
     }
 
     const T* __restrict__ A = reinterpret_cast<const T*>(p.a);
@@ -806,7 +809,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
             enter_wave(cur_wave + 1);
             new_wave = true;
         }
-        return !PRODUCER && new_wave && cur_sig >= 0;
+        return new_wave && cur_wait >= 0;
     };
 
     struct Tile {
@@ -865,7 +868,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
 
     if (tiles_here == 0) return;
     if (advance(pid)) {
-        if (!wait_flag(cur_sig)) return;
+        if (!wait_flag(cur_wait)) return;
     }
     if (cur_wave < 0) return;
     Tile tile = locate(pid);
@@ -979,7 +982,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
         }
 
         if (has_next && gated) {
-            if (!wait_flag(cur_sig)) return;
+            if (!wait_flag(cur_wait)) return;
             next = locate(next_id);
             Pipe::prologue(panel_a(next), panel_b(next), row_bytes, next.k_len, next.k_rot, lane, wave);
         }
@@ -1036,9 +1039,12 @@ static int dispatch_pipe(const GemmParams& p, int bm, int bn, bool eight, bool r
 }
 
 static int gemm_entry(const syn_gemm_desc* d, hipStream_t stream, int mode,
-                      const syn_gemm_remote* remote = nullptr) {
+                      const syn_gemm_remote* remote = nullptr, const uint64_t* wait_flags = nullptr,
+                      const int32_t* wait_signal_offsets = nullptr) {
     if (d == nullptr) return SYN_EINVAL;
     const bool producer = mode == kProducer;
+    if ((wait_flags == nullptr) != (wait_signal_offsets == nullptr)) return SYN_EINVAL;
+    if (wait_flags && !producer) return SYN_EINVAL;      // a consumer waits on `flags` itself
     const bool a_remote = remote && remote->a_peers, c_remote = remote && remote->c_peers;
     if (mode == kRemote) {
         if (!remote || (!a_remote && !c_remote)) return SYN_EINVAL;
@@ -1073,6 +1079,8 @@ static int gemm_entry(const syn_gemm_desc* d, hipStream_t stream, int mode,
     p.b = d->b;
     p.c = d->c;
     p.flags = d->flags;
+    p.wait_flags = wait_flags;
+    p.wait_offsets = wait_signal_offsets;
     p.wave_sizes = d->wave_sizes;
     p.wave_offsets = d->wave_offsets;
     p.signal_offsets = d->signal_offsets;
@@ -1123,6 +1131,13 @@ int syn_gemm_consumer(const syn_gemm_desc* desc, syn_stream_t stream) {
 
 int syn_gemm_producer(const syn_gemm_desc* desc, syn_stream_t stream) {
     return syn::gemm_entry(desc, reinterpret_cast<hipStream_t>(stream), syn::kProducer);
+}
+
+int syn_gemm_consumer_producer(const syn_gemm_desc* desc, const uint64_t* wait_flags,
+                               const int32_t* wait_signal_offsets, syn_stream_t stream) {
+    if (wait_flags == nullptr || wait_signal_offsets == nullptr) return SYN_EINVAL;
+    return syn::gemm_entry(desc, reinterpret_cast<hipStream_t>(stream), syn::kProducer, nullptr, wait_flags,
+                           wait_signal_offsets);
 }
 
 int syn_gemm_remote_binding(const syn_gemm_desc* desc, const syn_gemm_remote* remote, syn_stream_t stream) {

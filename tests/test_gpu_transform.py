@@ -74,6 +74,63 @@ def test_gemm_bindings_consumer_producer_and_one_tile_per_program(hip):
     assert torch.equal(c3, plain)
 
 
+def test_gemm_in_both_roles_waits_on_one_flag_array_and_reports_into_another(hip):
+    """Consumer and producer annotations on one kernel (both transform passes applied): the GEMM
+    waits for a wave's consumer flag before it reads that wave's rows of A and counts finished tiles
+    into the producer's flags.  The last two row chunks of A arrive late, on a side stream."""
+    from syncopate_amd import _lib
+    from syncopate_amd.communication.comm_runtime.streams import pick_side_streams
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.gemm import gemm
+    from syncopate_amd.computation.transform import AnnotationTransformer
+
+    M, N, K, BM, BN, world = 1024, 512, 256, 128, 128, 4
+    g = torch.Generator().manual_seed(13)
+    a_full = (0.05 * torch.randn(M, K, generator=g)).bfloat16().cuda()
+    b = (0.05 * torch.randn(N, K, generator=g)).bfloat16().cuda()
+    rows = M // world
+    sizes = [[rows, N]] * world
+    offsets = [[i * rows, 0] for i in range(world)]
+    a = a_full.clone()
+    a[2 * rows:].fill_(float("nan"))          # chunks 2 and 3 are not there yet
+    wait_flags = torch.zeros(2, dtype=torch.int64, device="cuda")
+    done_flags = torch.zeros(world, dtype=torch.int64, device="cuda")
+    counters = torch.zeros(world, dtype=torch.int32, device="cuda")
+    c = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
+    side = pick_side_streams(1)[0]
+    main = torch.cuda.current_stream()
+    side.wait_stream(main)
+    both = AnnotationTransformer(enable_consumer=True, enable_producer=True) \
+        .transform(SNIPPETS["gemm_persistent_with_epilogue"])
+    assert both.template == "gemm" and both.consumer and both.producer
+    both.launch(a, b, c, world, 40, BM, BN, 64, 8, cur_wave_sizes=_table(sizes), wave_offsets=_table(offsets),
+                producer_signal_ptr=done_flags, producer_signal_offsets=_table([0, 1, 2, 3]),
+                producer_counter_ptr=counters, consumer_signal_ptr=wait_flags,
+                consumer_signal_offsets=_table([-1, -1, 0, 1]), cum_tiles=M * N, spin_timeout_us=3_000_000)
+    lib = _lib.load()
+    for i in range(2):
+        _lib.check("syn_delay_us", lib.syn_delay_us(300, _lib.stream_handle(side)))
+        with torch.cuda.stream(side):
+            a[(2 + i) * rows:(3 + i) * rows].copy_(a_full[(2 + i) * rows:(3 + i) * rows])
+        _lib.check("syn_flag_set", lib.syn_flag_set(wait_flags.data_ptr() + 8 * i, 1, _lib.stream_handle(side)))
+    main.wait_stream(side)
+    check_status()
+    assert _rel(c, numerics.gemm_fp32(a_full.cpu(), b.cpu())) <= REL_TOL
+    assert done_flags.tolist() == [1] * world and counters.tolist() == [(rows // BM) * (N // BN)] * world
+
+    # the second flag pair: both or neither, with counters only, indices inside the array
+    kw = dict(cur_wave_sizes=_table(sizes), wave_offsets=_table(offsets), signal_ptr=done_flags,
+              signal_offsets=_table([0, 1, 2, 3]), cum_tiles=M * N)
+    with pytest.raises(ValueError):
+        gemm(a_full, b, c, world, 40, BM, BN, 64, 8, consumer_signal_ptr=wait_flags,
+             consumer_signal_offsets=_table([-1, -1, 0, 1]), **kw)                             # no counters
+    with pytest.raises(ValueError):
+        gemm(a_full, b, c, world, 40, BM, BN, 64, 8, counter_ptr=counters, consumer_signal_ptr=wait_flags, **kw)
+    with pytest.raises(ValueError):
+        gemm(a_full, b, c, world, 40, BM, BN, 64, 8, counter_ptr=counters, consumer_signal_ptr=wait_flags,
+             consumer_signal_offsets=_table([-1, -1, 0, 2]), **kw)                             # beyond the array
+
+
 def test_gemm_binding_with_a_peer_bound_result(hip):
     """Reduce-scatter by direct reduction inside the kernel (tests/test_gemm_rs_direct_reduce.py:102-192):
     the schedule of the push plan makes `c_desc` a producer-side, reducing descriptor, so every

@@ -160,5 +160,9 @@ def test_launch_checks_its_tables_before_touching_the_device():
     with pytest.raises(ValueError, match="counter_ptr"):
         producer.launch(None, None, None, 4, 8, cur_wave_sizes=[[1, 1]], wave_offsets=[[0, 0]])
     both = AnnotationTransformer(enable_consumer=True, enable_producer=True).transform(source)
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(ValueError, match="counter_ptr"):          # the producer's tables go by producer_* names
         both.launch(None, None, None, 4, 8, cur_wave_sizes=[[1, 1]], wave_offsets=[[0, 0]])
+    split = AnnotationTransformer(enable_consumer=True, enable_producer=True) \
+        .transform(GOLDEN["snippets"]["gemm_split_k_persistent"])
+    with pytest.raises(NotImplementedError):                      # both roles: GEMM and attention templates only
+        split.launch(None, None, None, 4, 8, cur_wave_sizes=[[1, 1, 1]], wave_offsets=[[0, 0, 0]])
