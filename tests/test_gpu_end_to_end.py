@@ -104,6 +104,79 @@ def test_gemm_rs_iteration(hip, rank, shape):
     assert _rel(out, total) <= 2e-2
 
 
+@pytest.mark.parametrize("rank", [0, 3])
+def test_allgather_gemm_reduce_scatter_in_one_kernel(hip, rank):
+    """One GEMM in both roles between two plans: the row chunks of A arrive by all-gather (copy,
+    then flag, on side streams), the GEMM waits for a chunk's flag before the wave that reads it,
+    and every finished wave's rows of the partial result are pushed to their owner behind the
+    wave's COMPUTE_DONE flag.  The waves follow the producer's order (peers' chunks first), so the
+    first wave already waits for a remote chunk."""
+    from syncopate_amd.communication.comm_runtime.communication_context import CommContext
+    from syncopate_amd.communication.common_descriptors import build_all_gather_plan_1d_swizzle, build_all_to_all_plan
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.gemm import gemm
+    from syncopate_amd.interface.wave_tables import gemm_consumer_tables, gemm_producer_tables
+
+    world, M, N, K, BM, BN, programs = 4, 1024, 512, 256, 128, 128, 13
+    rows = M // world
+    g = torch.Generator().manual_seed(21 + rank)
+    a = (0.1 * torch.randn(M, K, generator=g)).bfloat16()
+    b = (0.1 * torch.randn(N, K, generator=g)).bfloat16()
+
+    gather_plans = {r: build_all_gather_plan_1d_swizzle((M, K), torch.bfloat16, 0, world, r, "a", "pull")
+                    for r in range(world)}
+    gather_schedules, gather_info = _compile(gather_plans)
+    scatter_plans = {r: build_all_to_all_plan(shape=(M, N), dtype=torch.bfloat16, mesh_size=world, rank=r,
+                                              src_buffer="src", dst_buffer="dst", transfer_kind="push",
+                                              compute_producer=True) for r in range(world)}
+    scatter_schedules, scatter_info = _compile(scatter_plans)
+    arrival = gemm_consumer_tables(gather_schedules[rank]["a"], N)        # which flag announces which row chunk
+    flag_of_chunk = {off[0] // rows: sig for off, sig in zip(arrival.block_offsets, arrival.signal_offsets)}
+    waves = gemm_producer_tables(scatter_schedules[rank]["src"])           # the kernel's waves, owner by owner
+    wait_for = [flag_of_chunk[off[0] // rows] for off in waves.block_offsets]
+    assert wait_for.count(-1) == 1 and wait_for[-1] == -1                  # only the rank's own chunk is resident
+
+    gather = CommContext(rank, gather_info)
+    scatter = CommContext(rank, scatter_info)
+    for r in range(world):                 # every rank's symmetric buffer holds its own shard, NaN elsewhere
+        gather.comm_buffers["a"][r].fill_(float("nan"))
+        gather.comm_buffers["a"][r][r * rows:(r + 1) * rows].copy_(a[r * rows:(r + 1) * rows])
+    src = scatter.comm_buffers["src"][rank]
+    src.fill_(float("nan"))
+    bd = b.cuda()
+    counters = torch.zeros(world, dtype=torch.int32, device="cuda")
+    comm_stream = torch.cuda.Stream()
+    main = torch.cuda.current_stream()
+
+    gather.reset_signals()
+    scatter.reset_signals()
+    comm_stream.wait_stream(main)
+    gather.start_after(main)
+    gather.execute()                       # ahead of the scatter's spinning waits on any queue they share
+    gemm(gather.comm_buffers["a"][rank], bd, src, world, programs, BM, BN, 64, 8,
+         cur_wave_sizes=waves.block_shapes, wave_offsets=waves.block_offsets,
+         signal_ptr=scatter.compute_signal_bufs[rank], signal_offsets=waves.signal_offsets, counter_ptr=counters,
+         consumer_signal_ptr=gather.recv_signal_bufs[rank], consumer_signal_offsets=wait_for,
+         cum_tiles=waves.cum_tiles)
+    scatter.start_after(comm_stream)
+    scatter.execute(neglect_local=True)
+    scatter.end_before(comm_stream)
+    gather.end_before(main)
+    main.wait_stream(comm_stream)
+    check_status()
+    gather.check_status()
+    scatter.check_status()
+
+    assert torch.equal(gather.comm_buffers["a"][rank].cpu(), a)
+    partial = numerics.gemm_fp32(a, b)
+    assert _rel(src, partial) <= REL_TOL
+    assert scatter.compute_signal_bufs[rank].tolist() == [1] * world
+    assert counters.tolist() == [(rows // BM) * (N // BN)] * world
+    for peer in range(world):
+        if peer != rank:
+            assert torch.equal(scatter.comm_buffers["dst"][peer][rank], src[peer * rows:(peer + 1) * rows])
+
+
 @pytest.mark.parametrize("rank,layout", [(1, "bhsd"), (3, "bhsd"), (2, "bshd")])
 def test_allgather_attention_iteration(hip, rank, layout):
     """K/V chunks pulled from their owners on a side stream (copy, then flag) while the
