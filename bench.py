@@ -42,7 +42,8 @@ SETTLE_STEPS = 40                    # untimed steps ahead of the W warm-up step
                                      # take some ten milliseconds of this work to settle (20 steps behind 5
                                      # warm-up steps measure 0.49 ms per step, behind 40 of them 0.43 ms)
 XCD_REMAP = False                    # consecutive tile ids on one XCD (see --xcd-remap)
-LEAD_OPS = 4                         # ops of the side stream the consumer launch waits for: two chunks and their flags
+LEAD_OPS = 3                         # ops of the side stream the consumer launch waits for: two chunks copied, the
+                                     # first one's flag set (the second flag lands while the first tiles run)
 EIGHT_WAVES = False                  # 256-thread workgroups: one wavefront per SIMD, 128x128 of C each
 
 
@@ -107,7 +108,7 @@ def run_ag_gemm(state, steps, warmup, resident_only=False, use_graph=True):
         ctx.reset_signals()               # switches to the zeroed flag set
         ctx.start_after(cur)
         ctx.execute(lead_ops=LEAD_OPS)
-        ctx.wait_lead(cur)                # the kernel starts behind the first two chunks (copies are 3x faster before it does)
+        ctx.wait_lead(cur)                # the kernel starts behind the first two chunk copies (3x faster before it does)
         consumer(ctx.recv_signal_bufs[RANK])
         ctx.end_before(cur)
 
@@ -466,6 +467,7 @@ def main():
                         "fp32 accumulate",
             "tile": [BM, BN, BK],
             "programs": NUM_SMS,
+            "lead_ops": LEAD_OPS,
             "producer": "side stream: " + (
                 f"one kernel of {args.copy_blocks} workgroups per chunk that copies, then sets the flag"
                 if args.fuse_flags else
