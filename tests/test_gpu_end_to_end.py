@@ -231,6 +231,64 @@ def test_allgather_attention_iteration(hip, rank, layout):
     assert (log[:, 0] >= 0).all()                    # every tile of every wave ran
 
 
+@pytest.mark.parametrize("kind,rank", [("ring", 1), ("double_ring", 2)])
+def test_ring_allgather_attention_over_the_mesh(hip, kind, rank):
+    """K/V forwarded round a ring, or round two nested rings, instead of pulled from their owners
+    (tests/test_ring_allgather_attn_transform.py:160-230, tests/test_double_ring_ag_attn.py:160-230):
+    a chunk reaches this rank only after its upstream neighbours have received and forwarded it,
+    so every rank's op list is replayed; the attention kernel walks the waves in arrival order."""
+    from syncopate_amd.communication.comm_runtime.communication_context import CommContext
+    from syncopate_amd.communication.common_descriptors import (
+        build_double_ring_all_gather_plan,
+        build_ring_all_gather_plan,
+    )
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.attn import attention_forward
+    from syncopate_amd.interface.wave_tables import allgather_attn_tables, plan_layout_spec
+
+    world, B, H, SEQ, D = 4, 1, 2, 1024, 128
+    per_rank = SEQ // world
+    shape, seq_axis, axes = plan_layout_spec("bhsd", B, H, SEQ, D)
+    if kind == "ring":
+        plans = {r: build_ring_all_gather_plan(shape, torch.bfloat16, seq_axis, world, r, "kv") for r in range(world)}
+    else:
+        plans = {r: build_double_ring_all_gather_plan(shape, torch.bfloat16, seq_axis, world, 2, r, "kv")
+                 for r in range(world)}
+    schedules, info = _compile(plans)
+    tables = allgather_attn_tables(schedules[rank]["kv"], per_rank, axes)
+    arrival = [off[3] // per_rank for off in tables.wave_offsets]
+    assert sorted(arrival) == list(range(world)) and arrival[0] == rank
+    if kind == "ring":
+        assert arrival == [(rank - k) % world for k in range(world)]
+    assert tables.signal_offsets[0] == -1 and all(sig >= 0 for sig in tables.signal_offsets[1:])
+
+    g = torch.Generator().manual_seed(15)
+    kv = torch.randn(*shape, generator=g).bfloat16()
+    q = torch.randn(B, H, per_rank, D, generator=g).bfloat16()
+    ctx = CommContext(rank, info, link_delay_us=10)
+    for r in range(world):
+        own = [slice(None)] * 5
+        own[seq_axis] = slice(r * per_rank, (r + 1) * per_rank)
+        ctx.comm_buffers["kv"][r][tuple(own)].copy_(kv[tuple(own)])
+    buf = ctx.comm_buffers["kv"][rank]
+    main = torch.cuda.current_stream()
+
+    ctx.reset_signals(whole_mesh=True)
+    ctx.start_after(main)
+    ctx.execute_mesh()
+    out = attention_forward(q.cuda(), buf[0], buf[1], D ** -0.5, wave_offsets=tables.wave_offsets,
+                            wave_sizes=tables.wave_sizes, cum_wave_sizes=tables.cum_wave_sizes,
+                            signal_ptr=ctx.recv_signal_bufs[rank], signal_offsets=tables.signal_offsets,
+                            NUM_WAVES=len(tables.signal_offsets), cum_tiles=tables.cum_tiles)
+    ctx.end_before(main)
+    check_status()
+    ctx.check_status()
+
+    for r in range(world):                           # the gather completed on every simulated rank
+        assert torch.equal(ctx.comm_buffers["kv"][r].cpu(), kv), f"rank {r}"
+    assert _rel(out, numerics.sdpa_fp32(q, kv[0], kv[1], D ** -0.5)) <= REL_TOL
+
+
 def test_all2all_attention_iteration_with_graph_replay(hip):
     """Ulysses exchange of stacked Q/K/V captured as a HIP graph (the reference captures the
     comm side, tests/test_all2all_attn_transform.py:278) and replayed several times: every
