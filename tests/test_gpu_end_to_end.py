@@ -919,23 +919,32 @@ def test_gemm_all2all_gemm_chain(hip, rank):
     assert ctx.recv_signal_bufs[rank].tolist() == [1] * world
 
 
-def test_all2all_then_split_k_gemm(hip):
+@pytest.mark.parametrize("slices", [0, 2])
+def test_all2all_then_split_k_gemm(hip, slices):
     """Attention output [B, S, H/W, D] per rank -> all-to-all (heads gathered, sequence scattered,
     4-D boxes copied on compute units) -> output projection over the gathered heads, a source
-    rank's heads at a time (tests/test_all2all_gemm.py:80-160, 222-275)."""
+    rank's heads at a time (tests/test_all2all_gemm.py:80-160, 222-275).  With `slices` every
+    shard is pulled in that many slices of the sequence, each a wave of its own
+    (build_all_to_all_plan_dim_waves, tests/test_all2all_gemm_split_collective.py:212-240)."""
     from syncopate_amd.communication.code_gen import CodeGenOptions, CommGenerator
     from syncopate_amd.communication.comm_runtime.communication_context import CommContext
-    from syncopate_amd.communication.common_descriptors import build_all_to_all_plan_dim
+    from syncopate_amd.communication.common_descriptors import build_all_to_all_plan_dim, build_all_to_all_plan_dim_waves
     from syncopate_amd.computation._launch import check_status
     from syncopate_amd.computation.gemm import gemm_splitk
     from syncopate_amd.interface import lower_comm_plan_to_raw_schedules
 
-    world, rank, B, S, H, D, BM, BN = 4, 3, 2, 512, 8, 128, 128, 256
+    world, rank, S, H, D, BM, BN = 4, 3, 1024 if slices else 512, 8, 128, 128, 256
+    B = 1 if slices else 2            # a slice of the sequence is one run of GEMM rows only for a single batch
     s_local, h_local, hidden = S // world, H // world, H * D
     dtype = torch.float16
-    gen = CommGenerator({r: build_all_to_all_plan_dim(
-        shape=(B, S, h_local, D), dtype=dtype, mesh_size=world, rank=r, src_buffer="src", dst_buffer="dst",
-        src_split_axis=2, dst_split_axis=1, transfer_kind="push") for r in range(world)})
+    common = dict(shape=(B, S, h_local, D), dtype=dtype, mesh_size=world, src_buffer="src", dst_buffer="dst",
+                  src_split_axis=2, dst_split_axis=1)
+    if slices:
+        gen = CommGenerator({r: build_all_to_all_plan_dim_waves(rank=r, transfer_kind="pull", num_waves=slices, **common)
+                             for r in range(world)})
+    else:
+        gen = CommGenerator({r: build_all_to_all_plan_dim(rank=r, transfer_kind="push", **common)
+                             for r in range(world)})
     gen.plan_signals()
     schedules = lower_comm_plan_to_raw_schedules(gen)
     info = gen.generate_code_for_plan(CodeGenOptions(copy_engine=False))
@@ -953,9 +962,12 @@ def test_all2all_then_split_k_gemm(hip):
 
     dst = schedules[rank]["dst"]
     shapes = [[b * s, hidden, h * d] for b, s, h, d in dst.gen_block_shape_lists()]
-    offsets = [[0, 0, oh * D + od] for _, _, oh, od in dst.gen_block_offset_lists()]
+    offsets = [[ob * s_local + os_, 0, oh * D + od] for ob, os_, oh, od in dst.gen_block_offset_lists()]
     signals = dst.gen_signal_lists()
-    assert sorted(o[2] for o in offsets) == [q * h_local * D for q in range(world)]
+    assert sorted(o[2] for o in offsets) == sorted(q * h_local * D for q in range(world) for _ in range(max(slices, 1)))
+    assert len(shapes) == world * max(slices, 1)
+    if slices:
+        assert sorted({o[0] for o in offsets}) == [i * (s_local // slices) for i in range(slices)]
 
     gemm_input = ctx.comm_buffers["dst"][rank].reshape(-1, hidden)          # [B * S/W, H * D]
     out = torch.zeros(gemm_input.shape[0], hidden, dtype=dtype, device="cuda")
@@ -974,4 +986,4 @@ def test_all2all_then_split_k_gemm(hip):
     assert torch.equal(ctx.comm_buffers["dst"][rank].cpu(), want_in)
     want = want_in.reshape(-1, hidden).float() @ w.float().t()
     assert _rel(out, want) <= 4 * REL_TOL
-    assert ctx.recv_signal_bufs[rank].tolist() == [1] * world
+    assert ctx.recv_signal_bufs[rank].tolist() == [1] * len(shapes)
