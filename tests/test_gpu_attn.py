@@ -94,7 +94,8 @@ def test_causal_extension_matches_sdpa(hip):
 
 def test_hand_template_form_resident(hip):
     """attention(q, k, v, sm_scale, wave_dicts) with the everything-resident table
-    (reference: syncopate/computation/attn/template.py:442-497, kv_divide waves)."""
+    (reference: syncopate/computation/attn/template.py:442-497, kv_divide waves; the hand-written
+    kernel is driven the same way in tests/test_allgather_attn.py:20-40, 70-120)."""
     from syncopate_amd.computation.attn import attention, build_waves_and_signals_divisible
     from syncopate_amd.computation._launch import check_status
 

@@ -20,23 +20,28 @@ def _rel(out, ref):
     return ((out.float().cpu() - ref.float()).abs().max() / ref.float().abs().max()).item()
 
 
-def _compile(plans):
+def _compile(plans, options=None):
     from syncopate_amd.communication.code_gen import CommGenerator
     from syncopate_amd.interface import lower_comm_plan_to_raw_schedules
 
     gen = CommGenerator(plans)
     gen.plan_signals()
     schedules = lower_comm_plan_to_raw_schedules(gen)
-    info = gen.generate_code_for_plan()
+    info = gen.generate_code_for_plan(options) if options is not None else gen.generate_code_for_plan()
     info.local_world_size = info.world_size
     return schedules, info
 
 
-@pytest.mark.parametrize("rank,shape", [(0, (4, 1024, 512, 256, 128, 128, 13)), (2, (4, 1024, 512, 256, 128, 128, 13)),
-                                        (5, (8, 8192, 4096, 512, 256, 256, 224))])
-def test_gemm_rs_iteration(hip, rank, shape):
+@pytest.mark.parametrize("rank,shape,copy_units", [(0, (4, 1024, 512, 256, 128, 128, 13), 0),
+                                                   (2, (4, 1024, 512, 256, 128, 128, 13), 0),
+                                                   (5, (8, 8192, 4096, 512, 256, 256, 224), 0),
+                                                   (1, (4, 1024, 512, 256, 128, 128, 13), 8)])
+def test_gemm_rs_iteration(hip, rank, shape, copy_units):
     """Producer GEMM -> comm stream waits on each wave's COMPUTE_DONE flag and pushes the chunk
-    to its owner -> ring reduce of the received partials."""
+    to its owner -> ring reduce of the received partials.  With `copy_units` the pushes are box
+    copies on that many compute units instead of copy-engine ops (CodeGenOptions(copy_engine=False),
+    tests/test_gemm_rs_sm.py:92-135)."""
+    from syncopate_amd.communication.code_gen import CodeGenOptions
     from syncopate_amd.communication.comm_runtime.communication_context import CommContext
     from syncopate_amd.communication.common_descriptors import build_all_to_all_plan
     from syncopate_amd.computation._launch import check_status
@@ -54,7 +59,9 @@ def test_gemm_rs_iteration(hip, rank, shape):
     plans = {r: build_all_to_all_plan(shape=(M, N), dtype=torch.bfloat16, mesh_size=world, rank=r,
                                       src_buffer="src", dst_buffer="dst", transfer_kind="push",
                                       compute_producer=True) for r in range(world)}
-    schedules, info = _compile(plans)
+    schedules, info = _compile(plans, CodeGenOptions(copy_engine=False) if copy_units else None)
+    if copy_units:
+        info.num_copy_sms = copy_units
     tables = gemm_producer_tables(schedules[rank]["src"])
     # the chunk a peer owns is computed (and shipped) before the rank's own chunk
     assert [off[0] // rows for off in tables.block_offsets] == [(rank + 1 + i) % world for i in range(world)]
@@ -756,7 +763,9 @@ def test_gemm_rs_sm_reduce_iteration(hip, kind, rank, split):
 @pytest.mark.parametrize("form", ["reduce_scatter", "all_reduce", "all_reduce_two_buffers"])
 def test_gemm_then_library_collective_whole_mesh(hip, form):
     """Producer GEMM -> per slab: wait for its COMPUTE_DONE flag, one collective of the mesh, one
-    RECEIVE flag (tests/test_gemm_rs_collective.py:90-165, tests/test_gemm_ar_collective.py).  The
+    RECEIVE flag (tests/test_gemm_rs_collective.py:90-165, tests/test_gemm_ar_collective.py,
+    tests/test_gemm_ar_collective_nvsharp.py; the second GEMM of tests/test_domino_alike_mlp_collective.py:121-200
+    and tests/test_domino_alike_mlp_collective_nvsharp.py is this flow on an MLP's shapes).  The
     other ranks' partial products are computed beforehand; this rank's kernel runs beside the
     replay of the mesh, which carries each collective out over the ranks' buffers."""
     from syncopate_amd.communication.code_gen import CommGenerator

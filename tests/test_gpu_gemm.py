@@ -121,7 +121,8 @@ def test_consumer_group_size_and_column_waves(hip):
 
 def test_consumer_gated_by_side_stream_producer(hip):
     """Chunks land in the symmetric buffer on a side stream (copy, then flag) while the
-    consumer is already running; the result must be bitwise the resident one."""
+    consumer is already running; the result must be bitwise the resident one (the flow of
+    tests/test_ag_gemm_hand.py:19-45, 70-130 with the hand-written consumer)."""
     from syncopate_amd import _lib
     from syncopate_amd.communication.comm_runtime.streams import pick_side_streams
     from syncopate_amd.computation.gemm import gemm_consumer
