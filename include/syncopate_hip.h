@@ -161,6 +161,13 @@ int syn_gemm_remote_binding(const syn_gemm_desc* desc, const syn_gemm_remote* re
  * the tables they get live in device memory.  All pointers are HOST pointers.
  * Returns 0, SYN_EINVAL or SYN_ERANGE.  No reference counterpart: the
  * reference launches unchecked (template.py:177-185 asserts shapes only).
+ *
+ * CALLERS FROM C: syn_gemm_consumer / _producer / _consumer_producer /
+ * _remote_binding and syn_attn_fwd do NOT validate wave tables (they are in
+ * device memory); a table that names rows beyond an operand or a flag beyond
+ * its array makes the kernel read or write out of bounds.  Call
+ * syn_gemm_check_waves / syn_attn_check_waves on the host copy of every new
+ * table before its first launch, as the Python launchers do.
  */
 int syn_gemm_check_waves(const int32_t* wave_sizes, const int32_t* wave_offsets,
                          const int32_t* signal_offsets, int32_t num_waves,

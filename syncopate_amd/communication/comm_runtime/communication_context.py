@@ -473,7 +473,15 @@ class CommContext:
 
     def get_graph(self) -> torch.cuda.CUDAGraph:
         """Capture start_after / execute / end_before into a HIP graph.  The op list
-        consists of memcpy nodes and small kernels only (no memset nodes)."""
+        consists of memcpy nodes and small kernels only (no memset nodes).
+
+        A graph holds the flag pointers of the set that is current at capture.  With two flag
+        sets `reset_signals()` switches sets between iterations, and a replay would keep
+        writing the first set while the kernels wait on the other: refused.  (Capture two
+        iterations, reset_signals() included, into a graph of one's own instead.)"""
+        if len(self._flag_sets) != 1:
+            raise RuntimeError("get_graph() captures one flag set: not with flag_sets=2, where reset_signals() "
+                               "alternates between two (capture two whole iterations instead)")
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             self.start_after(torch.cuda.current_stream(self.device))

@@ -3,6 +3,8 @@
 from __future__ import annotations
 
 import ctypes
+import functools
+import inspect
 import weakref
 from typing import Dict, Optional, Sequence, Tuple, Union
 
@@ -50,6 +52,25 @@ def check_status(device: Optional[torch.device] = None, *, reset: bool = True) -
                     f"signal offset {words[3]}"
                 )
             raise RuntimeError(f"kernel status {words} on cuda:{idx}")
+
+
+def launches_on_stream(fn):
+    """Decorator of a launcher with a `stream` argument: the whole call - wave tables built
+    from lists or CPU tensors, zeroed counters, locks, outputs, and the kernel launch - runs
+    with `stream` as torch's current stream.  The temporaries' fills are then ordered in front
+    of the kernel, and the caching allocator hands their memory on only behind it."""
+    sig = inspect.signature(fn)
+
+    @functools.wraps(fn)
+    def wrapper(*args, **kwargs):
+        bound = sig.bind(*args, **kwargs)
+        stream = bound.arguments.get("stream")
+        if stream is None:
+            return fn(*args, **kwargs)
+        with torch.cuda.stream(stream):
+            return fn(*args, **kwargs)
+
+    return wrapper
 
 
 def as_device_table(table: TableLike, device: torch.device, width: Optional[int]) -> torch.Tensor:

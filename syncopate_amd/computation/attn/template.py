@@ -33,6 +33,7 @@ from .._launch import (
     flag_buffer,
     host_copy,
     host_ptr,
+    launches_on_stream,
     remember_checked,
     require_cuda,
     status_words,
@@ -43,6 +44,7 @@ BLOCK_N = 128
 DEFAULT_SPIN_TIMEOUT_US = 2_000_000
 
 
+@launches_on_stream
 def attention_forward(
     q: torch.Tensor,
     k: torch.Tensor,

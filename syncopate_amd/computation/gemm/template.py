@@ -26,6 +26,7 @@ from .._launch import (
     flag_buffer,
     host_copy,
     host_ptr,
+    launches_on_stream,
     remember_checked,
     require_cuda,
     status_words,
@@ -34,6 +35,7 @@ from .._launch import (
 DEFAULT_SPIN_TIMEOUT_US = 2_000_000
 
 
+@launches_on_stream
 def _launch(
     producer: bool,
     a: torch.Tensor,

@@ -25,7 +25,8 @@ from typing import Optional, Sequence
 import torch
 
 from ... import _lib
-from .._launch import TableLike, as_device_table, host_copy, host_ptr, require_cuda, status_words
+from .._launch import (TableLike, as_device_table, host_copy, host_ptr, launches_on_stream, require_cuda,
+                       status_words)
 
 _pointer_tables: dict = {}
 
@@ -51,6 +52,7 @@ def _check_ranks(name: str, ranks: torch.Tensor, count: int, num_waves: int) -> 
         raise ValueError(f"{name} names a rank outside 0..{count - 1}")
 
 
+@launches_on_stream
 def gemm_remote(
     a,
     b: torch.Tensor,

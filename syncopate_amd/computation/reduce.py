@@ -14,11 +14,12 @@ from typing import Optional
 import torch
 
 from .. import _lib
-from ._launch import require_cuda
+from ._launch import launches_on_stream, require_cuda
 
 ACC_MODES = {"dtype": 0, "fp32": 1}
 
 
+@launches_on_stream
 def ring_reduce(
     input: torch.Tensor,         # [W, M_per_rank, N] received partials (slot begin_idx unused)
     output: torch.Tensor,        # [M_per_rank, N]

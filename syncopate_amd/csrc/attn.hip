@@ -198,9 +198,25 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
             rec[1] = make_int4(kv_lo, kv_hi, sig, (int)blockIdx.x);
         }
 
-        // causal: kv blocks strictly above the diagonal contribute nothing
+        // producer form (generated epilogue, transform/transformer.py:880-901): count the tile in
+        // its wave; the tile that completes the wave (all z, h and q blocks of it: the kv range is
+        // not counted) publishes the wave's flag.  Called by one thread, behind the tile's stores.
+        auto count_tile = [&]() {
+            if (p.counters != nullptr && sig >= 0) {
+                const int wave_tiles = p.wave_sizes[w * 4 + 0] * size_h * nq;
+                const int done = __hip_atomic_fetch_add(p.counters + w, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+                if (done == wave_tiles - 1)
+                    __hip_atomic_store(p.flags + sig, 1ull, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+            }
+        };
+
+        // causal: kv blocks strictly above the diagonal contribute nothing; a tile that lies wholly
+        // above it has no output of its own but still counts towards its wave
         const int kv_end = p.causal ? min(kv_hi, qb + 1) : kv_hi;
-        if (kv_lo >= kv_end) continue;
+        if (kv_lo >= kv_end) {
+            if (tid == 0) count_tile();
+            continue;
+        }
 
         // producer form (counters given): the wave's flag is one this kernel SETS; it waits only if a
         // second flag array says what for (a kernel that consumes one exchange and feeds another)
@@ -464,15 +480,7 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
         if (tid == 0) {
             __hip_atomic_store(p.first + lock_idx, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __hip_atomic_store(p.lock + lock_idx, 0, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-            // producer form (generated epilogue, transform/transformer.py:880-901): count the tile
-            // in its wave; the tile that completes the wave (all z, h and q blocks of it: the kv
-            // range is not counted) publishes the wave's flag
-            if (p.counters != nullptr && sig >= 0) {
-                const int wave_tiles = p.wave_sizes[w * 4 + 0] * size_h * nq;
-                const int done = __hip_atomic_fetch_add(p.counters + w, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-                if (done == wave_tiles - 1)
-                    __hip_atomic_store(p.flags + sig, 1ull, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
-            }
+            count_tile();
         }
     }
 }

@@ -268,3 +268,35 @@ def test_producer_form_that_also_waits(hip):
         attention_forward(qd, kd, vd, sm_scale, wave_offsets=offsets, wave_sizes=sizes, cum_wave_sizes=cums,
                           signal_ptr=done_flags, signal_offsets=[0, 1, 2, 3], cum_tiles=total, counter_ptr=counters,
                           consumer_signal_ptr=wait_flags, consumer_signal_offsets=[-1, -1, 0, 2])     # beyond the array
+
+
+def test_causal_producer_counts_tiles_above_the_diagonal(hip):
+    """Producer form under the causal mask: a (q block, kv chunk) tile that lies wholly above the
+    diagonal computes nothing, but it is one of its wave's tiles - every counter must reach the
+    wave's tile count and every flag must be published (a consumer of the flags would hang
+    otherwise).  Also on a stream that is not the current one, with the launcher's own
+    temporaries (tables from lists, locks, lse)."""
+    from syncopate_amd.computation.attn import attention_forward
+    from syncopate_amd.computation._launch import check_status
+
+    Z, H, S = 1, 2, 512
+    q, k, v = _qkv(Z, H, S, S, torch.bfloat16, seed=12)
+    chunks = [(0, 128), (128, 384), (384, 512)]
+    offsets, sizes, cums, _, total = _kv_waves(Z, H, S, chunks, [0, 1, 2])
+    scale = 128 ** -0.5
+    ref = numerics.sdpa_fp32(q, k, v, scale, causal=True)
+    side = torch.cuda.Stream()
+    for stream in (None, side):
+        flags = torch.zeros(3, dtype=torch.int64, device="cuda")
+        counters = torch.zeros(3, dtype=torch.int32, device="cuda")
+        qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+        torch.cuda.synchronize()
+        o = attention_forward(qd, kd, vd, scale, wave_offsets=offsets, wave_sizes=sizes, cum_wave_sizes=cums,
+                              signal_ptr=flags, signal_offsets=[0, 1, 2], cum_tiles=total, causal=True,
+                              counter_ptr=counters, spin_timeout_us=200_000, stream=stream)
+        if stream is not None:
+            stream.synchronize()
+        check_status()
+        assert counters.tolist() == [Z * H * S // 128] * 3
+        assert flags.tolist() == [1, 1, 1]
+        assert _rel(o, ref) <= REL_TOL

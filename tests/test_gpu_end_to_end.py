@@ -348,6 +348,9 @@ def test_all2all_attention_iteration_with_graph_replay(hip):
     want = numerics.sdpa_fp32(gathered[0], gathered[1], gathered[2], D ** -0.5)
     assert _rel(eager, want) <= REL_TOL
 
+    # with two flag sets a captured graph would keep writing the set of its capture: refused
+    with pytest.raises(RuntimeError, match="flag set"):
+        CommContext(rank, info, flag_sets=2).get_graph()
     graph = ctx.get_graph()
     comm_stream = torch.cuda.Stream()
     for replay in range(3):

@@ -169,3 +169,67 @@ def test_all2all_attention_16384_causal(hip):
             ref = torch.softmax(s, dim=-1) @ v[0, h].float()
             assert _rel(o[0, h], ref) <= REL_TOL
             del s, ref
+
+
+def test_c1_mesh4_fp16_gathered_4096x512_times_512x1024(hip):
+    """The reference's own CPU-runnable case on the HIP consumer: mesh of 4, 1-D swizzle pull,
+    per-rank A (1024, 512) fp16 gathered to (4096, 512), B (512, 1024), seed 0; every rank's wave
+    tables are the golden schedule the reference's compiler gives for this plan
+    (tests/golden/host_compiler.json, case ag_swizzle_pull_c1_gathered).  Result against the
+    fp32 matmul of the same fp16 values, visit log against the oracle, every rank, resident and
+    with the chunks arriving behind flags on a side stream."""
+    import json
+    import os
+
+    from oracle import numerics
+    from syncopate_amd import _lib
+    from syncopate_amd.communication.comm_runtime.streams import pick_side_streams
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.gemm import gemm_consumer
+
+    golden = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "host_compiler.json")))
+    schedules = golden["ag_swizzle_pull_c1_gathered"]["schedules"]
+    world, rows, K, N = 4, 1024, 512, 1024
+    M = world * rows
+    torch.manual_seed(0)
+    a = torch.cat([torch.randn(rows, K).half() for _ in range(world)])      # generated in rank order
+    b = torch.randn(K, N).half()
+    ref = numerics.gemm_fp32(a, b.t().contiguous())
+    ad, b_nk = a.cuda(), b.t().contiguous().cuda()
+    side = pick_side_streams(1)[0]
+    for rank in range(world):
+        sched = schedules[str(rank)]["a"]
+        assert sched["global_shape"] == [M, K]
+        offsets = [[o[0], 0] for o in sched["offsets"]]
+        sizes = [[s[0], N] for s in sched["shapes"]]
+        signals = sched["signals"]
+        assert [o[0] for o in offsets] == [((rank + k) % world) * rows for k in range(world)]
+        for BM, BN, num_sms in [(128, 128, 256), (256, 256, 48)]:
+            flags = torch.ones(world - 1, dtype=torch.int64, device="cuda")
+            c = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+            log = torch.full(((M // BM) * (N // BN), 4), -1, dtype=torch.int32, device="cuda")
+            gemm_consumer(ad, b_nk, c, flags, sizes, offsets, signals, world, num_sms, BM, BN, 64, 8,
+                          cum_tiles=M * N, visit_log=log)
+            check_status()
+            assert _rel(c.cpu(), ref) <= REL_TOL
+            _check_visit_log(log, sizes, offsets, signals, M, N, BM, BN, num_sms)
+        # gated: the symmetric buffer holds the own shard only (the rest poisoned); peers' chunks
+        # arrive on a side stream in schedule order, copy then flag
+        symm = torch.full((M, K), float("nan"), dtype=torch.float16, device="cuda")
+        symm[rank * rows:(rank + 1) * rows].copy_(ad[rank * rows:(rank + 1) * rows])
+        flags = torch.zeros(world - 1, dtype=torch.int64, device="cuda")
+        c_gated = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+        torch.cuda.synchronize()
+        side.wait_stream(torch.cuda.current_stream())
+        gemm_consumer(symm, b_nk, c_gated, flags, sizes, offsets, signals, world, 48, 256, 256, 64, 8,
+                      cum_tiles=M * N, spin_timeout_us=3_000_000)
+        nbytes = rows * K * 2
+        for wave in range(1, world):
+            row0 = offsets[wave][0]
+            _lib.check("syn_delay_us", hip.syn_delay_us(50, _lib.stream_handle(side)))
+            _lib.check("syn_copy_async", hip.syn_copy_async(symm.data_ptr() + row0 * K * 2, ad.data_ptr() + row0 * K * 2,
+                                                            nbytes, _lib.stream_handle(side)))
+            _lib.check("syn_flag_set", hip.syn_flag_set(flags.data_ptr() + 8 * signals[wave], 1, _lib.stream_handle(side)))
+        torch.cuda.current_stream().wait_stream(side)
+        check_status()
+        assert torch.equal(c_gated, c)          # same tile shape: bitwise the resident result

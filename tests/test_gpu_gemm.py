@@ -249,3 +249,40 @@ def test_consumer_256x224_tiles(hip, dtype):
         check_status()
         assert _max_rel_err(c, numerics.gemm_fp32(a, b)) <= REL_TOL
         _check_visits(log, sizes, offsets, signals, M, N, 256, 224, 8, num_sms, M * N, True)
+
+
+def test_launch_on_a_stream_that_is_not_current(hip):
+    """`stream=` with tables given as lists and no counter buffer: the device tables and the
+    zeroed counters the launcher creates must be filled on that stream, ahead of the kernel.
+    The stream is kept busy first so that a fill on the wrong stream would overtake nothing."""
+    from syncopate_amd import _lib
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.gemm import gemm_consumer, gemm_producer
+
+    M, N, K, world, rank = 1024, 512, 256, 4, 1
+    a, b = _inputs(M, N, K, torch.bfloat16, seed=11)
+    ad, bd = a.cuda(), b.cuda()
+    ref = numerics.gemm_fp32(a, b)
+    rows = M // world
+    sizes = [[rows, N]] * world
+    offsets = [[((rank + k + 1) % world) * rows, 0] for k in range(world)]
+    side = torch.cuda.Stream()
+    for trial in range(3):
+        flags = torch.zeros(world, dtype=torch.int64, device="cuda")
+        c = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
+        torch.cuda.synchronize()
+        _lib.check("syn_delay_us", hip.syn_delay_us(2000, _lib.stream_handle(side)))
+        gemm_producer(ad, bd, c, flags, sizes, offsets, list(range(world)), 64, 128, 128, cum_tiles=M * N,
+                      stream=side)
+        c2 = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
+        side.wait_stream(torch.cuda.current_stream())       # c2's fill
+        gemm_consumer(ad, bd, c2, flags, sizes, offsets, list(range(world)), world, 64, 128, 128, cum_tiles=M * N,
+                      stream=side)
+        # churn the allocator on the current stream while the side stream is still busy
+        junk = [torch.full((world,), 7, dtype=torch.int32, device="cuda") for _ in range(8)]
+        del junk
+        side.synchronize()
+        check_status()
+        assert flags.tolist() == [1] * world
+        assert _max_rel_err(c, ref) <= REL_TOL
+        assert torch.equal(c, c2)

@@ -116,6 +116,41 @@ def test_attention_tile_work_covers_every_q_kv_pair_once():
         visit_order.attn_tile_work(total // bm, offsets, sizes, cums, sigs)
 
 
+def test_attention_in_wave_order_matches_the_reference_generated_dispatch():
+    """The golden tuples come from the reference's own generated dispatch text evaluated tile by
+    tile (tests/golden/make_attn_dispatch_fixtures.py): q fastest, then h, then z inside a wave
+    (attn/template.py:39-44), wave offsets added afterwards (transformer.py:561-676)."""
+    import json
+    import os
+
+    golden = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "attn_dispatch_cases.json")))
+    bm, bn = golden["block_m"], golden["block_n"]
+    assert set(golden["cases"]) >= {"one_wave_z2_h3_q2", "ragged_offsets", "double_ring_w8_small"}
+    for name, case in golden["cases"].items():
+        assert len(case["tiles"]) == case["cum_wave_sizes"][-1] // bm
+        for tile_id, expect in enumerate(case["tiles"]):
+            w = visit_order.attn_tile_work(tile_id, case["wave_offsets"], case["wave_sizes"],
+                                           case["cum_wave_sizes"], case["signal_offsets"], block_m=bm, block_n=bn)
+            got = [w["wave"], w["z"], w["h"], w["q_block"], w["kv_lo"], w["kv_hi"], w["signal"]]
+            assert got == expect, (name, tile_id, got, expect)
+
+
+def test_attention_in_wave_order_hand_evaluated_literal():
+    """get_pid_range (attn/template.py:39-44) by hand for Z=2, H=3, two q blocks:
+    tile t -> q = t % 2, h = (t // 2) % 3, z = t // 6.  Swapping any two of z, h, q fails it."""
+    expect_zhq = [(0, 0, 0), (0, 0, 1), (0, 1, 0), (0, 1, 1), (0, 2, 0), (0, 2, 1),
+                  (1, 0, 0), (1, 0, 1), (1, 1, 0), (1, 1, 1), (1, 2, 0), (1, 2, 1)]
+    offsets, sizes, cums, sigs = [[0, 0, 0, 0]], [[2, 3, 256, 384]], [2 * 3 * 256], [-1]
+    for t, (z, h, q) in enumerate(expect_zhq):
+        w = visit_order.attn_tile_work(t, offsets, sizes, cums, sigs)
+        assert (w["z"], w["h"], w["q_block"], w["kv_lo"], w["kv_hi"]) == (z, h, q, 0, 3)
+    # a second wave at offsets (z 1, h 2, q block 1, kv block 2) of shape 1 x 2 x 2 q blocks x 1 kv block
+    offsets, sizes, cums, sigs = [[0, 0, 0, 0], [1, 2, 128, 256]], [[1, 1, 128, 128], [1, 2, 256, 128]], [128, 128 + 512], [-1, 3]
+    got = [visit_order.attn_tile_work(t, offsets, sizes, cums, sigs) for t in range(5)]
+    assert [(g["wave"], g["z"], g["h"], g["q_block"], g["kv_lo"], g["kv_hi"], g["signal"]) for g in got] == [
+        (0, 0, 0, 0, 0, 1, -1), (1, 1, 2, 1, 2, 3, 3), (1, 1, 2, 2, 2, 3, 3), (1, 1, 3, 1, 2, 3, 3), (1, 1, 3, 2, 2, 3, 3)]
+
+
 # ---------------------------------------------------------------- rounding and ring reduce
 
 def test_bf16_rounding_is_round_to_nearest_even():
