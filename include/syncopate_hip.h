@@ -32,6 +32,10 @@ extern "C" {
 #define SYN_EINVAL (-22)   /* malformed argument / unsupported configuration */
 #define SYN_ERANGE (-34)   /* wave table addresses tiles outside the operand  */
 #define SYN_EALIGN (-75)   /* pointer or extent not aligned as the kernel needs */
+#define SYN_E2BIG (-7)     /* more waves than the static scratch of syn_gemm_producer_static holds */
+
+/* capacity of syn_gemm_producer_static: waves per launch (one int32 counter each, 16 KB per device) */
+#define SYN_STATIC_MAX_WAVES 4096
 
 /* device-side status words (int32[SYN_STATUS_WORDS], caller-zeroed) */
 #define SYN_STATUS_WORDS 4
@@ -105,6 +109,21 @@ int syn_gemm_consumer(const syn_gemm_desc* desc, syn_stream_t stream);
  * (syncopate/computation/gemm/template.py:224-412).
  */
 int syn_gemm_producer(const syn_gemm_desc* desc, syn_stream_t stream);
+
+/*
+ * syn_gemm_producer for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
+ * reference, whose launcher allocates a zeroed counter tensor per call (template.py:388).
+ * desc->counters must be NULL: the per-wave tile counters live in a static device array of
+ * SYN_STATIC_MAX_WAVES words inside the library (each device holds its own copy until the
+ * process ends), cleared by a small fill kernel on `stream` in front of the GEMM.  The call
+ * itself allocates nothing and frees nothing.  More than SYN_STATIC_MAX_WAVES waves:
+ * SYN_E2BIG.  Every call on a device shares that device's array: calls that overlap on one
+ * device (two streams, two threads) race on the counters and must be serialised by the caller.
+ * The first call on a device looks the array's address up (hipGetSymbolAddress); make that
+ * call outside stream capture.
+ */
+int syn_gemm_producer_static(const syn_gemm_desc* desc, syn_stream_t stream);
 
 /*
  * A GEMM in both roles: the producer above that, before the first tile of a wave, also waits

@@ -21,6 +21,8 @@ SYN_DTYPE_FP16 = 1
 SYN_EINVAL = -22
 SYN_ERANGE = -34
 SYN_EALIGN = -75
+SYN_E2BIG = -7
+SYN_STATIC_MAX_WAVES = 4096
 SYN_STATUS_WORDS = 4
 SYN_STATUS_SPIN_TIMEOUT = 1
 SYN_GEMM_XCD_REMAP = 1
@@ -38,6 +40,8 @@ _ERRORS = {
     SYN_EINVAL: "SYN_EINVAL (malformed argument or unsupported configuration)",
     SYN_ERANGE: "SYN_ERANGE (wave table addresses tiles or flags outside the operands)",
     SYN_EALIGN: "SYN_EALIGN (pointer or extent not aligned as the kernel needs)",
+    SYN_E2BIG: "SYN_E2BIG (more waves than the static counter array of syn_gemm_producer_static holds: "
+               f"{SYN_STATIC_MAX_WAVES})",
 }
 
 
@@ -135,6 +139,7 @@ class AttnDesc(ctypes.Structure):
 _SIGNATURES = {
     "syn_gemm_consumer": (c_int32, [POINTER(GemmDesc), c_void_p]),
     "syn_gemm_producer": (c_int32, [POINTER(GemmDesc), c_void_p]),
+    "syn_gemm_producer_static": (c_int32, [POINTER(GemmDesc), c_void_p]),
     "syn_gemm_consumer_producer": (c_int32, [POINTER(GemmDesc), c_void_p, c_void_p, c_void_p]),
     "syn_gemm_remote_binding": (c_int32, [POINTER(GemmDesc), POINTER(GemmRemote), c_void_p]),
     "syn_gemm_check_waves": (

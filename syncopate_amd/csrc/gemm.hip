@@ -25,6 +25,8 @@
 // the flag word, then the whole workgroup takes an acquire fence (template.py:121-128).
 // Producer form: after the C tile is stored the workgroup bumps counters[wave] and the last
 // tile of the wave publishes the flag (template.py:343-348).
+#include <mutex>
+
 #include "common.h"
 
 namespace syn {
@@ -1121,9 +1123,65 @@ static int gemm_entry(const syn_gemm_desc* d, hipStream_t stream, int mode,
                     : dispatch_pipe<_Float16, kConsumer>(p, bm, bn, eight, ring, two, grid, stream);
 }
 
+// ---- the producer entry point that allocates nothing ----
+//
+// Its per-wave tile counters live in a file-scope device array instead of caller memory.  Every
+// device the library runs on holds its own copy of the array at its own address; the address is
+// looked up once per device and used from then on wherever host code needs the array's memory.
+constexpr int kStaticCounterWords = SYN_STATIC_MAX_WAVES;      // 16 KB per device
+static __device__ __align__(256) int32_t scratch[kStaticCounterWords];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static int32_t* g_scratch_ptr[kMaxDevices] = {};
+
+// device address of `scratch` on the current device (0, a SYN_E* code or a hipError_t)
+static int scratch_address(int32_t** out) {
+    int dev = -1;
+    hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess) return (int)err;
+    if (dev < 0 || dev >= kMaxDevices) return SYN_EINVAL;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* ptr = nullptr;
+        err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (err != hipSuccess) return (int)err;
+        if (ptr == nullptr) return (int)hipErrorInvalidSymbol;
+        g_scratch_ptr[dev] = reinterpret_cast<int32_t*>(ptr);
+    }
+    *out = g_scratch_ptr[dev];
+    return 0;
+}
+
+// a fill kernel rather than a memset: a memset node in a captured graph is not reliable on replay
+__global__ void __launch_bounds__(256) clear_words_kernel(int32_t* words, int n) {
+    const int i = (int)(blockIdx.x * blockDim.x + threadIdx.x);
+    if (i < n) words[i] = 0;
+}
+
 }  // namespace syn
 
 extern "C" {
+
+int syn_gemm_producer_static(const syn_gemm_desc* desc, syn_stream_t stream) {
+    using namespace syn;
+    if (desc == nullptr) return SYN_EINVAL;
+    if (desc->counters != nullptr) return SYN_EINVAL;        // the counters are the library's here
+    if (desc->num_waves <= 0) return SYN_EINVAL;
+    if (desc->num_waves > kStaticCounterWords) return SYN_E2BIG;
+    int32_t* counters = nullptr;
+    const int rc = scratch_address(&counters);
+    if (rc != 0) return rc;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    // the array keeps the last call's counts: the words this launch uses start at zero
+    hipLaunchKernelGGL(clear_words_kernel, dim3((desc->num_waves + 255) / 256), dim3(256), 0, s, counters,
+                       desc->num_waves);
+    const hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return (int)err;
+    syn_gemm_desc d = *desc;
+    d.counters = counters;
+    return gemm_entry(&d, s, kProducer);
+}
 
 int syn_gemm_consumer(const syn_gemm_desc* desc, syn_stream_t stream) {
     return syn::gemm_entry(desc, reinterpret_cast<hipStream_t>(stream), syn::kConsumer);
