@@ -1,14 +1,22 @@
-"""Benchmark of the chunk-scheduled AG+GEMM on one MI355X.
+"""Benchmark of the chunk-scheduled compute path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only ag_gemm,reduce,...]
 
-A step is one fused all-gather+GEMM iteration of rank 0 of a simulated mesh of 8
+The headline step is one fused all-gather+GEMM iteration of rank 0 of a simulated mesh of 8
 (M, K, N = 8192, 8192, 3584): flags reset, the 7 peer chunks of A (1024 x 8192 bf16 each)
 copied into the symmetric buffer on a side stream in the order the lowered schedule
 prescribes (copy, then flag), the consumer GEMM (8192 x 8192 x 3584) on the compute stream
 waiting on each chunk's flag.  All operands are resident in HBM before the timed region.
 The W warm-up steps follow SETTLE_STEPS further untimed steps (an idle device's clocks settle
 over the first ~10 ms of work); the timed region is exactly K steps.  Prints ONE JSON line.
+
+Beside the headline the same line carries the other workloads of the path, each with the number
+of launches its figure averages over: the matrix-pipe ceiling of the board (a loop of nothing
+but MFMAs, constant and random operands) and the consumer kernel on zero operands, the producer
+throttled to a link's rate, the chunked reduce, the GEMM+RS producer and the fused GEMM+RS step
+(producer, pushes gated by its flags, reduce), all-gather attention (resident and with the kv
+chunks arriving behind flags), all-to-all attention (causal; resident and gated), box copies,
+and CPU baselines of the same workloads on the host's cores.
 """
 
 from __future__ import annotations
@@ -27,11 +35,10 @@ import torch  # noqa: E402
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0      # MI355X dense bf16
 HBM_PEAK_GBPS = 8000.0
-# Bytes one launch of the 256x256 consumer kernel moves between L2 and the fabric: FETCH_SIZE and
-# WRITE_SIZE of two counter runs of `bench.py --resident-only`, scaled by the readings of the
-# library's copy kernel (profiles/bench_kernels_hbm_traffic.txt).  Counter runs
-# serialise kernels, so this cannot be sampled while the benchmark itself runs.
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 823.1e6
+# HBM bytes per launch of the kernels below come from hardware-counter runs, which serialise
+# kernels and therefore cannot be taken while the benchmark itself runs; the readings are kept
+# in this tracked file together with the commands that made them.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
 
 # AG+GEMM, the headline configuration
 M, K, N, WORLD, RANK = 8192, 8192, 3584, 8, 0
@@ -45,13 +52,39 @@ XCD_REMAP = False                    # consecutive tile ids on one XCD (see --xc
 LEAD_OPS = 3                         # ops of the side stream the consumer launch waits for: two chunks copied, the
                                      # first one's flag set (the second flag lands while the first tiles run)
 EIGHT_WAVES = False                  # 256-thread workgroups: one wavefront per SIMD, 128x128 of C each
+LEAD_COPY_BLOCKS = 0                 # see --lead-copy-blocks
+LEAD_ON_COMPUTE_STREAM = False       # see --lead-on-compute-stream
+LINK_CHUNK_US = 110                  # one 16.8 MB chunk over one xGMI link (~153 GB/s)
+
+SECTIONS = ("ag_gemm", "throttled", "mfma_ceiling", "reduce", "box_copies", "gemm_rs", "attn_ag", "attn_a2a", "cpu")
 
 
 def _events(n):
     return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
 
 
-def build_ag_gemm(device, copy_blocks=0, split_units=0, fuse_flags=False):
+def _timed(fn, launches, warmup, stream=None):
+    """Average milliseconds of `launches` calls of fn(i), timed as one batch between two events."""
+    stream = torch.cuda.current_stream() if stream is None else stream
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    begin, end = _events(2)
+    begin.record(stream)
+    for i in range(launches):
+        fn(i)
+    end.record(stream)
+    torch.cuda.synchronize()
+    return begin.elapsed_time(end) / launches
+
+
+def _table(rows, device):
+    return torch.tensor(rows, dtype=torch.int32, device=device)
+
+
+# ----------------------------------------------------------------------------------- AG+GEMM
+
+def build_ag_gemm(device, copy_blocks=0, split_units=0, fuse_flags=False, link_delay_us=0, lead_copy_blocks=0):
     from syncopate_amd.communication.code_gen import CommGenerator
     from syncopate_amd.communication.comm_runtime.communication_context import CommContext
     from syncopate_amd.communication.common_descriptors import build_all_gather_plan_1d_swizzle
@@ -77,38 +110,41 @@ def build_ag_gemm(device, copy_blocks=0, split_units=0, fuse_flags=False):
     a = (0.02 * torch.randn(M, K, device=device)).bfloat16()
     b = (0.02 * torch.randn(N, K, device=device)).bfloat16()
     # two flag sets: the reset of one iteration's flags happens behind the next one's copies
-    ctx = CommContext(RANK, info, device=device, copy_blocks=copy_blocks, flag_sets=2, fuse_flags=fuse_flags)
+    ctx = CommContext(RANK, info, device=device, copy_blocks=copy_blocks, flag_sets=2, fuse_flags=fuse_flags,
+                      link_delay_us=link_delay_us, lead_copy_blocks=lead_copy_blocks)
     rows = M // WORLD
     for r in range(WORLD):     # every rank's symmetric buffer holds its own shard
         ctx.comm_buffers["a"][r][r * rows:(r + 1) * rows].copy_(a[r * rows:(r + 1) * rows])
     dev_tables = dict(
-        cur_wave_sizes=torch.tensor(tables.block_shapes, dtype=torch.int32, device=device),
-        wave_offsets=torch.tensor(tables.block_offsets, dtype=torch.int32, device=device),
-        signal_offsets=torch.tensor(tables.signal_offsets, dtype=torch.int32, device=device),
+        cur_wave_sizes=_table(tables.block_shapes, device),
+        wave_offsets=_table(tables.block_offsets, device),
+        signal_offsets=_table(tables.signal_offsets, device),
         cum_tiles=tables.cum_tiles,
     )
     c = torch.empty(M, N, dtype=torch.bfloat16, device=device)
     return dict(a=a, b=b, c=c, ctx=ctx, tables=dev_tables, compile_ms=compile_ms)
 
 
-def run_ag_gemm(state, steps, warmup, resident_only=False, use_graph=True):
+def run_ag_gemm(state, steps, warmup, resident_only=False, use_graph=True, lead_ops=None):
     from syncopate_amd.computation._launch import check_status
     from syncopate_amd.computation.gemm import gemm
 
+    lead_ops = LEAD_OPS if lead_ops is None else lead_ops
     ctx, b, c, tables = state["ctx"], state["b"], state["c"], state["tables"]
     symm = ctx.comm_buffers["a"][RANK]
     stream = torch.cuda.current_stream()
 
-    def consumer(flag_words):
-        gemm(symm, b, c, WORLD, NUM_SMS, BM, BN, BK, GROUP_M, signal_ptr=flag_words, xcd_remap=XCD_REMAP,
+    def consumer(flag_words, a_operand=symm, b_operand=b):
+        gemm(a_operand, b_operand, c, WORLD, NUM_SMS, BM, BN, BK, GROUP_M, signal_ptr=flag_words, xcd_remap=XCD_REMAP,
              eight_waves=EIGHT_WAVES, **tables)
 
     def fused_step():
         cur = torch.cuda.current_stream()
         ctx.reset_signals()               # switches to the zeroed flag set
         ctx.start_after(cur)
-        ctx.execute(lead_ops=LEAD_OPS)
-        ctx.wait_lead(cur)                # the kernel starts behind the first two chunk copies (3x faster before it does)
+        ctx.execute(lead_ops=lead_ops, lead_on=cur if LEAD_ON_COMPUTE_STREAM else None)
+        if lead_ops:
+            ctx.wait_lead(cur)            # the kernel starts behind the first chunk copies (3x faster before it does)
         consumer(ctx.recv_signal_bufs[RANK])
         ctx.end_before(cur)
 
@@ -170,7 +206,7 @@ def run_ag_gemm(state, steps, warmup, resident_only=False, use_graph=True):
             for i in range(count):
                 ctx.reset_signals()
                 ctx.start_after(stream)
-                ctx.execute(lead_ops=lead)
+                ctx.execute(lead_ops=lead, lead_on=stream if (lead and LEAD_ON_COMPUTE_STREAM) else None)
                 if lead:
                     ctx.wait_lead(stream)
                 begin[i].record(stream)
@@ -179,27 +215,69 @@ def run_ag_gemm(state, steps, warmup, resident_only=False, use_graph=True):
                 ctx.end_before(stream)
             torch.cuda.synchronize()
             return sum(s.elapsed_time(e) for s, e in zip(begin, end)) / count
-        gated_kernel_ms = kernel_ms(steps, LEAD_OPS)
-        no_lead_kernel_ms = kernel_ms(min(steps, 20), 0) if LEAD_OPS else gated_kernel_ms
+        gated_kernel_ms = kernel_ms(steps, lead_ops)
+        no_lead_kernel_ms = kernel_ms(min(steps, 20), 0) if lead_ops else gated_kernel_ms
     check_status()
     ctx.check_status()
 
     # ---- same kernel, every chunk resident and every flag already set ----
     resident_flags = torch.ones_like(ctx.recv_signal_bufs[RANK])
-    for _ in range(warmup):
-        consumer(resident_flags)
-    torch.cuda.synchronize()
-    begin, end = _events(steps), _events(steps)
-    for i in range(steps):
-        begin[i].record(stream)
-        consumer(resident_flags)
-        end[i].record(stream)
-    torch.cuda.synchronize()
-    resident_kernel_ms = sum(s.elapsed_time(e) for s, e in zip(begin, end)) / steps
+
+    def resident_ms(a_operand=symm, b_operand=b):
+        for _ in range(warmup):
+            consumer(resident_flags, a_operand, b_operand)
+        torch.cuda.synchronize()
+        begin, end = _events(steps), _events(steps)
+        for i in range(steps):
+            begin[i].record(stream)
+            consumer(resident_flags, a_operand, b_operand)
+            end[i].record(stream)
+        torch.cuda.synchronize()
+        return sum(s.elapsed_time(e) for s, e in zip(begin, end)) / steps
+
+    resident_kernel_ms = resident_ms()
     check_status()
     if resident_only:
         wall_ms = gated_kernel_ms = no_lead_kernel_ms = resident_kernel_ms
+    state["resident_ms_fn"] = resident_ms
     return wall_ms, gated_kernel_ms, no_lead_kernel_ms, resident_kernel_ms
+
+
+def run_throttled(device, steps):
+    """The same fused step with the producer throttled to one link's rate: a delay in front of
+    every chunk copy brings a chunk to ~LINK_CHUNK_US, the time 16.8 MB take over one xGMI link.
+    Seven chunks in sequence then take longer than the GEMM: the step is bound by the producer,
+    and what the wave order buys is that only the last chunk's tiles are left when it lands."""
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.gemm import gemm
+
+    delay = LINK_CHUNK_US - 28          # a chunk copy beside the running GEMM takes ~28 us
+    state = build_ag_gemm(device, link_delay_us=delay)
+    ctx, b, c, tables = state["ctx"], state["b"], state["c"], state["tables"]
+    symm = ctx.comm_buffers["a"][RANK]
+    stream = torch.cuda.current_stream()
+
+    def step(i):
+        ctx.reset_signals()
+        ctx.start_after(stream)
+        ctx.execute()
+        gemm(symm, b, c, WORLD, NUM_SMS, BM, BN, BK, GROUP_M, signal_ptr=ctx.recv_signal_bufs[RANK],
+             xcd_remap=XCD_REMAP, eight_waves=EIGHT_WAVES, **tables)
+        ctx.end_before(stream)
+
+    ms = _timed(step, steps, 5, stream)
+    check_status()
+    ctx.check_status()
+    # the producer alone: the same op list with nothing to overlap
+    def comm_only(i):
+        ctx.reset_signals()
+        ctx.start_after(stream)
+        ctx.execute()
+        ctx.end_before(stream)
+    comm_ms = _timed(comm_only, steps, 3, stream)
+    del state
+    return {"launches": steps, "link_delay_us_per_chunk": delay, "ms_per_step": ms, "producer_alone_ms": comm_ms,
+            "exposed_compute_ms": ms - comm_ms}
 
 
 def traffic_calibration(device):
@@ -227,6 +305,37 @@ def check_ag_gemm(state):
     return err, gathered
 
 
+# ---------------------------------------------------------------------------- matrix-pipe ceiling
+
+def run_mfma_ceiling(device, state, launches=8):
+    """What the matrix pipes of this board sustain: a loop of nothing but the GEMM's MFMA on
+    register-resident operands, one workgroup of four wavefronts per compute unit, with constant
+    and with random operands (the board is power-limited: toggling operand bits cost clock);
+    and the consumer kernel itself, every chunk resident, on operands that are all zero."""
+    from syncopate_amd import _lib
+
+    lib = _lib.load()
+    sink = torch.empty(256 * 256, dtype=torch.float32, device=device)
+    stream = _lib.stream_handle(torch.cuda.current_stream())
+    iters = 2000
+    out = {"launches": launches, "mfma": "v_mfma_f32_32x32x16_bf16, 4x4 accumulators per wavefront, 64 per round",
+           "rounds_per_launch": iters}
+    for workgroups in (256, NUM_SMS):
+        for pattern, name in ((1, "constant"), (2, "random")):
+            def probe(i):
+                _lib.check("syn_probe_mfma_rate", lib.syn_probe_mfma_rate(sink.data_ptr(), workgroups, iters, pattern, stream))
+            ms = _timed(probe, launches, 3)
+            out[f"{name}_operands_{workgroups}_workgroups_tflops"] = workgroups * 4.0 * iters * 64 * 32768 / ms / 1e9
+    if state is not None and "resident_ms_fn" in state:
+        zeros_a, zeros_b = torch.zeros_like(state["a"]), torch.zeros_like(state["b"])
+        ms = state["resident_ms_fn"](zeros_a, zeros_b)
+        out["consumer_kernel_zero_operands_tflops"] = 2.0 * M * N * K / ms / 1e9
+        out["consumer_kernel_zero_operands_ms"] = ms
+    return out
+
+
+# --------------------------------------------------------------------------------------- reduce
+
 def run_reduce(device, steps, warmup):
     """GEMM+RS chunked reduce of the headline GEMM+RS configuration: 8 x (1024, 8192) bf16 -> (1024, 8192).
     Launches rotate over three sets of operands (3 x 151 MB, more than the 256 MB of memory-side
@@ -238,17 +347,7 @@ def run_reduce(device, steps, warmup):
     recv = [torch.randn(world, rows, n, device=device).bfloat16() for _ in range(sets)]
     local = [torch.randn(world * rows, n, device=device).bfloat16() for _ in range(sets)]
     out = [torch.empty(rows, n, dtype=torch.bfloat16, device=device) for _ in range(sets)]
-    stream = torch.cuda.current_stream()
-    for i in range(max(warmup, sets)):
-        ring_reduce(recv[i % sets], out[i % sets], local[i % sets], RANK)
-    torch.cuda.synchronize()
-    begin, end = _events(1)[0], _events(1)[0]
-    begin.record(stream)
-    for i in range(steps):
-        ring_reduce(recv[i % sets], out[i % sets], local[i % sets], RANK)
-    end.record(stream)
-    torch.cuda.synchronize()
-    ms = begin.elapsed_time(end) / steps
+    ms = _timed(lambda i: ring_reduce(recv[i % sets], out[i % sets], local[i % sets], RANK), steps, max(warmup, sets))
     nbytes = (world + 1) * rows * n * 2          # 8 reads + 1 write of a (1024, 8192) bf16 block
     return ms, nbytes
 
@@ -265,97 +364,270 @@ def run_box_copies(device, steps, warmup):
     torch.manual_seed(3)
     src = [torch.randn(rows, n, device=device).bfloat16() for _ in range(sets)]
     dst = [torch.zeros(rows, n, dtype=torch.bfloat16, device=device) for _ in range(sets)]
-    stream = torch.cuda.current_stream()
     nbytes = rows * n * 2
     forms = {"copy": (None, False, 2 * nbytes), "add_exclusive": (ReduceOp.SUM, True, 3 * nbytes),
              "add_atomic": (ReduceOp.SUM, False, 3 * nbytes)}
     result = {}
     for name, (op, exclusive, traffic) in forms.items():
-        for i in range(max(warmup, sets)):
-            persistent_copy_last_contig(src[i % sets], dst[i % sets], num_sms=blocks, reduce_op=op, exclusive=exclusive)
-        torch.cuda.synchronize()
-        begin, end = _events(1)[0], _events(1)[0]
-        begin.record(stream)
-        for i in range(steps):
-            persistent_copy_last_contig(src[i % sets], dst[i % sets], num_sms=blocks, reduce_op=op, exclusive=exclusive)
-        end.record(stream)
-        torch.cuda.synchronize()
-        result[name] = (begin.elapsed_time(end) / steps, traffic)
+        ms = _timed(lambda i: persistent_copy_last_contig(src[i % sets], dst[i % sets], num_sms=blocks, reduce_op=op,
+                                                          exclusive=exclusive), steps, max(warmup, sets))
+        result[name] = (ms, traffic)
     return result
 
 
-def run_attention(device, steps, warmup):
-    """All-gather attention at the headline ring / all-gather configuration: 4096 local q rows, 32 heads, against 32768
-    kv rows as 8 chunks of 4096 in double-ring arrival order (every chunk resident), head dim 128; two q
-    blocks per workgroup in opposite phases (pair_q_blocks)."""
+# -------------------------------------------------------------------------------------- GEMM+RS
+
+def run_gemm_rs(device, steps, warmup, gated=True):
+    """GEMM+RS of rank 0 of 8: partial C (8192, 8192) = A (8192, 3584) B^T in wave order 1..7, 0 with
+    per-wave counters and flags.  Timed twice: the producer kernel alone, and the fused step the
+    reference times (tests/test_gemm_rs.py:196-244) - producer on the compute stream, the pushes
+    of the finished chunks to their owners on a side stream, each behind its wave's COMPUTE_DONE
+    flag, then the chunked reduce of the 7 received partials and the rank's own block."""
+    from syncopate_amd.communication.code_gen import CommGenerator
+    from syncopate_amd.communication.comm_runtime.communication_context import CommContext
+    from syncopate_amd.communication.common_descriptors import build_all_to_all_plan
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.gemm import gemm_producer
+    from syncopate_amd.computation.reduce import ring_reduce
+    from syncopate_amd.interface import lower_comm_plan_to_raw_schedules
+    from syncopate_amd.interface.wave_tables import gemm_producer_tables
+
+    m, k, n, world = 8192, 3584, 8192, 8
+    rows = m // world
+    plans = {r: build_all_to_all_plan(shape=(m, n), dtype=torch.bfloat16, mesh_size=world, rank=r, src_buffer="src",
+                                      dst_buffer="dst", transfer_kind="push", compute_producer=True)
+             for r in range(world)}
+    gen = CommGenerator(plans)
+    gen.plan_signals()
+    tables = gemm_producer_tables(lower_comm_plan_to_raw_schedules(gen)[RANK]["src"])
+    info = gen.generate_code_for_plan()
+    info.local_world_size = info.world_size
+    ctx = CommContext(RANK, info, device=device)
+    torch.manual_seed(3)
+    a = (0.02 * torch.randn(m, k, device=device)).bfloat16()
+    b = (0.02 * torch.randn(n, k, device=device)).bfloat16()
+    src, dst = ctx.comm_buffers["src"][RANK], ctx.comm_buffers["dst"][RANK]
+    dst.copy_(torch.randn(world, rows, n, device=device).bfloat16())       # what the peers pushed
+    out = torch.empty(rows, n, dtype=torch.bfloat16, device=device)
+    sizes, offsets = _table(tables.block_shapes, device), _table(tables.block_offsets, device)
+    signals = _table(tables.signal_offsets, device)
+    counters = torch.zeros(world, dtype=torch.int32, device=device)
+    main = torch.cuda.current_stream()
+
+    def producer(flags, programs=256):
+        counters.zero_()
+        # 1024 tiles of 256 x 256: four full rounds of 256 programs
+        gemm_producer(a, b, src, flags, sizes, offsets, signals, programs, 256, 256, BK, GROUP_M,
+                      cum_tiles=tables.cum_tiles, counter_buffer=counters, xcd_remap=False, eight_waves=EIGHT_WAVES)
+
+    alone_flags = torch.zeros(world, dtype=torch.int64, device=device)
+    producer_ms = _timed(lambda i: producer(alone_flags), steps, warmup)
+    assert alone_flags.tolist() == [1] * world
+
+    if not gated:
+        return {"launches": steps, "producer_ms": producer_ms, "flop": 2.0 * m * n * k}
+
+    def fused(programs):
+        ctx.reset_signals()
+        ctx.start_after(main)
+        producer(ctx.compute_signal_bufs[RANK], programs)
+        ctx.execute(neglect_local=True)
+        ctx.end_before(main)
+        ring_reduce(dst, out, src, RANK)
+
+    # On one GPU the pushes are copy kernels that need compute units: beside 256 persistent programs
+    # they only run once the producer has finished; 224 programs leave them 32 units but cost the
+    # GEMM a fifth round of tiles.  Both are timed; a node's copy engines need neither.
+    fused_by_programs = {programs: _timed(lambda i: fused(programs), steps, max(3, warmup // 4)) for programs in (224, 256)}
+    fused_ms = min(fused_by_programs.values())
+    check_status()
+    ctx.check_status()
+    sample = torch.arange(7, rows, 97, device=device)
+    acc = src[RANK * rows:(RANK + 1) * rows][sample].clone()
+    for i in range(1, world):
+        acc = acc + dst[(RANK + i) % world][sample]
+    reduce_matches = torch.equal(out[sample], acc)
+    pushed = all(torch.equal(ctx.comm_buffers["dst"][p][RANK], src[p * rows:(p + 1) * rows]) for p in (1, 4, 7))
+    return {"launches": steps, "producer_ms": producer_ms, "flop": 2.0 * m * n * k, "fused_step_ms": fused_ms,
+            "fused_step_ms_by_programs": {str(k_): v for k_, v in fused_by_programs.items()},
+            "reduce_matches": bool(reduce_matches), "pushed_chunks_match": bool(pushed)}
+
+
+# ------------------------------------------------------------------------------------ attention
+
+def _gated_attention(q, staged_kv, buf, arrival, chunk, tables, launches, device, causal=False, pair=False,
+                     programs=0, copy_units=32):
+    """Attention over `buf` (stacked K, V of shape [2, B, H, S, D]) while the kv chunks arrive:
+    chunk arrival[0] is resident, the others are copied from `staged_kv` by a side-stream
+    producer in arrival order - a box copy on `copy_units` compute units, then the chunk's flag.
+    The kernel runs `programs` persistent workgroups so that the copies find compute units."""
+    from syncopate_amd import _lib
+    from syncopate_amd.communication.comm_runtime.persistent_copy import persistent_copy_last_contig
+    from syncopate_amd.communication.comm_runtime.streams import pick_side_streams
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.attn import attention_forward
+
+    lib = _lib.load()
+    D = q.shape[-1]
+    main = torch.cuda.current_stream()
+    side = pick_side_streams(1, main, device)[0]
+    flags = torch.zeros(len(arrival), dtype=torch.int64, device=device)
+    out = torch.empty_like(q)
+    signals = tables["signal_offsets"].tolist()
+    own = arrival[0]
+    buf.zero_()
+    buf[:, :, :, own * chunk:(own + 1) * chunk].copy_(staged_kv[:, :, :, own * chunk:(own + 1) * chunk])
+
+    def step(i):
+        flags.zero_()
+        side.wait_stream(main)
+        with torch.cuda.stream(side):
+            for wave in range(1, len(arrival)):
+                c = arrival[wave]
+                persistent_copy_last_contig(staged_kv[:, :, :, c * chunk:(c + 1) * chunk],
+                                            buf[:, :, :, c * chunk:(c + 1) * chunk], num_sms=copy_units)
+                _lib.check("syn_flag_set", lib.syn_flag_set(flags.data_ptr() + 8 * signals[wave], 1,
+                                                            _lib.stream_handle(side)))
+        attention_forward(q, buf[0], buf[1], D ** -0.5, out=out, signal_ptr=flags, causal=causal, pair_q_blocks=pair,
+                          num_programs=programs, **tables)
+        main.wait_stream(side)
+
+    ms = _timed(step, launches, 2)
+    check_status()
+    return ms, out
+
+
+def run_attention_ag(device, launches=5, gated=True):
+    """All-gather attention at the headline ring / all-gather configuration: 4096 local q rows, 32 heads,
+    against 32768 kv rows as 8 chunks of 4096 in double-ring arrival order, head dim 128; two q
+    blocks per workgroup in opposite phases (pair_q_blocks).  Resident (every flag set), and gated."""
     from syncopate_amd.computation._launch import check_status
     from syncopate_amd.computation.attn import attention_forward
 
     B, H, Sq, Skv, D, chunks = 1, 32, 4096, 32768, 128, 8
     torch.manual_seed(2)
     q = torch.randn(B, H, Sq, D, device=device).bfloat16()
-    k = torch.randn(B, H, Skv, D, device=device).bfloat16()
-    v = torch.randn(B, H, Skv, D, device=device).bfloat16()
+    kv = torch.randn(2, B, H, Skv, D, device=device).bfloat16()
     chunk = Skv // chunks
-    as_table = lambda rows: torch.tensor(rows, dtype=torch.int32, device=device)
+    arrival = [0, 1, 7, 6, 4, 5, 3, 2]
     cums = [(i + 1) * B * H * Sq for i in range(chunks)]
-    tables = dict(wave_offsets=as_table([[0, 0, 0, o * chunk] for o in (0, 1, 7, 6, 4, 5, 3, 2)]),
-                  wave_sizes=as_table([[B, H, Sq, chunk]] * chunks), cum_wave_sizes=as_table(cums),
-                  signal_offsets=as_table([-1, 0, 4, 1, 5, 2, 6, 3]), cum_tiles=cums[-1],
-                  signal_ptr=torch.ones(chunks, dtype=torch.int64, device=device))
+    tables = dict(wave_offsets=_table([[0, 0, 0, o * chunk] for o in arrival], device),
+                  wave_sizes=_table([[B, H, Sq, chunk]] * chunks, device), cum_wave_sizes=_table(cums, device),
+                  signal_offsets=_table([-1, 0, 4, 1, 5, 2, 6, 3], device), cum_tiles=cums[-1])
+    ones = torch.ones(chunks, dtype=torch.int64, device=device)
     out = torch.empty_like(q)
-    for _ in range(warmup):
-        attention_forward(q, k, v, D ** -0.5, out=out, pair_q_blocks=True, **tables)
-    torch.cuda.synchronize()
-    begin, end = _events(1)[0], _events(1)[0]
-    begin.record()
-    for _ in range(steps):
-        attention_forward(q, k, v, D ** -0.5, out=out, pair_q_blocks=True, **tables)
-    end.record()
-    torch.cuda.synchronize()
+    ms = _timed(lambda i: attention_forward(q, kv[0], kv[1], D ** -0.5, out=out, pair_q_blocks=True, signal_ptr=ones,
+                                            **tables), launches, 2)
     check_status()
-    s = (q[0, 7].float() @ k[0, 7].float().t()) * D ** -0.5
-    ref = torch.softmax(s, dim=-1) @ v[0, 7].float()
+    persistent_ms = _timed(lambda i: attention_forward(q, kv[0], kv[1], D ** -0.5, out=out, pair_q_blocks=True,
+                                                       signal_ptr=ones, num_programs=224, **tables), launches, 2)
+    s = (q[0, 7].float() @ kv[0, 0, 7].float().t()) * D ** -0.5
+    ref = torch.softmax(s, dim=-1) @ kv[1, 0, 7].float()
     err = ((out[0, 7].float() - ref).abs().max() / ref.abs().max()).item()
-    return begin.elapsed_time(end) / steps, 4.0 * B * H * Sq * Skv * D, err
+    result = {"launches": launches, "ms": ms, "flop": 4.0 * B * H * Sq * Skv * D, "max_rel_err_vs_fp32": err,
+              "ms_224_programs_resident": persistent_ms}
+    if not gated:
+        return result
+    buf = torch.empty_like(kv)
+    gated_ms, gated_out = _gated_attention(q, kv, buf, arrival, chunk, tables, launches, device, pair=True, programs=224)
+    gated_err = ((gated_out[0, 7].float() - ref).abs().max() / ref.abs().max()).item()
+    result.update({"ms_gated": gated_ms, "gated_max_rel_err_vs_fp32": gated_err,
+                   "gathered_kv_matches": bool(torch.equal(buf, kv)),
+                   "flag_wait_overhead_pct": 100.0 * (gated_ms - persistent_ms) / persistent_ms,
+                   "gated_tflops": result["flop"] / (gated_ms * 1e-3) / 1e12})
+    return result
 
 
-def run_producer(device, steps, warmup):
-    """GEMM+RS producer of the headline GEMM+RS configuration: partial C (8192, 8192) = A (8192, 3584) B^T in
-    wave order 1..7, 0 with per-wave counters and flags."""
-    from syncopate_amd.computation.gemm import gemm_producer
+def run_attention_a2a(device, launches=5, gated=True):
+    """All-to-all (Ulysses) attention of rank 0 of 8: the whole sequence of 16384, 4 local heads, head
+    dim 128, causal; Q, K and V arrive as 8 sequence chunks of 2048 (the rank's own first), and
+    arrival w unlocks (Q_w x KV_w), (Q_p x KV_w) and (Q_w x KV_p) for every earlier p: 64 waves.
+    Resident, and with the chunks copied in behind flags.  flop counts the causal half."""
+    from syncopate_amd.communication.code_gen import CommGenerator
+    from syncopate_amd.communication.common_descriptors import build_all_to_all_plan_dim
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.attn import attention_forward
+    from syncopate_amd.interface import lower_comm_plan_to_raw_schedules
+    from syncopate_amd.interface.wave_tables import all2all_attn_tables
 
-    m, k, n, world = 8192, 3584, 8192, 8
-    torch.manual_seed(3)
-    a = (0.02 * torch.randn(m, k, device=device)).bfloat16()
-    b = (0.02 * torch.randn(n, k, device=device)).bfloat16()
-    c = torch.empty(m, n, dtype=torch.bfloat16, device=device)
-    rows = m // world
-    as_table = lambda rows_: torch.tensor(rows_, dtype=torch.int32, device=device)
-    sizes = as_table([[rows, n]] * world)
-    offsets = as_table([[((RANK + i + 1) % world) * rows, 0] for i in range(world)])
-    signals = as_table(list(range(world)))
-    flags = torch.zeros(world, dtype=torch.int64, device=device)
-    counters = torch.zeros(world, dtype=torch.int32, device=device)
+    world, B, H, S_local, D = 8, 1, 32, 2048, 128
+    H_local, S = H // world, world * S_local
+    plans = {r: build_all_to_all_plan_dim(shape=(3, B, H, S_local, D), dtype=torch.bfloat16, mesh_size=world, rank=r,
+                                          src_buffer="src", dst_buffer="dst", src_split_axis=3, dst_split_axis=2,
+                                          transfer_kind="pull", compute_producer=False) for r in range(world)}
+    gen = CommGenerator(plans)
+    gen.plan_signals()
+    host = all2all_attn_tables(lower_comm_plan_to_raw_schedules(gen)[RANK]["dst"], {"batch": 1, "head": 2, "seq": 3})
+    tables = dict(wave_offsets=_table(host.wave_offsets, device), wave_sizes=_table(host.wave_sizes, device),
+                  cum_wave_sizes=_table(host.cum_wave_sizes, device), signal_offsets=_table(host.signal_offsets, device),
+                  cum_tiles=host.cum_tiles)
+    num_flags = max(host.signal_offsets) + 1
+    torch.manual_seed(4)
+    qkv = torch.randn(3, B, H_local, S, D, device=device).bfloat16()
+    scale = D ** -0.5
+    ones = torch.ones(num_flags, dtype=torch.int64, device=device)
+    out = torch.empty_like(qkv[0])
+    ms = _timed(lambda i: attention_forward(qkv[0], qkv[1], qkv[2], scale, out=out, signal_ptr=ones, causal=True,
+                                            **tables), launches, 2)
+    check_status()
+    noncausal_ms = _timed(lambda i: attention_forward(qkv[0], qkv[1], qkv[2], scale, out=out, signal_ptr=ones,
+                                                      **tables), launches, 2)
+    attention_forward(qkv[0], qkv[1], qkv[2], scale, out=out, signal_ptr=ones, causal=True, **tables)
+    rows = torch.arange(3, S, 61, device=device)
+    s = (qkv[0, 0, 1][rows].float() @ qkv[1, 0, 1].float().t()) * scale
+    s = s.masked_fill(torch.arange(S, device=device)[None, :] > rows[:, None], float("-inf"))
+    ref = torch.softmax(s, dim=-1) @ qkv[2, 0, 1].float()
+    err = ((out[0, 1][rows].float() - ref).abs().max() / ref.abs().max()).item()
 
-    def launch():
-        counters.zero_()
-        # 1024 tiles of 256 x 256: four full rounds of 256 programs
-        gemm_producer(a, b, c, flags, sizes, offsets, signals, 256, 256, 256, BK, GROUP_M, cum_tiles=m * n,
-                      counter_buffer=counters, xcd_remap=False, eight_waves=EIGHT_WAVES)
+    result = {"launches": launches, "waves": len(host.signal_offsets), "ms_causal": ms, "ms_non_causal": noncausal_ms,
+              "flop_causal": 2.0 * B * H_local * S * S * D, "flop_non_causal": 4.0 * B * H_local * S * S * D,
+              "max_rel_err_vs_fp32": err}
+    result["causal_tflops"] = result["flop_causal"] / (ms * 1e-3) / 1e12
+    result["non_causal_tflops"] = result["flop_non_causal"] / (noncausal_ms * 1e-3) / 1e12
+    if not gated:
+        return result
 
-    for _ in range(warmup):
-        launch()
-    torch.cuda.synchronize()
-    begin, end = _events(1)[0], _events(1)[0]
-    begin.record()
-    for _ in range(steps):
-        launch()
-    end.record()
-    torch.cuda.synchronize()
-    assert flags.tolist() == [1] * world
-    return begin.elapsed_time(end) / steps, 2.0 * m * n * k
+    # gated: Q, K and V of sequence chunk w land together (one box copy of the stacked buffer, then flag w)
+    from syncopate_amd import _lib
+    from syncopate_amd.communication.comm_runtime.persistent_copy import persistent_copy_last_contig
+    from syncopate_amd.communication.comm_runtime.streams import pick_side_streams
 
+    lib = _lib.load()
+    main = torch.cuda.current_stream()
+    side = pick_side_streams(1, main, device)[0]
+    flags = torch.zeros(num_flags, dtype=torch.int64, device=device)
+    buf = torch.zeros_like(qkv)
+    # arrival order of the sequence chunks and each arrival's flag: the (Q_w x KV_w) waves of the table
+    diag = [i for i in range(len(host.signal_offsets))
+            if host.wave_offsets[i][2] == host.wave_offsets[i][3] and host.wave_sizes[i][2] == host.wave_sizes[i][3]]
+    arrivals = [(host.wave_offsets[i][2] // S_local, host.signal_offsets[i]) for i in diag]
+    persistent_ms = _timed(lambda i: attention_forward(qkv[0], qkv[1], qkv[2], scale, out=out, signal_ptr=ones, causal=True,
+                                                       num_programs=448, **tables), launches, 2)
+
+    def step(i):
+        flags.zero_()
+        side.wait_stream(main)
+        with torch.cuda.stream(side):
+            for c, sig in arrivals:
+                persistent_copy_last_contig(qkv[:, :, :, c * S_local:(c + 1) * S_local],
+                                            buf[:, :, :, c * S_local:(c + 1) * S_local], num_sms=32)
+                if sig >= 0:
+                    _lib.check("syn_flag_set", lib.syn_flag_set(flags.data_ptr() + 8 * sig, 1, _lib.stream_handle(side)))
+        attention_forward(buf[0], buf[1], buf[2], scale, out=out, signal_ptr=flags, causal=True, num_programs=448,
+                          **tables)
+        main.wait_stream(side)
+
+    gated_ms = _timed(step, launches, 2)
+    check_status()
+    gated_err = ((out[0, 1][rows].float() - ref).abs().max() / ref.abs().max()).item()
+    result.update({"ms_causal_448_programs_resident": persistent_ms, "ms_causal_gated": gated_ms,
+                   "gated_max_rel_err_vs_fp32": gated_err, "gathered_qkv_matches": bool(torch.equal(buf, qkv)),
+                   "flag_wait_overhead_pct": 100.0 * (gated_ms - persistent_ms) / persistent_ms,
+                   "gated_causal_tflops": result["flop_causal"] / (gated_ms * 1e-3) / 1e12})
+    return result
+
+
+# -------------------------------------------------------------------------------- CPU baselines
 
 def cpu_baseline(state):
     """torch CPU matmul over the gathered operands (fp32 values of the same bf16 inputs):
@@ -369,7 +641,7 @@ def cpu_baseline(state):
     b = state["b"].cpu()
     numerics.gemm_fp32(a[:128], b)          # warm-up
     reps, spent = 0, 0.0
-    while spent < 10.0 and reps < 40:
+    while spent < 8.0 and reps < 40:
         t0 = time.perf_counter()
         numerics.gemm_fp32(a, b)
         spent += time.perf_counter() - t0
@@ -385,18 +657,94 @@ def cpu_baseline(state):
     }
 
 
+def cpu_baselines_other():
+    """The other workloads on the host's cores, bounded samples, one to three repetitions each:
+    the reference's CPU case (mesh 4: plan -> signals -> lowered schedules -> op lists, then the
+    fp16 matmul of the gathered A), the chunked reduce, and both attention shapes through
+    torch's CPU attention over the gathered operands."""
+    import numpy as np
+
+    from oracle import numerics
+    from syncopate_amd.communication.code_gen import CommGenerator
+    from syncopate_amd.communication.common_descriptors import build_all_gather_plan_1d_swizzle
+    from syncopate_amd.interface import lower_comm_plan_to_raw_schedules
+
+    threads = min(16, os.cpu_count() or 1)
+    torch.set_num_threads(threads)
+    result = {"cores": threads}
+
+    def compile_c1():
+        plans = {r: build_all_gather_plan_1d_swizzle((4096, 512), torch.float16, 0, 4, r, "a", "pull") for r in range(4)}
+        gen = CommGenerator(plans)
+        gen.plan_signals()
+        schedules = lower_comm_plan_to_raw_schedules(gen)
+        gen.generate_code_for_plan()
+        return [schedules[r]["a"].gen_block_offset_lists() for r in range(4)]
+    compile_c1()
+    t0 = time.perf_counter()
+    for _ in range(5):
+        compile_c1()
+    result["c1_compile_us"] = (time.perf_counter() - t0) / 5 * 1e6
+    torch.manual_seed(0)
+    a = torch.cat([torch.randn(1024, 512).half() for _ in range(4)])
+    b = torch.randn(512, 1024).half()
+    a @ b
+    t0 = time.perf_counter()
+    for _ in range(3):
+        a @ b
+    result["c1_fp16_matmul_ms"] = (time.perf_counter() - t0) / 3 * 1e3
+    t0 = time.perf_counter()
+    a.float() @ b.float()
+    result["c1_fp32_matmul_ms"] = (time.perf_counter() - t0) * 1e3
+
+    rng = np.random.default_rng(1)
+    recv = rng.standard_normal((8, 1024, 8192), dtype=np.float32)
+    local = rng.standard_normal((8192, 8192), dtype=np.float32)
+    t0 = time.perf_counter()
+    numerics.ring_reduce(recv, local, 0, dtype="bf16")
+    spent = time.perf_counter() - t0
+    result["c3_reduce_ms"] = spent * 1e3
+    result["c3_reduce_GBps"] = 9 * 1024 * 8192 * 2 / spent / 1e9
+    result["c3_reduce_sample"] = "1 x numpy ring reduce of 8 x (1024, 8192), one bf16 rounding per add"
+
+    torch.manual_seed(2)
+    for name, (H, Sq, Skv, causal, heads) in {"c5_attention": (32, 4096, 32768, False, 8),
+                                              "c4_attention_causal": (4, 16384, 16384, True, 2)}.items():
+        q = torch.randn(1, heads, Sq, 128)
+        k = torch.randn(1, heads, Skv, 128)
+        v = torch.randn(1, heads, Skv, 128)
+        t0 = time.perf_counter()
+        numerics.sdpa_fp32(q, k, v, 128 ** -0.5, causal=causal)
+        spent = time.perf_counter() - t0
+        flop = 4.0 * heads * Sq * Skv * 128 * (0.5 if causal else 1.0)
+        result[name + "_tflops"] = flop / spent / 1e12
+        result[name + "_sample"] = (f"1 x torch CPU fp32 attention of {heads} of the {H} heads "
+                                    f"({Sq} q rows x {Skv} kv rows), {spent:.1f} s")
+    return result
+
+
+def _traffic():
+    try:
+        with open(TRAFFIC_FILE) as f:
+            return json.load(f)
+    except (OSError, ValueError):
+        return {}
+
+
 def main():
-    global BM, BN, NUM_SMS, LEAD_OPS, XCD_REMAP
+    global BM, BN, NUM_SMS, LEAD_OPS, XCD_REMAP, LEAD_ON_COMPUTE_STREAM
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     # a step is ~0.45 ms: the defaults time a few hundred of them (the whole run still takes well under a minute)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only", default="", help="comma-separated subset of: " + ", ".join(SECTIONS) +
+                    " (ag_gemm always runs; for profiler runs that want one kernel)")
     ap.add_argument("--no-graph", action="store_true", help="launch every step's operations from the host "
                     "instead of replaying them as one HIP graph")
     ap.add_argument("--resident-only", action="store_true",
-                    help="skip the flag-gated steps (for hardware-counter runs, which serialise kernels: "
+                    help="skip every flag-gated run (for hardware-counter runs, which serialise kernels: "
                          "a gated consumer would wait for copies that can only start after it)")
     ap.add_argument("--copy-blocks", type=int, default=0,
                     help="0: the producer's chunk copies are hipMemcpyAsync (default); N > 0: the library's "
@@ -410,6 +758,10 @@ def main():
     ap.add_argument("--split-device", type=int, default=0, metavar="N",
                     help="give N compute units (a multiple of 8) to the producer's stream and the rest to the "
                          "consumer's, by compute-unit masks")
+    ap.add_argument("--lead-copy-blocks", type=int, default=LEAD_COPY_BLOCKS,
+                    help="N > 0: a leading chunk copy and its flag write are one kernel of N workgroups")
+    ap.add_argument("--lead-on-compute-stream", action="store_true",
+                    help="the leading ops run on the compute stream itself, in front of the kernel")
     ap.add_argument("--lead-ops", type=int, default=LEAD_OPS,
                     help="the consumer launch waits for this many leading ops of the side stream (0: none)")
     args = ap.parse_args()
@@ -425,27 +777,37 @@ def main():
     NUM_SMS = args.programs
     LEAD_OPS = args.lead_ops
     XCD_REMAP = args.xcd_remap
+    LEAD_ON_COMPUTE_STREAM = args.lead_on_compute_stream
+    only = set(x for x in args.only.split(",") if x) or set(SECTIONS)
+    unknown = only - set(SECTIONS)
+    if unknown:
+        sys.exit(f"--only: unknown section(s) {sorted(unknown)}")
+    if args.no_cpu_baseline:
+        only.discard("cpu")
+    gated = not args.resident_only
     device = torch.device("cuda", 0)
     torch.cuda.set_device(device)
 
     if args.split_device and (args.copy_blocks == 0 or not args.no_graph):
         sys.exit("--split-device splits the compute units between two streams: it needs the copy kernel "
                  "(--copy-blocks N) and launches from the host (--no-graph; a graph's kernel nodes carry no mask)")
-    state = build_ag_gemm(device, args.copy_blocks, args.split_device, args.fuse_flags)
+    state = build_ag_gemm(device, args.copy_blocks, args.split_device, args.fuse_flags,
+                          lead_copy_blocks=args.lead_copy_blocks)
     with torch.cuda.stream(state["ctx"].compute_stream):
         wall_ms, gated_ms, no_lead_ms, resident_ms = run_ag_gemm(state, args.steps, args.warmup, args.resident_only,
-                                                     not args.no_graph)
+                                                                 not args.no_graph)
+        torch.cuda.synchronize()
+        traffic_calibration(device)
+        err, gathered = check_ag_gemm(state)
+        ceiling = run_mfma_ceiling(device, state) if "mfma_ceiling" in only else None
     torch.cuda.synchronize()
-    traffic_calibration(device)
-    err, gathered = check_ag_gemm(state)
-    reduce_ms, reduce_bytes = run_reduce(device, max(args.steps, 30), args.warmup)
-    boxes = run_box_copies(device, max(args.steps, 20), args.warmup)
-    attn_ms, attn_flop, attn_err = run_attention(device, 5, 2)
-    prod_ms, prod_flop = run_producer(device, args.steps, args.warmup)
 
     flop = 2.0 * M * N * K
     value = flop / (wall_ms * 1e-3) / 1e12
     kernel_tflops = flop / (gated_ms * 1e-3) / 1e12
+    kernel_name = (f"gemm_wave_kernel<bf16, {'EarlyPipe' if (BM, BN) in ((256, 256), (256, 224)) else 'SlabPipe<3 stages>'}, "
+                   f"{BM}x{BN}, {8 if EIGHT_WAVES else 4} wavefronts, consumer>")
+    traffic = _traffic().get("gemm_consumer_256x256_224_programs", {}) if (BM, BN, NUM_SMS) == (256, 256, 224) else {}
     line = {
         "metric": "AG-GEMM TFLOP/s",
         "value": value,
@@ -468,6 +830,7 @@ def main():
             "tile": [BM, BN, BK],
             "programs": NUM_SMS,
             "lead_ops": LEAD_OPS,
+            "lead_copy_blocks": args.lead_copy_blocks,
             "producer": "side stream: " + (
                 f"one kernel of {args.copy_blocks} workgroups per chunk that copies, then sets the flag"
                 if args.fuse_flags else
@@ -477,39 +840,77 @@ def main():
             "split_device": state["ctx"].cu_split,
         },
         "pct_bf16_mfma_peak": 100.0 * value / MFMA_BF16_PEAK_TFLOPS,
-        "flag_wait_overhead_pct": 100.0 * (gated_ms - resident_ms) / resident_ms,
-        "step_over_resident_kernel_pct": 100.0 * (wall_ms - resident_ms) / resident_ms,
+        # gated step against the same kernel with every chunk resident: the whole iteration, lead-in copies,
+        # flag reset and stream joins included
+        "flag_wait_overhead_pct": 100.0 * (wall_ms - resident_ms) / resident_ms,
+        # the kernel alone, in the launch shape of the timed steps (behind the leading chunks)
+        "kernel_only_gated_over_resident_pct": 100.0 * (gated_ms - resident_ms) / resident_ms,
+        "kernel_launches_timed": args.steps,
         "kernel_ms_gated": gated_ms,
         "kernel_ms_gated_launched_with_first_copy": no_lead_ms,
         "kernel_ms_resident": resident_ms,
         "resident_tflops": flop / (resident_ms * 1e-3) / 1e12,
-        "rs_reduce_GBps": reduce_bytes / (reduce_ms * 1e-3) / 1e9,
-        "rs_reduce_us": reduce_ms * 1e3,
-        "rs_reduce_pct_hbm_peak": 100.0 * reduce_bytes / (reduce_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-        "box_copy_GBps": {name: traffic / (ms * 1e-3) / 1e9 for name, (ms, traffic) in boxes.items()},
-        "box_copy_us": {name: ms * 1e3 for name, (ms, _) in boxes.items()},
-        "rs_producer_tflops": prod_flop / (prod_ms * 1e-3) / 1e12,
-        "rs_producer_pct_bf16_mfma_peak": 100.0 * prod_flop / (prod_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
-        "attn_tflops": attn_flop / (attn_ms * 1e-3) / 1e12,
-        "attn_pct_bf16_mfma_peak": 100.0 * attn_flop / (attn_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
-        "attn_ms": attn_ms,
-        "attn_max_rel_err_vs_fp32": attn_err,
         "host_compile_ms": state["compile_ms"],
         "max_rel_err_vs_fp32": err,
         "gathered_a_matches": gathered,
         "roofline": {
-            "kernel": f"gemm_wave_kernel<bf16, {'EarlyPipe' if (BM, BN) in ((256, 256), (256, 224)) else 'SlabPipe<3 stages>'}, "
-                      f"{BM}x{BN}, {8 if EIGHT_WAVES else 4} wavefronts, consumer>",
+            "kernel": kernel_name,
             "bound": "mfma",
             "achieved": kernel_tflops,
             "peak": MFMA_BF16_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": kernel_tflops / MFMA_BF16_PEAK_TFLOPS,
-            "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH,
+            "traffic": traffic.get("bytes_per_launch"),
+            "traffic_source": traffic.get("source"),
         },
     }
-    if not args.no_cpu_baseline:
+    if ceiling is not None:
+        line["mfma_ceiling"] = ceiling
+        random_ceiling = ceiling.get("random_operands_256_workgroups_tflops")
+        if random_ceiling:
+            line["roofline"]["frac_of_random_operand_mfma_ceiling"] = kernel_tflops / random_ceiling
+    steps_small = max(20, min(args.steps, 60))
+    if "throttled" in only and gated:
+        line["throttled_producer"] = run_throttled(device, 20)
+    if "reduce" in only:
+        reduce_ms, reduce_bytes = run_reduce(device, max(args.steps, 30), args.warmup)
+        line.update({
+            "rs_reduce_launches": max(args.steps, 30),
+            "rs_reduce_GBps": reduce_bytes / (reduce_ms * 1e-3) / 1e9,
+            "rs_reduce_us": reduce_ms * 1e3,
+            "rs_reduce_pct_hbm_peak": 100.0 * reduce_bytes / (reduce_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+        })
+    if "box_copies" in only:
+        boxes = run_box_copies(device, steps_small, args.warmup)
+        line["box_copy_launches"] = steps_small
+        line["box_copy_GBps"] = {name: traffic_ / (ms * 1e-3) / 1e9 for name, (ms, traffic_) in boxes.items()}
+        line["box_copy_us"] = {name: ms * 1e3 for name, (ms, _) in boxes.items()}
+    if "gemm_rs" in only:
+        rs = run_gemm_rs(device, steps_small, args.warmup, gated)
+        line["gemm_rs"] = {
+            "launches": rs["launches"],
+            "producer_tflops": rs["flop"] / (rs["producer_ms"] * 1e-3) / 1e12,
+            "producer_pct_bf16_mfma_peak": 100.0 * rs["flop"] / (rs["producer_ms"] * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+            "producer_ms": rs["producer_ms"],
+        }
+        if gated:
+            line["gemm_rs"].update({
+                "fused_step_ms": rs["fused_step_ms"],
+                "fused_step_ms_by_programs": rs["fused_step_ms_by_programs"],
+                "fused_step_tflops": rs["flop"] / (rs["fused_step_ms"] * 1e-3) / 1e12,
+                "fused_step_over_producer_pct": 100.0 * (rs["fused_step_ms"] - rs["producer_ms"]) / rs["producer_ms"],
+                "reduce_matches": rs["reduce_matches"],
+                "pushed_chunks_match": rs["pushed_chunks_match"],
+            })
+    if "attn_ag" in only:
+        ag = run_attention_ag(device, gated=gated)
+        line["attn_allgather"] = dict(ag, tflops=ag["flop"] / (ag["ms"] * 1e-3) / 1e12,
+                                      pct_bf16_mfma_peak=100.0 * ag["flop"] / (ag["ms"] * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS)
+    if "attn_a2a" in only:
+        line["attn_all2all"] = run_attention_a2a(device, gated=gated)
+    if "cpu" in only:
         line["cpu_baseline"] = cpu_baseline(state)
+        line["cpu_baselines_other"] = cpu_baselines_other()
     print(json.dumps(line))
 
 

@@ -364,6 +364,15 @@ int syn_stream_destroy(syn_stream_t stream);
  * No counterpart in the reference; it is how a partition of the device is checked. */
 int syn_where_async(uint32_t* out, int32_t workgroups, int32_t dwell, syn_stream_t stream);
 
+/* Measurement aid, no counterpart in the reference: `workgroups` workgroups of four wavefronts
+ * each run `iters` rounds of 64 v_mfma_f32_32x32x16_bf16 per wavefront (the GEMM kernels' 4 x 4
+ * accumulator pattern) on register-resident operands - no LDS, no memory.  pattern 0: zero
+ * operands, 1: all ones, 2: pseudo-random N(0, 0.02)-like values.  flop = workgroups * 4 * iters *
+ * 64 * 32768.  sink: device float[workgroups * 256].  The rate with pattern 2 is what the matrix
+ * pipes sustain under the board's power limit when operand bits toggle. */
+int syn_probe_mfma_rate(float* sink, int32_t workgroups, int32_t iters, int32_t pattern,
+                        syn_stream_t stream);
+
 /* Library/ABI version: major*10000 + minor*100 + patch. */
 int syn_version(void);
 

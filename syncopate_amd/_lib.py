@@ -170,6 +170,7 @@ _SIGNATURES = {
     "syn_stream_create_cu_mask": (c_int32, [POINTER(ctypes.c_uint32), ctypes.c_uint32, POINTER(c_void_p)]),
     "syn_stream_destroy": (c_int32, [c_void_p]),
     "syn_where_async": (c_int32, [c_void_p, c_int32, c_int32, c_void_p]),
+    "syn_probe_mfma_rate": (c_int32, [c_void_p, c_int32, c_int32, c_int32, c_void_p]),
     "syn_version": (c_int32, []),
 }
 

@@ -56,7 +56,8 @@ class CommContext:
     def __init__(self, rank: int, info: CommInfo, multi_info: bool = False, *,
                  device: Optional[torch.device] = None, link_delay_us: int = 0,
                  wait_timeout_us: int = 2_000_000, copy_blocks: int = 0, flag_sets: int = 1,
-                 compute_stream: Optional[torch.cuda.Stream] = None, fuse_flags: bool = False) -> None:
+                 compute_stream: Optional[torch.cuda.Stream] = None, fuse_flags: bool = False,
+                 lead_copy_blocks: int = 0) -> None:
         if info.local_world_size <= 0:
             info.local_world_size = info.world_size
         if info.local_world_size != info.world_size:
@@ -79,6 +80,10 @@ class CommContext:
         self.fuse_flags = bool(fuse_flags)
         if self.fuse_flags and self.copy_blocks <= 0:
             raise ValueError("fuse_flags needs the copy kernel: copy_blocks > 0")
+        # > 0: among the leading ops of execute(lead_ops=n), a copy that is followed by its flag
+        # write is ONE kernel of that many workgroups that copies and then sets the flag.  The
+        # compute kernel has not been launched yet, so these copies may take the whole device.
+        self.lead_copy_blocks = int(lead_copy_blocks)
         self._lib = _lib.load()
         world = info.local_world_size
 
@@ -187,32 +192,46 @@ class CommContext:
             return self.recv_signal_bufs[rank]
         raise NotImplementedError(f"Signal type {signal_type} not implemented yet.")
 
-    def execute(self, neglect_local: bool = False, lead_ops: int = 0) -> None:
+    def execute(self, neglect_local: bool = False, lead_ops: int = 0,
+                lead_on: Optional[torch.cuda.Stream] = None) -> None:
         """Enqueue this rank's ops, stream by stream, in list order.
 
         `lead_ops` > 0 records an event behind the first `lead_ops` ops of every stream;
         `wait_lead(stream)` makes a stream wait for them.  Launch order gives the copies that
         head start over the compute kernel when everything is launched from the host; inside a
         replayed graph the kernel and the first copy become ready at the same moment, the kernel
-        takes the compute units, and every chunk of the iteration arrives later."""
+        takes the compute units, and every chunk of the iteration arrives later.
+
+        `lead_on` (with `lead_ops`): the leading ops are enqueued on THAT stream - the compute
+        stream, in front of the kernel - and the communication stream carries on behind them.
+        A kernel that waits for an event of another hardware queue starts some 10 us after the
+        event; behind ops of its own stream it starts at once.  Only for leading ops that wait
+        for nothing the compute stream's later kernels set."""
         self._lead_events = []
         self._check_copy_units(self.info.operations[self.rank])
         for lane, (stream, ops) in enumerate(zip(self.streams, self.info.operations[self.rank])):
-            handle = int(stream.cuda_stream)
             lead = min(lead_ops, len(ops))
             index = 0
             while index < len(ops):
                 op, done = ops[index], 1
-                if (self.fuse_flags and isinstance(op, CopyEngineOp) and index + 1 < len(ops)
+                on = lead_on if (lead_on is not None and index < lead) else stream
+                handle = int(on.cuda_stream)
+                blocks = self.copy_blocks if self.fuse_flags else 0
+                if self.lead_copy_blocks > 0 and index + 1 < lead:
+                    blocks = self.lead_copy_blocks
+                if (blocks > 0 and isinstance(op, CopyEngineOp) and index + 1 < len(ops)
                         and isinstance(ops[index + 1], IntraNodeSignal)
-                        and self._issue_copy_with_flag(op, ops[index + 1], lane, handle, neglect_local)):
+                        and self._issue_copy_with_flag(op, ops[index + 1], lane, handle, neglect_local, blocks)):
                     done = 2
                 else:
-                    self._issue(op, self.rank, stream, handle, neglect_local)
+                    self._issue(op, self.rank, on, handle, neglect_local)
                 if lead_ops > 0 and index < lead <= index + done:
                     event = torch.cuda.Event()
-                    event.record(stream)
-                    self._lead_events.append(event)
+                    event.record(on)
+                    if lead_on is not None:
+                        stream.wait_event(event)      # the rest of the list follows the leading ops
+                    else:
+                        self._lead_events.append(event)
                 index += done
         self._zero_stale_set()
 
@@ -375,7 +394,7 @@ class CommContext:
             raise ValueError("box copies run on compute units: set CommInfo.num_copy_sms first")
 
     def _issue_copy_with_flag(self, op: CopyEngineOp, flag_op: IntraNodeSignal, lane: int, handle: int,
-                              neglect_local: bool) -> bool:
+                              neglect_local: bool, blocks: int) -> bool:
         """A copy and the flag write behind it as one kernel; False if the pair does not qualify
         (then both are issued on their own)."""
         world = self.info.local_world_size
@@ -399,7 +418,7 @@ class CommContext:
             _lib.check("syn_delay_us", lib.syn_delay_us(self.link_delay_us, handle))
         _lib.check("syn_copy_flag_async",
                    lib.syn_copy_flag_async(dst_ptr, src_ptr, op.size, flags.data_ptr() + 8 * flag_op.offset, 1,
-                                           self._tickets.data_ptr() + 4 * lane, self.copy_blocks, handle))
+                                           self._tickets.data_ptr() + 4 * lane, blocks, handle))
         return True
 
     def _issue(self, op, owner: int, stream: torch.cuda.Stream, handle: int, neglect_local: bool) -> None:
