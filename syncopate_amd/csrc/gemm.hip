@@ -693,6 +693,17 @@ __device__ __forceinline__ void atomic_add4<_Float16>(_Float16* dst, uint2 v) {
     __builtin_amdgcn_global_atomic_fadd_v2f16((gptr)(dst + 2), __builtin_bit_cast(v2, v.y));
 }
 
+// 16 bytes stored through the XCD's L2 to memory (the agent-scope form of a store: what a relaxed
+// atomic store at that scope compiles to, which exists for 8 bytes at most).  A vector store.
+// A store of more than 8 bytes reads its data registers for two more issue slots; the compiler
+// keeps vector instructions that write them away from its own stores but does not see this one,
+// hence the s_nop.
+__device__ __forceinline__ void store16_write_through(void* dst, uint4 v) {
+    typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+    const u32x4 data = {v.x, v.y, v.z, v.w};
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(dst), "v"(data) : "memory");
+}
+
 template <typename T, typename Pipe, int BM, int BN, int WGM, int WGN, int MODE>
 __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmParams p) {
     constexpr bool PRODUCER = MODE == kProducer;
@@ -953,12 +964,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
                         if (PRODUCER) {
                             // written through the XCD's L2: the release below then has nothing
                             // of this tile left to write back
-                            __hip_atomic_store(reinterpret_cast<uint64_t*>(dst),
-                                               (uint64_t)v.x | ((uint64_t)v.y << 32), __ATOMIC_RELAXED,
-                                               __HIP_MEMORY_SCOPE_AGENT);
-                            __hip_atomic_store(reinterpret_cast<uint64_t*>(dst) + 1,
-                                               (uint64_t)v.z | ((uint64_t)v.w << 32), __ATOMIC_RELAXED,
-                                               __HIP_MEMORY_SCOPE_AGENT);
+                            store16_write_through(dst, v);
                         } else {
                             *reinterpret_cast<uint4*>(dst) = v;
                         }
