@@ -611,8 +611,18 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
         const unsigned char* v_base = V + (z * p.v_st[0] + h * p.v_st[1]) * (int64_t)sizeof(T) +
                                       (size_t)kv_lo * kBlockN * v_pitch;
 
+        // With the XCD remap the workgroups of an XCD work on the q blocks of one or two heads at the
+        // same time and read the same K and V: each pair starts its walk over the wave's kv blocks
+        // one block after its neighbour's and wraps around, so that they ask the L2 for different
+        // lines at any moment while staying within a window of blocks that the L2 holds (the sum
+        // over kv blocks is order-free up to rounding).
+        const int rot = p.xcd_remap ? (int)((unsigned)pair % (unsigned)nkv) : 0;
+        auto blk = [&](const int m) {
+            const int b = m + rot;
+            return b >= nkv ? b - nkv : b;
+        };
         // every wavefront has passed the barrier that ended the previous pair: all four buffers are free
-        dma_kv_block8(k_lds, k_base, k_pitch, k_fill_off, wave8);
+        dma_kv_block8(k_lds, k_base + (size_t)blk(0) * kBlockN * k_pitch, k_pitch, k_fill_off, wave8);
 
         frag_t qf[8];
 #pragma unroll
@@ -638,10 +648,10 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
         // measured 1-6 % slower: a wavefront stalls at every fill wherever it is placed.)
         auto fetch = [&](const int m) {
             __builtin_amdgcn_sched_barrier(0);
-            dma_kv_block8(v_lds + (m & 1) * kBlockBytes, v_base + (size_t)m * kBlockN * v_pitch, v_pitch, v_fill_off,
+            dma_kv_block8(v_lds + (m & 1) * kBlockBytes, v_base + (size_t)blk(m) * kBlockN * v_pitch, v_pitch, v_fill_off,
                           wave8);
             if (m + 1 < nkv)
-                dma_kv_block8(k_lds + ((m + 1) & 1) * kBlockBytes, k_base + (size_t)(m + 1) * kBlockN * k_pitch,
+                dma_kv_block8(k_lds + ((m + 1) & 1) * kBlockBytes, k_base + (size_t)blk(m + 1) * kBlockN * k_pitch,
                               k_pitch, k_fill_off, wave8);
             __builtin_amdgcn_sched_barrier(0);
         };
