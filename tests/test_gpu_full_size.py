@@ -233,3 +233,48 @@ def test_c1_mesh4_fp16_gathered_4096x512_times_512x1024(hip):
         torch.cuda.current_stream().wait_stream(side)
         check_status()
         assert torch.equal(c_gated, c)          # same tile shape: bitwise the resident result
+
+
+def test_allgather_attention_full_size_with_chunks_arriving_behind_flags(hip):
+    """The all-gather attention configuration at its full size with real gating: only the rank's own
+    kv chunk is resident (the rest of the buffer is NaN), the other seven are copied in on a side
+    stream in double-ring arrival order - a box copy on 32 compute units, then the chunk's flag -
+    while 224 persistent workgroups (two q blocks each) already run.  Sampled heads against torch's
+    attention in fp32 on the GPU; the gathered buffer bit for bit."""
+    from syncopate_amd import _lib
+    from syncopate_amd.communication.comm_runtime.persistent_copy import persistent_copy_last_contig
+    from syncopate_amd.communication.comm_runtime.streams import pick_side_streams
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.attn import attention_forward
+
+    B, H, Sq, Skv, D, chunks = 1, 32, 4096, 32768, 128, 8
+    g = torch.Generator(device="cuda").manual_seed(1)
+    q = torch.randn(B, H, Sq, D, device="cuda", generator=g).bfloat16()
+    kv = torch.randn(2, B, H, Skv, D, device="cuda", generator=g).bfloat16()
+    chunk = Skv // chunks
+    arrival, signals = [0, 1, 7, 6, 4, 5, 3, 2], [-1, 0, 4, 1, 5, 2, 6, 3]
+    tables = _attn_tables(B, H, Sq, chunk, arrival, signals)
+    buf = torch.full_like(kv, float("nan"))
+    buf[:, :, :, :chunk].copy_(kv[:, :, :, :chunk])
+    flags = torch.zeros(chunks, dtype=torch.int64, device="cuda")
+    main = torch.cuda.current_stream()
+    side = pick_side_streams(1, main, torch.device("cuda", torch.cuda.current_device()))[0]
+    torch.cuda.synchronize()
+    side.wait_stream(main)
+    with torch.cuda.stream(side):
+        for wave in range(1, chunks):
+            c = arrival[wave]
+            _lib.check("syn_delay_us", hip.syn_delay_us(100, _lib.stream_handle(side)))
+            persistent_copy_last_contig(kv[:, :, :, c * chunk:(c + 1) * chunk], buf[:, :, :, c * chunk:(c + 1) * chunk],
+                                        num_sms=32)
+            _lib.check("syn_flag_set", hip.syn_flag_set(flags.data_ptr() + 8 * signals[wave], 1, _lib.stream_handle(side)))
+    o = attention_forward(q, buf[0], buf[1], D ** -0.5, signal_ptr=flags, pair_q_blocks=True, num_programs=224,
+                          spin_timeout_us=5_000_000, **tables)
+    main.wait_stream(side)
+    check_status()
+    assert flags.tolist()[:7] == [1] * 7
+    assert torch.equal(buf, kv)
+    assert not torch.isnan(o).any()
+    for h in (0, 17, 31):
+        s = (q[0, h].float() @ kv[0, 0, h].float().t()) * D ** -0.5
+        assert _rel(o[0, h], torch.softmax(s, dim=-1) @ kv[1, 0, h].float()) <= REL_TOL
