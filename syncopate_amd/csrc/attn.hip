@@ -88,6 +88,32 @@ struct AttnMfma<_Float16> {
     }
 };
 
+// The merged partial results (O, lse) of a q block pass from workgroup to workgroup, possibly on
+// different XCDs, whose L2s are not coherent with each other.  A release / acquire fence pair
+// would do it - but a release writes back every dirty line of the XCD's L2 and an acquire drops
+// its clean lines, for all 32 compute units, once per tile: measured, the fences alone kept the
+// kernel at two thirds of its time.  So these few words are stored THROUGH the L2 and loaded PAST
+// it (the agent-scope forms of a store and a load), and the lock hand-over needs no fence: the
+// stores have been acknowledged by memory before the lock word is written.
+template <typename V>
+__device__ __forceinline__ V load8_coherent(const void* ptr) {
+    const uint64_t bits = __hip_atomic_load(reinterpret_cast<const uint64_t*>(ptr), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return __builtin_bit_cast(V, bits);
+}
+template <typename V>
+__device__ __forceinline__ void store8_through(void* ptr, V value) {
+    __hip_atomic_store(reinterpret_cast<uint64_t*>(ptr), __builtin_bit_cast(uint64_t, value), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_f32_coherent(const float* ptr) {
+    return __builtin_bit_cast(float, __hip_atomic_load(reinterpret_cast<const uint32_t*>(ptr), __ATOMIC_RELAXED,
+                                                       __HIP_MEMORY_SCOPE_AGENT));
+}
+__device__ __forceinline__ void store_f32_through(float* ptr, float value) {
+    __hip_atomic_store(reinterpret_cast<uint32_t*>(ptr), __builtin_bit_cast(uint32_t, value), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
@@ -132,6 +158,7 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
     __shared__ __attribute__((aligned(1024))) unsigned char k_lds[kBlockBytes];
     __shared__ __attribute__((aligned(1024))) unsigned char v_lds[kBlockBytes];
     __shared__ int s_abort;
+    __shared__ int s_spun;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -224,14 +251,18 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
         if (wait_sig >= 0) {
             if (tid == 0) {
                 const uint64_t* wait_flags = p.wait_flags != nullptr ? p.wait_flags : p.flags;
-                const bool ok = spin_until_equal(wait_flags + wait_sig, 1ull, p.timeout_ticks);
-                if (!ok) {
+                s_spun = __hip_atomic_load(wait_flags + wait_sig, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 1ull;
+                if (s_spun && !spin_until_equal(wait_flags + wait_sig, 1ull, p.timeout_ticks)) {
                     report_status(p.status, SYN_STATUS_SPIN_TIMEOUT, w, (int)blockIdx.x, wait_sig);
                     s_abort = 1;
                 }
             }
             __syncthreads();
-            acquire_fence_agent();
+            // Nothing reads a chunk's lines before its flag is up, so this XCD's L2 cannot hold a stale one
+            // (it was emptied when the kernel began); the fence - it drops every clean line of the L2, the K
+            // and V blocks other workgroups are about to reuse among them - is kept for the workgroup that
+            // really had to wait.
+            if (s_spun) acquire_fence_agent();
             if (s_abort) return;
         }
 
@@ -438,7 +469,6 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
             }
         }
         __syncthreads();
-        acquire_fence_agent();
         if (s_abort) return;
 
         const bool is_first = __hip_atomic_load(p.first + lock_idx, __ATOMIC_RELAXED,
@@ -447,7 +477,7 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
         float* lse_ptr = p.lse + head * p.Sq + q_row;
         if (!is_first) {
             // merge with the stored partial (template.py:335-349)
-            const float m_old = *lse_ptr;
+            const float m_old = load_f32_coherent(lse_ptr);
             const float delta = m_old - lse2;
             const float mmax = fmaxf(m_old, lse2);
             lse_out = mmax + fast_log2(1.0f + fast_exp2(-fabsf(delta)));
@@ -464,22 +494,24 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
                 for (int c = 0; c < 4; ++c) x[c] = o_acc[i][4 * g + c] * inv_l * w_new;
                 T* dst = o_row + 32 * i + 8 * g;
                 if (!is_first) {
-                    const vec4_t old = *reinterpret_cast<const vec4_t*>(dst);
+                    const vec4_t old = load8_coherent<vec4_t>(dst);
 #pragma unroll
                     for (int c = 0; c < 4; ++c) x[c] += (float)old[c] * w_old;
                 }
                 vec4_t out;
 #pragma unroll
                 for (int c = 0; c < 4; ++c) out[c] = (T)x[c];
-                *reinterpret_cast<vec4_t*>(dst) = out;
+                store8_through(dst, out);
             }
-        if (half == 0) *lse_ptr = lse_out;
+        if (half == 0) store_f32_through(lse_ptr, lse_out);
 
-        __threadfence();
+        // every lane's stores have been acknowledged by memory; then the barrier; then the hand-over
+        __builtin_amdgcn_s_waitcnt(attn_vmcnt(0));
         __syncthreads();
         if (tid == 0) {
             __hip_atomic_store(p.first + lock_idx, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(p.lock + lock_idx, 0, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+            __builtin_amdgcn_s_waitcnt(attn_vmcnt(0));
+            __hip_atomic_store(p.lock + lock_idx, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             count_tile();
         }
     }
@@ -525,6 +557,7 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
     __shared__ __attribute__((aligned(1024))) unsigned char k_lds[2 * kBlockBytes];
     __shared__ __attribute__((aligned(1024))) unsigned char v_lds[2 * kBlockBytes];
     __shared__ int s_abort;
+    __shared__ int s_spun;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -592,14 +625,14 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
 
         if (sig >= 0) {
             if (tid == 0) {
-                const bool ok = spin_until_equal(p.flags + sig, 1ull, p.timeout_ticks);
-                if (!ok) {
+                s_spun = __hip_atomic_load(p.flags + sig, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 1ull;
+                if (s_spun && !spin_until_equal(p.flags + sig, 1ull, p.timeout_ticks)) {
                     report_status(p.status, SYN_STATUS_SPIN_TIMEOUT, w, (int)blockIdx.x, sig);
                     s_abort = 1;
                 }
             }
             __syncthreads();
-            acquire_fence_agent();
+            if (s_spun) acquire_fence_agent();       // see attn_fwd_kernel
             if (s_abort) return;
         }
 
@@ -836,14 +869,13 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
             }
         }
         __syncthreads();
-        acquire_fence_agent();
         if (s_abort) return;
 
         const bool is_first = __hip_atomic_load(p.first + lock_idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0;
         float w_old = 0.f, w_new = 1.f, lse_out = lse2;
         float* lse_ptr = p.lse + head * p.Sq + q_row;
         if (!is_first) {
-            const float m_old = *lse_ptr;
+            const float m_old = load_f32_coherent(lse_ptr);
             const float delta = m_old - lse2;
             const float mmax = fmaxf(m_old, lse2);
             lse_out = mmax + fast_log2(1.0f + fast_exp2(-fabsf(delta)));
@@ -860,25 +892,27 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
                 for (int c = 0; c < 4; ++c) x[c] = o_acc[i][4 * g + c] * inv_l * w_new;
                 T* dst = o_row + 32 * i + 8 * g;
                 if (!is_first) {
-                    const vec4_t old = *reinterpret_cast<const vec4_t*>(dst);
+                    const vec4_t old = load8_coherent<vec4_t>(dst);
 #pragma unroll
                     for (int c = 0; c < 4; ++c) x[c] += (float)old[c] * w_old;
                 }
                 vec4_t out;
 #pragma unroll
                 for (int c = 0; c < 4; ++c) out[c] = (T)x[c];
-                *reinterpret_cast<vec4_t*>(dst) = out;
+                store8_through(dst, out);
             }
-        if (half == 0) *lse_ptr = lse_out;
+        if (half == 0) store_f32_through(lse_ptr, lse_out);
 
-        __threadfence();
+        // every lane's stores have been acknowledged by memory; then the barrier; then the hand-over
+        __builtin_amdgcn_s_waitcnt(attn_vmcnt(0));
         __syncthreads();
         if (tid == 0) {
             // tid 0 is in group 0: its lock_idx is the lower q block of the pair
-            for (int which = 1; which >= 0; --which) {
-                __hip_atomic_store(p.first + lock_idx + which, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __hip_atomic_store(p.lock + lock_idx + which, 0, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-            }
+            __hip_atomic_store(p.first + lock_idx, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(p.first + lock_idx + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __builtin_amdgcn_s_waitcnt(attn_vmcnt(0));
+            __hip_atomic_store(p.lock + lock_idx + 1, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(p.lock + lock_idx, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
 }
