@@ -712,6 +712,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
     constexpr int TM = WM / 32, TN = WN / 32;     // 32x32 MFMA tiles per wavefront
 
     __shared__ int s_abort;
+    __shared__ int s_spun;
     // C staging of the epilogue: 32 rows x CS_COLS columns per wavefront, 64 columns where LDS allows
     constexpr int NWAVES = WGM * WGN;
     constexpr int CS_COLS = (!REMOTE && (BN / WGN / 32) % 2 == 0 &&
@@ -789,14 +790,18 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
     auto wait_flag = [&](int sig) -> bool {
         if (tid == 0) {
             const uint64_t* flags = PRODUCER ? p.wait_flags : p.flags;
-            const bool ok = spin_until_equal(flags + sig, 1ull, p.timeout_ticks);
-            if (!ok) {
+            s_spun = __hip_atomic_load(flags + sig, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 1ull;
+            if (s_spun && !spin_until_equal(flags + sig, 1ull, p.timeout_ticks)) {
                 report_status(p.status, SYN_STATUS_SPIN_TIMEOUT, cur_wave, pid, sig);
                 s_abort = 1;
             }
         }
         __syncthreads();
-        acquire_fence_agent();
+        // No program reads a chunk's rows before its flag is up, so the XCD's L2 (emptied when the kernel
+        // began) cannot hold a stale line of it.  The acquire fence drops every clean line of that L2 -
+        // the panels of A and B its 28 other programs are reusing - so only a program that really had
+        // to wait takes it.
+        if (s_spun) acquire_fence_agent();
         return s_abort == 0;
     };
 
@@ -974,13 +979,14 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
 
         if (PRODUCER) {
             if (tile.sig >= 0) {
-                // Every lane's C stores were agent-scope write-through stores; the barrier's wait for
-                // their acknowledgements makes them visible device-wide before thread 0 moves the
-                // count (a release).  No L2 write-back or invalidate: the next tile reuses that L2.
+                // Every lane's C stores were agent-scope write-through stores; the wait for their
+                // acknowledgements in front of the barrier makes them visible device-wide before
+                // thread 0 moves the count.  The count itself is a relaxed atomic: a release would
+                // make the L2 look for dirty lines to write back once per tile, and there are none.
                 __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, true));
                 __syncthreads();
                 if (tid == 0) {
-                    const int done = __hip_atomic_fetch_add(p.counters + tile.wave, 1, __ATOMIC_RELEASE,
+                    const int done = __hip_atomic_fetch_add(p.counters + tile.wave, 1, __ATOMIC_RELAXED,
                                                             __HIP_MEMORY_SCOPE_AGENT);
                     if (done == tile.wave_tiles - 1)
                         __hip_atomic_store(p.flags + tile.sig, 1ull, __ATOMIC_RELEASE,
