@@ -56,7 +56,8 @@ LEAD_COPY_BLOCKS = 0                 # see --lead-copy-blocks
 LEAD_ON_COMPUTE_STREAM = False       # see --lead-on-compute-stream
 LINK_CHUNK_US = 110                  # one 16.8 MB chunk over one xGMI link (~153 GB/s)
 
-SECTIONS = ("ag_gemm", "throttled", "mfma_ceiling", "reduce", "box_copies", "gemm_rs", "attn_ag", "attn_a2a", "cpu")
+SECTIONS = ("ag_gemm", "throttled", "mfma_ceiling", "library", "reduce", "box_copies", "gemm_rs", "attn_ag", "attn_a2a",
+            "cpu")
 
 
 def _events(n):
@@ -331,6 +332,36 @@ def run_mfma_ceiling(device, state, launches=8):
         ms = state["resident_ms_fn"](zeros_a, zeros_b)
         out["consumer_kernel_zero_operands_tflops"] = 2.0 * M * N * K / ms / 1e9
         out["consumer_kernel_zero_operands_ms"] = ms
+    return out
+
+
+def run_library_baselines(device, state):
+    """The vendor libraries on the same operands, for scale (not part of the path: they take whole,
+    resident operands and know nothing of chunks or flags): torch.matmul (hipBLASLt) on the two
+    GEMM shapes, torch's scaled_dot_product_attention on the two attention shapes."""
+    import torch.nn.functional as F
+
+    out = {"launches": 30}
+    a, b = state["a"], state["b"]
+    ms = _timed(lambda i: torch.matmul(a, b.t()), 30, 10)
+    out["matmul_8192x8192x3584_tflops"] = 2.0 * M * N * K / ms / 1e9
+    a2 = (0.02 * torch.randn(8192, 3584, device=device)).bfloat16()
+    b2 = (0.02 * torch.randn(8192, 3584, device=device)).bfloat16()
+    ms = _timed(lambda i: torch.matmul(a2, b2.t()), 30, 10)
+    out["matmul_8192x3584x8192_tflops"] = 2.0 * 8192 * 8192 * 3584 / ms / 1e9
+    za, zb = torch.zeros_like(a), torch.zeros_like(b)
+    ms = _timed(lambda i: torch.matmul(za, zb.t()), 30, 10)
+    out["matmul_8192x8192x3584_zero_operands_tflops"] = 2.0 * M * N * K / ms / 1e9
+    del a2, b2, za, zb
+    q = torch.randn(1, 32, 4096, 128, device=device).bfloat16()
+    k = torch.randn(1, 32, 32768, 128, device=device).bfloat16()
+    v = torch.randn(1, 32, 32768, 128, device=device).bfloat16()
+    ms = _timed(lambda i: F.scaled_dot_product_attention(q, k, v), 5, 2)
+    out["sdpa_4096x32768_32_heads_tflops"] = 4.0 * 32 * 4096 * 32768 * 128 / ms / 1e9
+    q = torch.randn(1, 4, 16384, 128, device=device).bfloat16()
+    k, v = torch.randn_like(q), torch.randn_like(q)
+    ms = _timed(lambda i: F.scaled_dot_product_attention(q, k, v, is_causal=True), 5, 2)
+    out["sdpa_16384_causal_4_heads_tflops"] = 2.0 * 4 * 16384 * 16384 * 128 / ms / 1e9
     return out
 
 
@@ -874,6 +905,8 @@ def main():
         random_ceiling = ceiling.get("random_operands_256_workgroups_tflops")
         if random_ceiling:
             line["roofline"]["frac_of_random_operand_mfma_ceiling"] = kernel_tflops / random_ceiling
+    if "library" in only:
+        line["library_baselines"] = run_library_baselines(device, state)
     steps_small = max(20, min(args.steps, 60))
     if "throttled" in only and gated:
         line["throttled_producer"] = run_throttled(device, 20)
