@@ -999,3 +999,48 @@ def test_all2all_then_split_k_gemm(hip, slices):
     want = want_in.reshape(-1, hidden).float() @ w.float().t()
     assert _rel(out, want) <= 4 * REL_TOL
     assert ctx.recv_signal_bufs[rank].tolist() == [1] * len(shapes)
+
+
+@pytest.mark.parametrize("lead_on_compute_stream,lead_copy_blocks", [(False, 0), (True, 0), (True, 64), (False, 64)])
+def test_leading_ops_ahead_of_the_consumer(hip, lead_on_compute_stream, lead_copy_blocks):
+    """execute(lead_ops=4): the first two chunk copies and their flags are in place before the
+    consumer is launched - through an event the compute stream waits for, or enqueued on the
+    compute stream itself (lead_on), as two kernels each or as one copy-and-flag kernel each
+    (lead_copy_blocks).  Every form must gather the same bytes and give the resident result."""
+    from syncopate_amd.communication.comm_runtime.communication_context import CommContext
+    from syncopate_amd.communication.common_descriptors import build_all_gather_plan_1d_swizzle
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.gemm import gemm
+    from syncopate_amd.interface.wave_tables import gemm_consumer_tables
+
+    world, rank, M, K, N, BM, BN = 4, 2, 2048, 512, 512, 128, 128
+    rows = M // world
+    plans = {r: build_all_gather_plan_1d_swizzle((M, K), torch.bfloat16, 0, world, r, "a", "pull")
+             for r in range(world)}
+    schedules, info = _compile(plans)
+    tables = gemm_consumer_tables(schedules[rank]["a"], N)
+    ctx = CommContext(rank, info, lead_copy_blocks=lead_copy_blocks)
+    g = torch.Generator().manual_seed(21)
+    a = (0.02 * torch.randn(M, K, generator=g)).bfloat16()
+    b = (0.02 * torch.randn(N, K, generator=g)).bfloat16()
+    ad, bd = a.cuda(), b.cuda()
+    for r in range(world):
+        ctx.comm_buffers["a"][r][r * rows:(r + 1) * rows].copy_(ad[r * rows:(r + 1) * rows])
+        if r != rank:
+            ctx.comm_buffers["a"][rank][r * rows:(r + 1) * rows].fill_(float("nan"))
+    c = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
+    cur = torch.cuda.current_stream()
+    for it in range(2):
+        ctx.reset_signals()
+        ctx.start_after(cur)
+        ctx.execute(lead_ops=4, lead_on=cur if lead_on_compute_stream else None)
+        ctx.wait_lead(cur)
+        gemm(ctx.comm_buffers["a"][rank], bd, c, world, 24, BM, BN, 64, 8, cur_wave_sizes=tables.block_shapes,
+             wave_offsets=tables.block_offsets, signal_ptr=ctx.recv_signal_bufs[rank],
+             signal_offsets=tables.signal_offsets, cum_tiles=tables.cum_tiles)
+        ctx.end_before(cur)
+        check_status()
+        ctx.check_status()
+        assert torch.equal(ctx.comm_buffers["a"][rank], ad)
+        assert ctx.recv_signal_bufs[rank].tolist() == [1] * (world - 1)
+        assert _rel(c, numerics.gemm_fp32(a, b)) <= REL_TOL

@@ -62,3 +62,23 @@ def test_device_split_by_compute_unit_masks(hip):
     assert a.sum().item() == b.sum().item() == float(1 << 20)
     assert cu_mask_words(8, 24, 64) == [0xFFFFFF00, 0]
     assert group_sizes(256, 2, 9) == [16, 16, 224]
+
+
+def test_mfma_rate_probe_runs_and_rejects_bad_arguments(hip):
+    """The measurement aid of the benchmark: every pattern runs; constant operands give the exact sum."""
+    from syncopate_amd import _lib
+
+    sink = torch.zeros(4 * 256, dtype=torch.float32, device="cuda")
+    stream = _lib.stream_handle(torch.cuda.current_stream())
+    for pattern in (0, 1, 2):
+        _lib.check("syn_probe_mfma_rate", hip.syn_probe_mfma_rate(sink.data_ptr(), 4, 3, pattern, stream))
+        torch.cuda.synchronize()
+        assert torch.isfinite(sink).all()
+        if pattern == 0:
+            assert (sink == 0).all()
+        if pattern == 1:
+            # 3 rounds x 4 fragment sets x 16 (k) ones per accumulator element, two elements of 16 accumulators summed
+            assert (sink == 3 * 4 * 16 * 2 * 16).all()
+    assert hip.syn_probe_mfma_rate(sink.data_ptr(), 4, 3, 3, stream) == _lib.SYN_EINVAL
+    assert hip.syn_probe_mfma_rate(None, 4, 3, 0, stream) == _lib.SYN_EINVAL
+    assert hip.syn_probe_mfma_rate(sink.data_ptr(), 0, 3, 0, stream) == _lib.SYN_EINVAL
