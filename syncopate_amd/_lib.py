@@ -8,13 +8,15 @@ opened so that both use the same HIP runtime.
 from __future__ import annotations
 
 import ctypes
+import os
 from ctypes import POINTER, c_float, c_int32, c_int64, c_uint32, c_uint64, c_void_p
 from pathlib import Path
 from typing import Optional
 
 import torch  # noqa: F401  (must precede CDLL: loads the HIP runtime the kernels run on)
 
-LIB_PATH = Path(__file__).resolve().parent / "csrc" / "libsyncopate_hip.so"
+# SYNCOPATE_HIP_LIBRARY names another build of the library (for comparing two builds on one device)
+LIB_PATH = Path(os.environ.get("SYNCOPATE_HIP_LIBRARY") or Path(__file__).resolve().parent / "csrc" / "libsyncopate_hip.so")
 
 SYN_DTYPE_BF16 = 0
 SYN_DTYPE_FP16 = 1
