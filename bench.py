@@ -85,7 +85,8 @@ def _table(rows, device):
 
 # ----------------------------------------------------------------------------------- AG+GEMM
 
-def build_ag_gemm(device, copy_blocks=0, split_units=0, fuse_flags=False, link_delay_us=0, lead_copy_blocks=0):
+def build_ag_gemm(device, copy_blocks=0, split_units=0, fuse_flags=False, link_delay_us=0, lead_copy_blocks=0,
+                  flag_write_values=False):
     from syncopate_amd.communication.code_gen import CommGenerator
     from syncopate_amd.communication.comm_runtime.communication_context import CommContext
     from syncopate_amd.communication.common_descriptors import build_all_gather_plan_1d_swizzle
@@ -112,7 +113,7 @@ def build_ag_gemm(device, copy_blocks=0, split_units=0, fuse_flags=False, link_d
     b = (0.02 * torch.randn(N, K, device=device)).bfloat16()
     # two flag sets: the reset of one iteration's flags happens behind the next one's copies
     ctx = CommContext(RANK, info, device=device, copy_blocks=copy_blocks, flag_sets=2, fuse_flags=fuse_flags,
-                      link_delay_us=link_delay_us, lead_copy_blocks=lead_copy_blocks)
+                      link_delay_us=link_delay_us, lead_copy_blocks=lead_copy_blocks, flag_write_values=flag_write_values)
     rows = M // WORLD
     for r in range(WORLD):     # every rank's symmetric buffer holds its own shard
         ctx.comm_buffers["a"][r][r * rows:(r + 1) * rows].copy_(a[r * rows:(r + 1) * rows])
@@ -796,6 +797,8 @@ def main():
                          "consumer's, by compute-unit masks")
     ap.add_argument("--lead-copy-blocks", type=int, default=LEAD_COPY_BLOCKS,
                     help="N > 0: a leading chunk copy and its flag write are one kernel of N workgroups")
+    ap.add_argument("--flag-write-values", action="store_true",
+                    help="with --no-graph: flag writes are stream memory operations instead of one-wavefront kernels")
     ap.add_argument("--lead-on-compute-stream", action="store_true",
                     help="the leading ops run on the compute stream itself, in front of the kernel")
     ap.add_argument("--lead-ops", type=int, default=LEAD_OPS,
@@ -828,7 +831,7 @@ def main():
         sys.exit("--split-device splits the compute units between two streams: it needs the copy kernel "
                  "(--copy-blocks N) and launches from the host (--no-graph; a graph's kernel nodes carry no mask)")
     state = build_ag_gemm(device, args.copy_blocks, args.split_device, args.fuse_flags,
-                          lead_copy_blocks=args.lead_copy_blocks)
+                          lead_copy_blocks=args.lead_copy_blocks, flag_write_values=args.flag_write_values)
     with torch.cuda.stream(state["ctx"].compute_stream):
         wall_ms, gated_ms, no_lead_ms, resident_ms = run_ag_gemm(state, args.steps, args.warmup, args.resident_only,
                                                                  not args.no_graph)

@@ -343,6 +343,11 @@ int syn_box_copy_async(void* dst, const void* src, int32_t ndim, const int64_t* 
                        const int64_t* src_strides, const int64_t* dst_strides, int32_t elem_kind,
                        int32_t reduce_mode, int32_t num_blocks, syn_stream_t stream);
 int syn_flag_set(uint64_t* flag, uint64_t value, syn_stream_t stream);
+/* The same flag write as a stream memory operation (hipStreamWriteValue64, the counterpart of the
+ * reference's cuStreamWriteValue, communication_context.py:150): no kernel, so no compute unit, and none
+ * of the cache maintenance a kernel boundary brings.  For streams driven from the host: recorded into a
+ * HIP graph such a write has been seen to take effect on the first replay only. */
+int syn_flag_write_value(uint64_t* flag, uint64_t value, syn_stream_t stream);
 int syn_flag_wait(const uint64_t* flag, uint64_t value, int64_t spin_timeout_us,
                   int32_t* status, syn_stream_t stream);
 /* Occupy the stream for about `us` microseconds with one sleeping wavefront

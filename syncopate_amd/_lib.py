@@ -167,6 +167,7 @@ _SIGNATURES = {
     "syn_box_copy_async": (c_int32, [c_void_p, c_void_p, c_int32, POINTER(c_int64), POINTER(c_int64),
                                      POINTER(c_int64), c_int32, c_int32, c_int32, c_void_p]),
     "syn_flag_set": (c_int32, [c_void_p, c_uint64, c_void_p]),
+    "syn_flag_write_value": (c_int32, [c_void_p, c_uint64, c_void_p]),
     "syn_flag_wait": (c_int32, [c_void_p, c_uint64, c_int64, c_void_p, c_void_p]),
     "syn_delay_us": (c_int32, [c_int64, c_void_p]),
     "syn_stream_create_cu_mask": (c_int32, [POINTER(ctypes.c_uint32), ctypes.c_uint32, POINTER(c_void_p)]),

@@ -57,7 +57,7 @@ class CommContext:
                  device: Optional[torch.device] = None, link_delay_us: int = 0,
                  wait_timeout_us: int = 2_000_000, copy_blocks: int = 0, flag_sets: int = 1,
                  compute_stream: Optional[torch.cuda.Stream] = None, fuse_flags: bool = False,
-                 lead_copy_blocks: int = 0) -> None:
+                 lead_copy_blocks: int = 0, flag_write_values: bool = False) -> None:
         if info.local_world_size <= 0:
             info.local_world_size = info.world_size
         if info.local_world_size != info.world_size:
@@ -84,6 +84,8 @@ class CommContext:
         # write is ONE kernel of that many workgroups that copies and then sets the flag.  The
         # compute kernel has not been launched yet, so these copies may take the whole device.
         self.lead_copy_blocks = int(lead_copy_blocks)
+        # flag writes as stream memory operations instead of one-wavefront kernels (outside graph capture)
+        self.flag_write_values = bool(flag_write_values)
         self._lib = _lib.load()
         world = info.local_world_size
 
@@ -450,7 +452,10 @@ class CommContext:
             flags = self.recv_signal_bufs[op.rank % world]
             if not 0 <= op.offset < flags.numel():
                 raise ValueError(f"{op} is outside the flag array")
-            _lib.check("syn_flag_set", lib.syn_flag_set(flags.data_ptr() + 8 * op.offset, 1, handle))
+            if self.flag_write_values and not torch.cuda.is_current_stream_capturing():
+                _lib.check("syn_flag_write_value", lib.syn_flag_write_value(flags.data_ptr() + 8 * op.offset, 1, handle))
+            else:
+                _lib.check("syn_flag_set", lib.syn_flag_set(flags.data_ptr() + 8 * op.offset, 1, handle))
         elif isinstance(op, WaitIntraNodeSignal):
             flags = self._flags(op.signal_type, op.rank % world)
             if not 0 <= op.offset < flags.numel():

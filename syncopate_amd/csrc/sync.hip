@@ -429,6 +429,11 @@ int syn_flag_set(uint64_t* flag, uint64_t value, syn_stream_t stream) {
     return (int)hipGetLastError();
 }
 
+int syn_flag_write_value(uint64_t* flag, uint64_t value, syn_stream_t stream) {
+    if (!flag) return SYN_EINVAL;
+    return (int)hipStreamWriteValue64(reinterpret_cast<hipStream_t>(stream), flag, value, 0);
+}
+
 int syn_flag_wait(const uint64_t* flag, uint64_t value, int64_t spin_timeout_us, int32_t* status,
                   syn_stream_t stream) {
     if (!flag) return SYN_EINVAL;

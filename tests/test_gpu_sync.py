@@ -82,3 +82,17 @@ def test_mfma_rate_probe_runs_and_rejects_bad_arguments(hip):
     assert hip.syn_probe_mfma_rate(sink.data_ptr(), 4, 3, 3, stream) == _lib.SYN_EINVAL
     assert hip.syn_probe_mfma_rate(None, 4, 3, 0, stream) == _lib.SYN_EINVAL
     assert hip.syn_probe_mfma_rate(sink.data_ptr(), 0, 3, 0, stream) == _lib.SYN_EINVAL
+
+
+def test_flag_write_as_a_stream_memory_operation(hip):
+    """syn_flag_write_value: the flag word is written by the stream itself, in stream order."""
+    from syncopate_amd import _lib
+
+    flags = torch.zeros(4, dtype=torch.int64, device="cuda")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    _lib.check("syn_delay_us", hip.syn_delay_us(500, _lib.stream_handle(side)))
+    _lib.check("syn_flag_write_value", hip.syn_flag_write_value(flags.data_ptr() + 16, 1, _lib.stream_handle(side)))
+    side.synchronize()
+    assert flags.tolist() == [0, 0, 1, 0]
+    assert hip.syn_flag_write_value(None, 1, _lib.stream_handle(side)) == _lib.SYN_EINVAL
