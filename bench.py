@@ -53,6 +53,7 @@ LEAD_OPS = 3                         # ops of the side stream the consumer launc
                                      # first one's flag set (the second flag lands while the first tiles run)
 EIGHT_WAVES = False                  # 256-thread workgroups: one wavefront per SIMD, 128x128 of C each
 LEAD_COPY_BLOCKS = 0                 # see --lead-copy-blocks
+LIST_BLOCKS = 0                      # see --list-blocks
 LEAD_ON_COMPUTE_STREAM = False       # see --lead-on-compute-stream
 LINK_CHUNK_US = 110                  # one 16.8 MB chunk over one xGMI link (~153 GB/s)
 
@@ -86,7 +87,7 @@ def _table(rows, device):
 # ----------------------------------------------------------------------------------- AG+GEMM
 
 def build_ag_gemm(device, copy_blocks=0, split_units=0, fuse_flags=False, link_delay_us=0, lead_copy_blocks=0,
-                  flag_write_values=False):
+                  flag_write_values=False, list_blocks=0):
     from syncopate_amd.communication.code_gen import CommGenerator
     from syncopate_amd.communication.comm_runtime.communication_context import CommContext
     from syncopate_amd.communication.common_descriptors import build_all_gather_plan_1d_swizzle
@@ -113,7 +114,8 @@ def build_ag_gemm(device, copy_blocks=0, split_units=0, fuse_flags=False, link_d
     b = (0.02 * torch.randn(N, K, device=device)).bfloat16()
     # two flag sets: the reset of one iteration's flags happens behind the next one's copies
     ctx = CommContext(RANK, info, device=device, copy_blocks=copy_blocks, flag_sets=2, fuse_flags=fuse_flags,
-                      link_delay_us=link_delay_us, lead_copy_blocks=lead_copy_blocks, flag_write_values=flag_write_values)
+                      link_delay_us=link_delay_us, lead_copy_blocks=lead_copy_blocks, flag_write_values=flag_write_values,
+                      list_blocks=list_blocks)
     rows = M // WORLD
     for r in range(WORLD):     # every rank's symmetric buffer holds its own shard
         ctx.comm_buffers["a"][r][r * rows:(r + 1) * rows].copy_(a[r * rows:(r + 1) * rows])
@@ -797,6 +799,9 @@ def main():
                          "consumer's, by compute-unit masks")
     ap.add_argument("--lead-copy-blocks", type=int, default=LEAD_COPY_BLOCKS,
                     help="N > 0: a leading chunk copy and its flag write are one kernel of N workgroups")
+    ap.add_argument("--list-blocks", type=int, default=LIST_BLOCKS,
+                    help="N > 0: the producer is ONE kernel of N workgroups that walks the list of chunk copies and raises "
+                         "each chunk's flag (two kernels with --lead-ops: the leading chunks, then the rest)")
     ap.add_argument("--flag-write-values", action="store_true",
                     help="with --no-graph: flag writes are stream memory operations instead of one-wavefront kernels")
     ap.add_argument("--lead-on-compute-stream", action="store_true",
@@ -831,7 +836,8 @@ def main():
         sys.exit("--split-device splits the compute units between two streams: it needs the copy kernel "
                  "(--copy-blocks N) and launches from the host (--no-graph; a graph's kernel nodes carry no mask)")
     state = build_ag_gemm(device, args.copy_blocks, args.split_device, args.fuse_flags,
-                          lead_copy_blocks=args.lead_copy_blocks, flag_write_values=args.flag_write_values)
+                          lead_copy_blocks=args.lead_copy_blocks, flag_write_values=args.flag_write_values,
+                          list_blocks=args.list_blocks)
     with torch.cuda.stream(state["ctx"].compute_stream):
         wall_ms, gated_ms, no_lead_ms, resident_ms = run_ag_gemm(state, args.steps, args.warmup, args.resident_only,
                                                                  not args.no_graph)

@@ -325,6 +325,25 @@ int syn_copy_kernel_async(void* dst, const void* src, int64_t nbytes, int32_t nu
  * syn_copy_kernel_async. */
 int syn_copy_flag_async(void* dst, const void* src, int64_t nbytes, uint64_t* flag, uint64_t value,
                         uint32_t* ticket, int32_t num_blocks, syn_stream_t stream);
+/* A list of such copies as ONE kernel: record k is copied, then *flag = value, in list order, by at
+ * most `num_blocks` workgroups of 1024 threads that walk the list (a workgroup goes on to the next
+ * record while others still finish the last one).  `ops` is a DEVICE array of `count` records
+ * (every dst / src 16-byte aligned, `bytes16` = length in 16-byte units), `tickets` `count` zeroed
+ * 32-bit words of device memory, left zero again.  `delay_ticks` > 0 lets that many ticks of the
+ * device's wall clock (100 MHz) pass in front of a record: a slow link.  The data is stored through the L2, so no
+ * kernel boundary - with its cache write-back and invalidate - falls into a consumer kernel that
+ * runs beside the list.  Replaces a whole stream of cudaMemcpyAsync + cuStreamWriteValue pairs of the
+ * reference's executor (communication_context.py:129-150). */
+typedef struct syn_copy_flag_op {
+    void* dst;
+    const void* src;
+    int64_t bytes16;
+    uint64_t* flag;
+    uint64_t value;
+    int64_t delay_ticks;
+} syn_copy_flag_op;
+int syn_copy_flag_list_async(const syn_copy_flag_op* ops, int32_t count, uint32_t* tickets, int32_t num_blocks,
+                             syn_stream_t stream);
 /* What syn_box_copy_async does with the destination */
 #define SYN_BOX_COPY 0            /* dst = src */
 #define SYN_BOX_ADD_ATOMIC 1      /* dst += src by atomic adds: several senders may add into one

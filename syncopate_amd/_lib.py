@@ -164,6 +164,7 @@ _SIGNATURES = {
     "syn_copy_kernel_async": (c_int32, [c_void_p, c_void_p, c_int64, c_int32, c_void_p]),
     "syn_copy_flag_async": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p, ctypes.c_uint64, c_void_p, c_int32,
                                       c_void_p]),
+    "syn_copy_flag_list_async": (c_int32, [c_void_p, c_int32, c_void_p, c_int32, c_void_p]),
     "syn_box_copy_async": (c_int32, [c_void_p, c_void_p, c_int32, POINTER(c_int64), POINTER(c_int64),
                                      POINTER(c_int64), c_int32, c_int32, c_int32, c_void_p]),
     "syn_flag_set": (c_int32, [c_void_p, c_uint64, c_void_p]),

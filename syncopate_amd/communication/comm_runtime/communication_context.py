@@ -57,7 +57,7 @@ class CommContext:
                  device: Optional[torch.device] = None, link_delay_us: int = 0,
                  wait_timeout_us: int = 2_000_000, copy_blocks: int = 0, flag_sets: int = 1,
                  compute_stream: Optional[torch.cuda.Stream] = None, fuse_flags: bool = False,
-                 lead_copy_blocks: int = 0, flag_write_values: bool = False) -> None:
+                 lead_copy_blocks: int = 0, flag_write_values: bool = False, list_blocks: int = 0) -> None:
         if info.local_world_size <= 0:
             info.local_world_size = info.world_size
         if info.local_world_size != info.world_size:
@@ -86,6 +86,13 @@ class CommContext:
         self.lead_copy_blocks = int(lead_copy_blocks)
         # flag writes as stream memory operations instead of one-wavefront kernels (outside graph capture)
         self.flag_write_values = bool(flag_write_values)
+        # > 0: an op list that is nothing but (copy, flag write) pairs is issued by execute() as ONE kernel
+        # of that many workgroups which walks the list (two kernels with lead_ops: the leading pairs, with
+        # lead_copy_blocks workgroups if given, and the rest).  No kernel starts or ends on the device while
+        # the consumer runs, so nothing writes back or invalidates the L2s its operands are cached in.
+        self.list_blocks = int(list_blocks)
+        self._list_records: Dict[tuple, torch.Tensor] = {}
+        self._list_tickets: Dict[int, torch.Tensor] = {}
         self._lib = _lib.load()
         world = info.local_world_size
 
@@ -213,6 +220,8 @@ class CommContext:
         self._check_copy_units(self.info.operations[self.rank])
         for lane, (stream, ops) in enumerate(zip(self.streams, self.info.operations[self.rank])):
             lead = min(lead_ops, len(ops))
+            if self.list_blocks > 0 and self._issue_as_list(lane, stream, ops, lead, lead_on, neglect_local):
+                continue
             index = 0
             while index < len(ops):
                 op, done = ops[index], 1
@@ -236,6 +245,67 @@ class CommContext:
                         self._lead_events.append(event)
                 index += done
         self._zero_stale_set()
+
+    def _issue_as_list(self, lane: int, stream: torch.cuda.Stream, ops, lead: int,
+                       lead_on: Optional[torch.cuda.Stream], neglect_local: bool) -> bool:
+        """The whole op list as one kernel (two with leading ops); False if the list is not made of
+        (copy, flag write) pairs that the list kernel can take."""
+        world = self.info.local_world_size
+        if len(ops) == 0 or len(ops) % 2:
+            return False
+        key = (lane, self._cur_set, neglect_local)
+        records = self._list_records.get(key)
+        if records is None:
+            rows = []
+            for i in range(0, len(ops), 2):
+                op, flag_op = ops[i], ops[i + 1]
+                if not (isinstance(op, CopyEngineOp) and isinstance(flag_op, IntraNodeSignal)
+                        and flag_op.signal_type == SignalType.RECEIVE_DATA):
+                    return False
+                src = self.comm_buffers[op.src][op.src_rank % world]
+                dst = self.comm_buffers[op.dst][op.dst_rank % world]
+                if op.src_offset + op.size > src.numel() * src.element_size() or \
+                        op.dst_offset + op.size > dst.numel() * dst.element_size():
+                    raise ValueError(f"{op} runs past the end of its buffer")
+                dst_ptr, src_ptr = dst.data_ptr() + op.dst_offset, src.data_ptr() + op.src_offset
+                if op.size <= 0 or op.size % 16 or dst_ptr % 16 or src_ptr % 16:
+                    return False
+                flags = self.recv_signal_bufs[flag_op.rank % world]
+                if not 0 <= flag_op.offset < flags.numel():
+                    raise ValueError(f"{flag_op} is outside the flag array")
+                skip = op.src_rank == op.dst_rank and neglect_local
+                delay = self.link_delay_us * 100 if (self.link_delay_us and op.src_rank != op.dst_rank) else 0
+                rows.append([dst_ptr, src_ptr, 0 if skip else op.size // 16, flags.data_ptr() + 8 * flag_op.offset, 1, delay])
+            records = torch.tensor(rows, dtype=torch.int64, device=self.device)
+            self._list_records[key] = records
+        tickets = self._list_tickets.get(lane)
+        if tickets is None or tickets.numel() < records.shape[0]:
+            tickets = torch.zeros(records.shape[0], dtype=torch.int32, device=self.device)
+            self._list_tickets[lane] = tickets
+        lib = self._lib
+        count = records.shape[0]
+        lead_pairs = min(lead // 2, count)
+        if lead_pairs > 0:
+            on = lead_on if lead_on is not None else stream
+            blocks = self.lead_copy_blocks if self.lead_copy_blocks > 0 else self.list_blocks
+            _lib.check("syn_copy_flag_list_async",
+                       lib.syn_copy_flag_list_async(records.data_ptr(), lead_pairs, tickets.data_ptr(), blocks,
+                                                    int(on.cuda_stream)))
+            if lead_on is None:
+                event = torch.cuda.Event()
+                event.record(on)
+                self._lead_events.append(event)
+            # with lead_on the rest of the list does NOT wait for the leading chunks: both kernels start
+            # together, the leading one with many workgroups in front of the compute kernel, the other with
+            # few beside it.  Chunks then land in list order in practice (the leading kernel is an order of
+            # magnitude faster) but not by construction; every chunk has its own flag, so a consumer does
+            # not depend on the order.
+        if count > lead_pairs:
+            _lib.check("syn_copy_flag_list_async",
+                       lib.syn_copy_flag_list_async(records.data_ptr() + 48 * lead_pairs, count - lead_pairs,
+                                                    tickets.data_ptr() + 4 * lead_pairs, self.list_blocks,
+                                                    int(stream.cuda_stream)))
+        return True
 
     def wait_lead(self, stream: Optional[torch.cuda.Stream] = None) -> None:
         """`stream` continues once the leading ops of the last execute(lead_ops=...) are done."""

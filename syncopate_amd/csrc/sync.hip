@@ -81,6 +81,56 @@ copy_then_flag_kernel(uint64_t* __restrict__ dst, const u32x4_t* __restrict__ sr
     }
 }
 
+// A whole list of chunk copies, each followed by its flag, as ONE kernel: the workgroups walk the list
+// in order, copy their share of a chunk with stores that go through the L2 to memory, wait for the
+// stores' acknowledgements and take a ticket; the workgroup that takes a chunk's last ticket raises
+// the chunk's flag.  Seven chunks then cost one kernel instead of fourteen - and, more to the point,
+// no kernel boundary while the consumer runs: every kernel that starts or ends on the device brings
+// an invalidate or a write-back of the L2s the consumer's panels live in.
+struct CopyFlagOp {
+    u32x4_t* dst;
+    const u32x4_t* src;
+    int64_t vecs;
+    uint64_t* flag;
+    uint64_t value;
+    int64_t delay_ticks;        // wall-clock ticks to let pass before the chunk is copied (a slow link)
+};
+
+__device__ __forceinline__ void store16_through(u32x4_t* dst, u32x4_t v) {
+    // a store of more than 8 bytes reads its data registers for two more issue slots (hence the s_nop)
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(dst), "v"(v) : "memory");
+}
+
+__global__ void __launch_bounds__(kCopyFlagThreads)
+copy_flag_list_kernel(const CopyFlagOp* __restrict__ ops, int count, uint32_t* tickets) {
+    const int64_t stride = (int64_t)gridDim.x * kCopyFlagThreads;
+    for (int k = 0; k < count; ++k) {
+        const CopyFlagOp op = ops[k];
+        if (op.delay_ticks > 0) {
+            const uint64_t t0 = wall_clock64();
+            while ((int64_t)(wall_clock64() - t0) < op.delay_ticks) __builtin_amdgcn_s_sleep(32);
+        }
+        for (int64_t i = (int64_t)blockIdx.x * kCopyFlagThreads + threadIdx.x; i < op.vecs; i += 4 * stride) {
+            u32x4_t v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (i + u * stride < op.vecs) v[u] = __builtin_nontemporal_load(op.src + i + u * stride);
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (i + u * stride < op.vecs) store16_through(op.dst + i + u * stride, v[u]);
+        }
+        __builtin_amdgcn_s_waitcnt(0x0070);          // vmcnt(0): this lane's stores have reached memory
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            const uint32_t taken = __hip_atomic_fetch_add(tickets + k, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (taken == gridDim.x - 1) {
+                __hip_atomic_store(tickets + k, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(op.flag, op.value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            }
+        }
+    }
+}
+
 // Box copy: a box of up to 5 dimensions, contiguous along the last one in source and
 // destination, byte strides otherwise arbitrary; optionally dst += src by atomic adds, so that
 // several senders may accumulate into one destination at a time.  The box is a list of rows
@@ -346,6 +396,17 @@ int syn_copy_flag_async(void* dst, const void* src, int64_t nbytes, uint64_t* fl
     hipLaunchKernelGGL(syn::copy_then_flag_kernel, dim3(blocks), dim3(syn::kCopyFlagThreads), 0,
                        reinterpret_cast<hipStream_t>(stream), reinterpret_cast<uint64_t*>(dst),
                        reinterpret_cast<const syn::u32x4_t*>(src), vecs, ticket, flag, value);
+    return (int)hipGetLastError();
+}
+
+int syn_copy_flag_list_async(const syn_copy_flag_op* ops, int32_t count, uint32_t* tickets, int32_t num_blocks,
+                             syn_stream_t stream) {
+    static_assert(sizeof(syn_copy_flag_op) == sizeof(syn::CopyFlagOp), "the kernel's record is the header's");
+    if (!ops || !tickets || count <= 0 || count > 4096) return SYN_EINVAL;
+    if (num_blocks <= 0 || num_blocks > 4096) return SYN_EINVAL;
+    hipLaunchKernelGGL(syn::copy_flag_list_kernel, dim3(num_blocks), dim3(syn::kCopyFlagThreads), 0,
+                       reinterpret_cast<hipStream_t>(stream), reinterpret_cast<const syn::CopyFlagOp*>(ops), count,
+                       tickets);
     return (int)hipGetLastError();
 }
 

@@ -1001,12 +1001,14 @@ def test_all2all_then_split_k_gemm(hip, slices):
     assert ctx.recv_signal_bufs[rank].tolist() == [1] * len(shapes)
 
 
-@pytest.mark.parametrize("lead_on_compute_stream,lead_copy_blocks", [(False, 0), (True, 0), (True, 64), (False, 64)])
-def test_leading_ops_ahead_of_the_consumer(hip, lead_on_compute_stream, lead_copy_blocks):
+@pytest.mark.parametrize("lead_on_compute_stream,lead_copy_blocks,list_blocks",
+                         [(False, 0, 0), (True, 0, 0), (True, 64, 0), (False, 64, 0), (False, 0, 8), (True, 64, 8)])
+def test_leading_ops_ahead_of_the_consumer(hip, lead_on_compute_stream, lead_copy_blocks, list_blocks):
     """execute(lead_ops=4): the first two chunk copies and their flags are in place before the
     consumer is launched - through an event the compute stream waits for, or enqueued on the
     compute stream itself (lead_on), as two kernels each or as one copy-and-flag kernel each
-    (lead_copy_blocks).  Every form must gather the same bytes and give the resident result."""
+    (lead_copy_blocks), or the whole op list as one kernel that walks it (list_blocks; two kernels
+    with leading ops).  Every form must gather the same bytes and give the resident result."""
     from syncopate_amd.communication.comm_runtime.communication_context import CommContext
     from syncopate_amd.communication.common_descriptors import build_all_gather_plan_1d_swizzle
     from syncopate_amd.computation._launch import check_status
@@ -1019,7 +1021,7 @@ def test_leading_ops_ahead_of_the_consumer(hip, lead_on_compute_stream, lead_cop
              for r in range(world)}
     schedules, info = _compile(plans)
     tables = gemm_consumer_tables(schedules[rank]["a"], N)
-    ctx = CommContext(rank, info, lead_copy_blocks=lead_copy_blocks)
+    ctx = CommContext(rank, info, lead_copy_blocks=lead_copy_blocks, list_blocks=list_blocks)
     g = torch.Generator().manual_seed(21)
     a = (0.02 * torch.randn(M, K, generator=g)).bfloat16()
     b = (0.02 * torch.randn(N, K, generator=g)).bfloat16()
@@ -1044,3 +1046,9 @@ def test_leading_ops_ahead_of_the_consumer(hip, lead_on_compute_stream, lead_cop
         assert torch.equal(ctx.comm_buffers["a"][rank], ad)
         assert ctx.recv_signal_bufs[rank].tolist() == [1] * (world - 1)
         assert _rel(c, numerics.gemm_fp32(a, b)) <= REL_TOL
+        if list_blocks:
+            assert ctx._list_tickets[0].tolist() == [0] * (world - 1)      # every ticket word left zero again
+        # the peers' rows are stale again for the next iteration
+        for r in range(world):
+            if r != rank:
+                ctx.comm_buffers["a"][rank][r * rows:(r + 1) * rows].fill_(float("nan"))
