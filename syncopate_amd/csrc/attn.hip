@@ -475,16 +475,23 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
                                                 __HIP_MEMORY_SCOPE_AGENT) == 0;
         float w_old = 0.f, w_new = 1.f, lse_out = lse2;
         float* lse_ptr = p.lse + head * p.Sq + q_row;
+        T* o_row = O + z * p.o_st[0] + h * p.o_st[1] + q_row * p.o_st[2] + 4 * half;
+        // what is there already: every load issued before the first is used (the loads go past the L2:
+        // one after the other, each waited for, they would cost a trip to memory each)
+        vec4_t old[4][4];
         if (!is_first) {
-            // merge with the stored partial (template.py:335-349)
             const float m_old = load_f32_coherent(lse_ptr);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) old[i][g] = load8_coherent<vec4_t>(o_row + 32 * i + 8 * g);
+            // merge with the stored partial (template.py:335-349)
             const float delta = m_old - lse2;
             const float mmax = fmaxf(m_old, lse2);
             lse_out = mmax + fast_log2(1.0f + fast_exp2(-fabsf(delta)));
             w_old = fast_exp2(m_old - lse_out);
             w_new = fast_exp2(lse2 - lse_out);
         }
-        T* o_row = O + z * p.o_st[0] + h * p.o_st[1] + q_row * p.o_st[2] + 4 * half;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -494,9 +501,8 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
                 for (int c = 0; c < 4; ++c) x[c] = o_acc[i][4 * g + c] * inv_l * w_new;
                 T* dst = o_row + 32 * i + 8 * g;
                 if (!is_first) {
-                    const vec4_t old = load8_coherent<vec4_t>(dst);
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) x[c] += (float)old[c] * w_old;
+                    for (int c = 0; c < 4; ++c) x[c] += (float)old[i][g][c] * w_old;
                 }
                 vec4_t out;
 #pragma unroll
@@ -874,15 +880,20 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
         const bool is_first = __hip_atomic_load(p.first + lock_idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0;
         float w_old = 0.f, w_new = 1.f, lse_out = lse2;
         float* lse_ptr = p.lse + head * p.Sq + q_row;
+        T* o_row = O + z * p.o_st[0] + h * p.o_st[1] + q_row * p.o_st[2] + 4 * half;
+        vec4_t old[4][4];              // every load issued before the first is used: see attn_fwd_kernel
         if (!is_first) {
             const float m_old = load_f32_coherent(lse_ptr);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) old[i][g] = load8_coherent<vec4_t>(o_row + 32 * i + 8 * g);
             const float delta = m_old - lse2;
             const float mmax = fmaxf(m_old, lse2);
             lse_out = mmax + fast_log2(1.0f + fast_exp2(-fabsf(delta)));
             w_old = fast_exp2(m_old - lse_out);
             w_new = fast_exp2(lse2 - lse_out);
         }
-        T* o_row = O + z * p.o_st[0] + h * p.o_st[1] + q_row * p.o_st[2] + 4 * half;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -892,9 +903,8 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
                 for (int c = 0; c < 4; ++c) x[c] = o_acc[i][4 * g + c] * inv_l * w_new;
                 T* dst = o_row + 32 * i + 8 * g;
                 if (!is_first) {
-                    const vec4_t old = load8_coherent<vec4_t>(dst);
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) x[c] += (float)old[c] * w_old;
+                    for (int c = 0; c < 4; ++c) x[c] += (float)old[i][g][c] * w_old;
                 }
                 vec4_t out;
 #pragma unroll
