@@ -117,6 +117,80 @@ __device__ __forceinline__ void store_f32_through(float* ptr, float value) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
+// The merge of a wavefront's 32 q rows into the output: O = O_stored * w_old + O_new * w_new, rounded to
+// the output type (template.py:335-361), with lse beside it.  In the accumulator layout a lane owns
+// scattered 8-byte pieces of one row (4 columns out of every 32, one row 256 bytes from the next): stored
+// through the L2 like that, every piece travels to memory as a partial line, and the merge of one
+// tile took 20 us - as much with the locks already held and the stored result read from the L2 as
+// with the whole protocol, so it was the traffic and not the round trips.  Here the rows pass
+// through a tile in LDS that belongs to the
+// wavefront (the K and V blocks are free during the epilogue): memory is read and written in the
+// layout "instruction k: rows 2k and 2k + 1, lane l the 8 bytes at 8 * (l % 32) of row 2k + l / 32",
+// i.e. whole 256-byte rows, two full lines each.  Rows are 272 bytes apart in the tile so that the
+// accumulator layout's accesses (32 rows at one column) spread over the banks.
+constexpr int kStageRowBytes = 272;
+constexpr int kStageBytes = 32 * kStageRowBytes;       // per wavefront
+
+template <typename T>
+__device__ __forceinline__ void merge_rows_through_lds(unsigned char* stage, T* o_rows, const int64_t o_pitch,
+                                                       float* lse_rows, const f32x16_t (&o_acc)[4], const float inv_l,
+                                                       const float lse2, const bool is_first, const int lane) {
+    typedef T vec4_t __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) vec4_t* lds_vec4_ptr;
+    const int r = lane & 31, half = lane >> 5;
+    const lds_vec4_ptr tile = (lds_vec4_ptr)(__attribute__((address_space(3))) void*)stage;
+    // element offsets in units of 8 bytes
+    auto by_row_pair = [&](const int k) { return ((2 * k + half) * kStageRowBytes >> 3) + r; };
+    auto by_accumulator = [&](const int i, const int g) { return (r * kStageRowBytes >> 3) + 8 * i + 2 * g + half; };
+    T* const mine = o_rows + (int64_t)half * o_pitch + 4 * r;      // instruction k: + 2 * k * o_pitch
+
+    float w_old = 0.f, w_new = 1.f, lse_out = lse2;
+    vec4_t old[4][4];
+    if (!is_first) {
+        vec4_t in[16];
+        const float m_old = load_f32_coherent(lse_rows + r);
+#pragma unroll
+        for (int k = 0; k < 16; ++k) in[k] = load8_coherent<vec4_t>(mine + 2 * k * o_pitch);
+#pragma unroll
+        for (int k = 0; k < 16; ++k) tile[by_row_pair(k)] = in[k];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) old[i][g] = tile[by_accumulator(i, g)];
+        const float delta = m_old - lse2;
+        const float mmax = fmaxf(m_old, lse2);
+        lse_out = mmax + fast_log2(1.0f + fast_exp2(-fabsf(delta)));
+        w_old = fast_exp2(m_old - lse_out);
+        w_new = fast_exp2(lse2 - lse_out);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            float x[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) x[c] = o_acc[i][4 * g + c] * inv_l * w_new;
+            if (!is_first) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) x[c] += (float)old[i][g][c] * w_old;
+            }
+            vec4_t out;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) out[c] = (T)x[c];
+            tile[by_accumulator(i, g)] = out;
+        }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int k = 0; k < 16; ++k) store8_through(mine + 2 * k * o_pitch, (vec4_t)tile[by_row_pair(k)]);
+    if (half == 0) store_f32_through(lse_rows + r, lse_out);
+}
+
+
 typedef __attribute__((address_space(3))) void* lds_void_ptr;
 typedef const __attribute__((address_space(1))) void* global_void_ptr;
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
@@ -473,43 +547,10 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
 
         const bool is_first = __hip_atomic_load(p.first + lock_idx, __ATOMIC_RELAXED,
                                                 __HIP_MEMORY_SCOPE_AGENT) == 0;
-        float w_old = 0.f, w_new = 1.f, lse_out = lse2;
-        float* lse_ptr = p.lse + head * p.Sq + q_row;
-        T* o_row = O + z * p.o_st[0] + h * p.o_st[1] + q_row * p.o_st[2] + 4 * half;
-        // what is there already: every load issued before the first is used (the loads go past the L2:
-        // one after the other, each waited for, they would cost a trip to memory each)
-        vec4_t old[4][4];
-        if (!is_first) {
-            const float m_old = load_f32_coherent(lse_ptr);
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int g = 0; g < 4; ++g) old[i][g] = load8_coherent<vec4_t>(o_row + 32 * i + 8 * g);
-            // merge with the stored partial (template.py:335-349)
-            const float delta = m_old - lse2;
-            const float mmax = fmaxf(m_old, lse2);
-            lse_out = mmax + fast_log2(1.0f + fast_exp2(-fabsf(delta)));
-            w_old = fast_exp2(m_old - lse_out);
-            w_new = fast_exp2(lse2 - lse_out);
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                float x[4];
-#pragma unroll
-                for (int c = 0; c < 4; ++c) x[c] = o_acc[i][4 * g + c] * inv_l * w_new;
-                T* dst = o_row + 32 * i + 8 * g;
-                if (!is_first) {
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) x[c] += (float)old[i][g][c] * w_old;
-                }
-                vec4_t out;
-#pragma unroll
-                for (int c = 0; c < 4; ++c) out[c] = (T)x[c];
-                store8_through(dst, out);
-            }
-        if (half == 0) store_f32_through(lse_ptr, lse_out);
+        // (the K and V blocks are free: every wavefront is past its last block and the barrier above)
+        merge_rows_through_lds<T>(wave < 3 ? k_lds + wave * kStageBytes : v_lds,
+                                  O + z * p.o_st[0] + h * p.o_st[1] + (int64_t)(qb * kBlockM + wave * 32) * p.o_st[2], p.o_st[2],
+                                  p.lse + head * p.Sq + qb * kBlockM + wave * 32, o_acc, inv_l, lse2, is_first, lane);
 
         // every lane's stores have been acknowledged by memory; then the barrier; then the hand-over
         __builtin_amdgcn_s_waitcnt(attn_vmcnt(0));
@@ -878,40 +919,10 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
         if (s_abort) return;
 
         const bool is_first = __hip_atomic_load(p.first + lock_idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0;
-        float w_old = 0.f, w_new = 1.f, lse_out = lse2;
-        float* lse_ptr = p.lse + head * p.Sq + q_row;
-        T* o_row = O + z * p.o_st[0] + h * p.o_st[1] + q_row * p.o_st[2] + 4 * half;
-        vec4_t old[4][4];              // every load issued before the first is used: see attn_fwd_kernel
-        if (!is_first) {
-            const float m_old = load_f32_coherent(lse_ptr);
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int g = 0; g < 4; ++g) old[i][g] = load8_coherent<vec4_t>(o_row + 32 * i + 8 * g);
-            const float delta = m_old - lse2;
-            const float mmax = fmaxf(m_old, lse2);
-            lse_out = mmax + fast_log2(1.0f + fast_exp2(-fabsf(delta)));
-            w_old = fast_exp2(m_old - lse_out);
-            w_new = fast_exp2(lse2 - lse_out);
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                float x[4];
-#pragma unroll
-                for (int c = 0; c < 4; ++c) x[c] = o_acc[i][4 * g + c] * inv_l * w_new;
-                T* dst = o_row + 32 * i + 8 * g;
-                if (!is_first) {
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) x[c] += (float)old[i][g][c] * w_old;
-                }
-                vec4_t out;
-#pragma unroll
-                for (int c = 0; c < 4; ++c) out[c] = (T)x[c];
-                store8_through(dst, out);
-            }
-        if (half == 0) store_f32_through(lse_ptr, lse_out);
+        // (the K and V blocks are free: every wavefront has passed the last slot's barrier)
+        merge_rows_through_lds<T>(wave8 < 4 ? k_lds + wave8 * kStageBytes : v_lds + (wave8 - 4) * kStageBytes,
+                                  O + z * p.o_st[0] + h * p.o_st[1] + (int64_t)(qb * kBlockM + wave * 32) * p.o_st[2], p.o_st[2],
+                                  p.lse + head * p.Sq + qb * kBlockM + wave * 32, o_acc, inv_l, lse2, is_first, lane);
 
         // every lane's stores have been acknowledged by memory; then the barrier; then the hand-over
         __builtin_amdgcn_s_waitcnt(attn_vmcnt(0));
