@@ -534,7 +534,9 @@ def _gated_attention(q, staged_kv, buf, arrival, chunk, tables, launches, device
 def run_attention_ag(device, launches=5, gated=True):
     """All-gather attention at the headline ring / all-gather configuration: 4096 local q rows, 32 heads,
     against 32768 kv rows as 8 chunks of 4096 in double-ring arrival order, head dim 128; two q
-    blocks per workgroup in opposite phases (pair_q_blocks).  Resident (every flag set), and gated."""
+    blocks per workgroup in opposite phases (pair_q_blocks).  Resident (every flag set) in the chained form
+    and in the forms that merge after every tile, and gated (224 persistent programs that merge: the
+    stand-in producer's copy kernels need the other 32 compute units)."""
     from syncopate_amd.computation._launch import check_status
     from syncopate_amd.computation.attn import attention_forward
 
@@ -554,16 +556,20 @@ def run_attention_ag(device, launches=5, gated=True):
         return _timed(lambda i: attention_forward(q, kv[0], kv[1], D ** -0.5, out=out, pair_q_blocks=True,
                                                   signal_ptr=ones, **tables, **kw), launches, 3)
     resident()                      # clocks settle
-    # 256 persistent workgroups, each XCD's on consecutive tiles (the q blocks of two heads at a time, whose K
-    # and V then pass through that XCD's L2 only)
-    ms = resident(xcd_remap=True, num_programs=256)
+    # one program per pair of q blocks of a wave (512), each XCD's on consecutive pairs (the q blocks of two
+    # heads at a time, whose K and V then pass through that XCD's L2 only); a program walks through the
+    # eight chunks with its sums in registers and writes its q blocks once
+    ms = resident(xcd_remap=True, chain_q_blocks=True)
     check_status()
+    # the reference's protocol: 256 persistent workgroups, every tile merged into the output under its q block's lock
+    merged_ms = resident(xcd_remap=True, num_programs=256)
     plain_ms = resident()           # one workgroup per pair of q blocks, dealt round-robin over the XCDs
     persistent_ms = resident(num_programs=224)
     s = (q[0, 7].float() @ kv[0, 0, 7].float().t()) * D ** -0.5
     ref = torch.softmax(s, dim=-1) @ kv[1, 0, 7].float()
     err = ((out[0, 7].float() - ref).abs().max() / ref.abs().max()).item()
     result = {"launches": launches, "ms": ms, "flop": 4.0 * B * H * Sq * Skv * D, "max_rel_err_vs_fp32": err,
+              "form": "chain_q_blocks, 512 programs, xcd_remap", "ms_256_programs_merge_per_tile": merged_ms,
               "ms_224_programs_resident": persistent_ms, "ms_one_workgroup_per_pair_no_xcd_remap": plain_ms}
     if not gated:
         return result

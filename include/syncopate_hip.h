@@ -43,6 +43,8 @@ extern "C" {
 #define SYN_STATUS_SPIN_TIMEOUT 1   /* [1]=wave index, [2]=program id, [3]=signal offset */
 #define SYN_STATUS_BAD_PAIRING 2    /* SYN_ATTN_PAIR_Q_BLOCKS on a wave with an odd number of q blocks:
                                        [1]=wave index, [2]=program id, [3]=q blocks of the wave */
+#define SYN_STATUS_BAD_CHAIN 3      /* SYN_ATTN_CHAIN_Q_BLOCKS: [1]=wave whose (z, h, q) ranges differ from wave 0's, or 0
+                                       and [3]=pairs per wave when the grid is not that many programs */
 
 /* gemm option bits */
 #define SYN_GEMM_XCD_REMAP 1u       /* permute hardware workgroup ids so that consecutive
@@ -288,6 +290,15 @@ typedef struct syn_attn_desc {
  * then work on consecutive tiles - the q blocks of one head - and that head's K and V pass through
  * one L2 instead of eight.  The visit log records the program each tile ran on either way. */
 #define SYN_ATTN_XCD_REMAP 2u
+/* with SYN_ATTN_PAIR_Q_BLOCKS: the caller vouches that every wave lists the same (z, h, q) ranges
+ * (the waves differ in their kv range and flag only, as in the all-gather attention) and passes
+ * num_programs = the number of q block pairs of one wave.  Program b's tiles are then pair b of
+ * wave 0, of wave 1, ... in this order - the same programs and the same order as without the
+ * option - and the kernel walks on from one wave's kv range into the next one's behind that wave's
+ * flag, with the running maxima, sums and output in registers: every q block is written once, and
+ * neither `lock` nor a stored partial result is read.  A table or grid that is not of that shape
+ * ends the launch with SYN_STATUS_BAD_CHAIN in `status`.  No counterpart in the reference. */
+#define SYN_ATTN_CHAIN_Q_BLOCKS 4u
 int syn_attn_fwd(const syn_attn_desc* desc, syn_stream_t stream);
 
 /* Host-only check of an attention wave table (HOST pointers). */

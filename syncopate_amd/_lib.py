@@ -34,7 +34,9 @@ SYN_GEMM_NO_K_STAGGER = 8
 SYN_GEMM_TWO_STAGE = 16
 SYN_ATTN_PAIR_Q_BLOCKS = 1
 SYN_ATTN_XCD_REMAP = 2
+SYN_ATTN_CHAIN_Q_BLOCKS = 4
 SYN_STATUS_BAD_PAIRING = 2
+SYN_STATUS_BAD_CHAIN = 3
 SYN_BOX_COPY, SYN_BOX_ADD_ATOMIC, SYN_BOX_ADD_EXCLUSIVE = range(3)
 SYN_ELEM_BF16, SYN_ELEM_FP16, SYN_ELEM_FP32, SYN_ELEM_1B, SYN_ELEM_2B, SYN_ELEM_4B, SYN_ELEM_8B = range(7)
 

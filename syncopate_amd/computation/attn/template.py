@@ -44,6 +44,9 @@ BLOCK_N = 128
 DEFAULT_SPIN_TIMEOUT_US = 2_000_000
 
 
+_chain_programs: dict = {}      # ids of a caller's four tables -> pairs of q blocks per wave (chain_q_blocks)
+
+
 @launches_on_stream
 def attention_forward(
     q: torch.Tensor,
@@ -67,6 +70,7 @@ def attention_forward(
     consumer_signal_offsets: Optional[TableLike] = None,
     pair_q_blocks: bool = False,
     xcd_remap: bool = False,
+    chain_q_blocks: bool = False,
     out: Optional[torch.Tensor] = None,
     return_lse: bool = False,
     visit_log: Optional[torch.Tensor] = None,
@@ -94,6 +98,14 @@ def attention_forward(
     number of q blocks; not with `causal` or `counter_ptr`.
     `xcd_remap` (an extension): the workgroups of one XCD take consecutive tiles (the q blocks of
     one head), so that a head's K and V are fetched into one L2 instead of eight.
+    `chain_q_blocks` (an extension, with `pair_q_blocks`): for tables whose waves all list the same
+    (z, h, q) ranges and differ in the kv range and the flag only (the all-gather attention).  With
+    as many programs as a wave has pairs of q blocks - `num_programs` must be that number, or 0 to
+    have it filled in - a program's tiles are one pair of q blocks in wave after wave, so it keeps
+    the running maxima, sums and output in registers from one wave's kv range to the next (each
+    behind its flag) and writes every q block once, without locks or merges.  Programs, tiles and
+    their order are those of the persistent launch with that `num_programs`.  A ValueError for
+    tables of another shape.
     """
     dev = require_cuda(q, k, v, signal_ptr)
     if not (q.dtype == k.dtype == v.dtype):
@@ -133,20 +145,43 @@ def attention_forward(
                        for t in (wave_offsets, wave_sizes, cum_wave_sizes, signal_offsets))
     if pair_q_blocks and (causal or counter_ptr is not None):
         raise ValueError("pair_q_blocks goes with neither causal nor counter_ptr")
-    params = (num_waves, Z, H, Sq, Skv, cum_tiles, flags.numel(), bool(pair_q_blocks))
-    if cum_tiles is None or not (caller_owned and already_checked(tables, params)):
+    if chain_q_blocks and not pair_q_blocks:
+        raise ValueError("chain_q_blocks goes with pair_q_blocks")
+    num_programs = int(num_programs)
+    if chain_q_blocks and num_programs <= 0 and caller_owned:
+        # filled in by an earlier call on these tables; `already_checked` below vouches for it
+        num_programs = _chain_programs.get(tuple(id(t) for t in tables), 0)
+    params = (num_waves, Z, H, Sq, Skv, cum_tiles, flags.numel(), bool(pair_q_blocks),
+              num_programs if chain_q_blocks else None)
+    if cum_tiles is None or (chain_q_blocks and num_programs <= 0) or \
+            not (caller_owned and already_checked(tables, params)):
         ho, hs, hc, hg = host_copy(offs), host_copy(sizes), host_copy(cums), host_copy(sigs)
         if cum_tiles is None:
             cum_tiles = int(hc[:num_waves].max().item())
         if pair_q_blocks and any(int(hs[i, 2]) % (2 * BLOCK_M) for i in range(num_waves) if int(hc[i]) > 0):
             raise ValueError("pair_q_blocks needs an even number of q blocks in every wave")
+        if chain_q_blocks:
+            real = [i for i in range(num_waves) if int(hc[i]) > 0]
+            if not real or any(ho[i, :3].tolist() != ho[real[0], :3].tolist() or
+                               hs[i, :3].tolist() != hs[real[0], :3].tolist() for i in real):
+                raise ValueError("chain_q_blocks needs the same (z, h, q) ranges in every wave")
+            pairs = int(hs[real[0], 0]) * int(hs[real[0], 1]) * int(hs[real[0], 2]) // (2 * BLOCK_M)
+            if num_programs <= 0:
+                num_programs = pairs
+            elif num_programs != pairs:
+                raise ValueError(f"chain_q_blocks needs num_programs = {pairs}, the pairs of q blocks of one wave")
+            params = params[:-1] + (num_programs,)
+            if caller_owned:
+                if len(_chain_programs) > 1024:
+                    _chain_programs.clear()
+                _chain_programs[tuple(id(t) for t in tables)] = num_programs
         _lib.check(
             "syn_attn_check_waves",
             lib.syn_attn_check_waves(host_ptr(ho), host_ptr(hs), host_ptr(hc), host_ptr(hg), num_waves,
                                      Z, H, Sq, Skv, BLOCK_M, BLOCK_N, int(cum_tiles), flags.numel()),
         )
         if caller_owned:
-            remember_checked(tables, (num_waves, Z, H, Sq, Skv, cum_tiles, flags.numel(), bool(pair_q_blocks)))
+            remember_checked(tables, params[:5] + (cum_tiles,) + params[6:])
 
     if output_buffer is not None:
         if out is not None and out is not output_buffer:
@@ -192,7 +227,8 @@ def attention_forward(
         sm_scale=float(sm_scale), cum_tiles=int(cum_tiles), spin_timeout_us=int(spin_timeout_us),
         q_strides=strides(q), k_strides=strides(k), v_strides=strides(v), o_strides=strides(o),
         counters=None if counter_ptr is None else counter_ptr.data_ptr(),
-        options=(_lib.SYN_ATTN_PAIR_Q_BLOCKS if pair_q_blocks else 0) | (_lib.SYN_ATTN_XCD_REMAP if xcd_remap else 0),
+        options=(_lib.SYN_ATTN_PAIR_Q_BLOCKS if pair_q_blocks else 0) | (_lib.SYN_ATTN_XCD_REMAP if xcd_remap else 0)
+        | (_lib.SYN_ATTN_CHAIN_Q_BLOCKS if chain_q_blocks else 0),
         wait_flags=None if wait_flags is None else wait_flags.data_ptr(),
         wait_signal_offsets=None if wait_sigs is None else wait_sigs.data_ptr(),
     )

@@ -596,7 +596,13 @@ __device__ __forceinline__ void dma_kv_block8(unsigned char* lds, const unsigned
     }
 }
 
-template <typename T>
+//
+// kChain (SYN_ATTN_CHAIN_Q_BLOCKS): every wave lists the same (z, h, q) ranges and there are as many
+// programs as a wave has pairs, so program b's tiles are pair b of wave 0, of wave 1, ...: the
+// same two q blocks against one kv range after the other.  The walk over kv blocks then simply
+// continues into the next wave's range (after that wave's flag), the running maxima, sums and
+// output stay in registers, and the q blocks are written once, at the end, without locks.
+template <typename T, bool kChain>
 __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnParams p) {
     typedef typename AttnMfma<T>::frag_t frag_t;
     typedef T vec4_t __attribute__((ext_vector_type(4)));
@@ -640,7 +646,12 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
     const unsigned char* __restrict__ V = reinterpret_cast<const unsigned char*>(p.v);
     T* __restrict__ O = reinterpret_cast<T*>(p.o);
 
-    const int num_pairs = p.num_tiles / 2;
+    const int pairs_per_wave = p.cum_wave_sizes[0] / kBlockM / 2;
+    const int num_pairs = kChain ? pairs_per_wave : p.num_tiles / 2;
+    if (kChain && (int)gridDim.x != pairs_per_wave) {
+        if (tid == 0) report_status(p.status, SYN_STATUS_BAD_CHAIN, 0, (int)blockIdx.x, pairs_per_wave);
+        return;
+    }
     const int first_pair = logical_program_id((int)blockIdx.x, (int)gridDim.x, p.xcd_remap != 0);
     for (int pair = first_pair; pair < num_pairs; pair += gridDim.x) {
         // ---- tile id -> wave -> (z, h, q block, kv range); the two tiles of a pair differ in the q block only ----
@@ -701,6 +712,63 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
             const int b = m + rot;
             return b >= nkv ? b - nkv : b;
         };
+
+        // kChain: where the walk stands, for the K fills (one block ahead) and for the V fills: wave,
+        // kv blocks of it, next block, rotation and base address.  `total` counts the kv blocks of all waves.
+        int total = nkv;
+        int k_wave = 0, k_nkv = nkv, k_next = 1, k_rot = rot;
+        int v_wave = 0, v_nkv = nkv, v_next = 0, v_rot = rot;
+        const unsigned char* k_walk = k_base;
+        const unsigned char* v_walk = v_base;
+        if (kChain) {
+            for (int x = 1; x < p.num_waves && p.cum_wave_sizes[x] != 0; ++x) total += p.wave_sizes[x * 4 + 3] / kBlockN;
+        }
+        // the K fills enter the next wave: its tile is visited now - log, the (z, h, q) ranges promised to
+        // be wave 0's, its flag - and then its first K block may be asked for
+        auto enter_wave_k = [&]() -> bool {
+            ++k_wave;
+            bool same = true;
+#pragma unroll
+            for (int a = 0; a < 3; ++a)
+                same = same && p.wave_offsets[k_wave * 4 + a] == p.wave_offsets[a] && p.wave_sizes[k_wave * 4 + a] == p.wave_sizes[a];
+            if (!same) {
+                if (tid == 0) report_status(p.status, SYN_STATUS_BAD_CHAIN, k_wave, (int)blockIdx.x, -1);
+                return false;
+            }
+            k_nkv = p.wave_sizes[k_wave * 4 + 3] / kBlockN;
+            const int lo = p.wave_offsets[k_wave * 4 + 3] / kBlockN;
+            const int sg = p.signal_offsets[k_wave];
+            if (p.visit_log != nullptr && lane == 0 && wave == 0) {
+                int4* rec = reinterpret_cast<int4*>(p.visit_log) + 2 * ((size_t)tile_id + 2 * (size_t)k_wave * pairs_per_wave);
+                rec[0] = make_int4(k_wave, z, h, qb);
+                rec[1] = make_int4(lo, lo + k_nkv, sg, (int)blockIdx.x);
+            }
+            if (sg >= 0) {
+                if (tid == 0) {
+                    s_spun = __hip_atomic_load(p.flags + sg, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 1ull;
+                    if (s_spun && !spin_until_equal(p.flags + sg, 1ull, p.timeout_ticks)) {
+                        report_status(p.status, SYN_STATUS_SPIN_TIMEOUT, k_wave, (int)blockIdx.x, sg);
+                        s_abort = 1;
+                    }
+                }
+                __syncthreads();
+                if (s_spun) acquire_fence_agent();
+                if (s_abort) return false;
+                __syncthreads();       // s_spun may be written again only when everyone has read it
+            }
+            k_walk = K + (z * p.k_st[0] + h * p.k_st[1]) * (int64_t)sizeof(T) + (size_t)lo * kBlockN * k_pitch;
+            k_rot = p.xcd_remap ? (int)((unsigned)pair % (unsigned)k_nkv) : 0;
+            k_next = 0;
+            return true;
+        };
+        auto enter_wave_v = [&]() {
+            ++v_wave;
+            v_nkv = p.wave_sizes[v_wave * 4 + 3] / kBlockN;
+            v_walk = V + (z * p.v_st[0] + h * p.v_st[1]) * (int64_t)sizeof(T) +
+                     (size_t)(p.wave_offsets[v_wave * 4 + 3] / kBlockN) * kBlockN * v_pitch;
+            v_rot = p.xcd_remap ? (int)((unsigned)pair % (unsigned)v_nkv) : 0;
+            v_next = 0;
+        };
         // every wavefront has passed the barrier that ended the previous pair: all four buffers are free
         dma_kv_block8(k_lds, k_base + (size_t)blk(0) * kBlockN * k_pitch, k_pitch, k_fill_off, wave8);
 
@@ -726,14 +794,31 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
         // slot 2m + 2; their buffers were last read in slot 2m - 1.  (Spreading the fills between the
         // products or the exponentials, or leaving them all to the group that is in its softmax,
         // measured 1-6 % slower: a wavefront stalls at every fill wherever it is placed.)
-        auto fetch = [&](const int m) {
+        auto fetch = [&](const int m) -> bool {
             __builtin_amdgcn_sched_barrier(0);
-            dma_kv_block8(v_lds + (m & 1) * kBlockBytes, v_base + (size_t)blk(m) * kBlockN * v_pitch, v_pitch, v_fill_off,
-                          wave8);
-            if (m + 1 < nkv)
-                dma_kv_block8(k_lds + ((m + 1) & 1) * kBlockBytes, k_base + (size_t)blk(m + 1) * kBlockN * k_pitch,
-                              k_pitch, k_fill_off, wave8);
+            if constexpr (kChain) {
+                if (v_next == v_nkv) enter_wave_v();
+                int b = v_next + v_rot;
+                b = b >= v_nkv ? b - v_nkv : b;
+                dma_kv_block8(v_lds + (m & 1) * kBlockBytes, v_walk + (size_t)b * kBlockN * v_pitch, v_pitch, v_fill_off, wave8);
+                ++v_next;
+                if (m + 1 < total) {
+                    if (k_next == k_nkv && !enter_wave_k()) return false;
+                    b = k_next + k_rot;
+                    b = b >= k_nkv ? b - k_nkv : b;
+                    dma_kv_block8(k_lds + ((m + 1) & 1) * kBlockBytes, k_walk + (size_t)b * kBlockN * k_pitch, k_pitch, k_fill_off,
+                                  wave8);
+                    ++k_next;
+                }
+            } else {
+                dma_kv_block8(v_lds + (m & 1) * kBlockBytes, v_base + (size_t)blk(m) * kBlockN * v_pitch, v_pitch, v_fill_off,
+                              wave8);
+                if (m + 1 < nkv)
+                    dma_kv_block8(k_lds + ((m + 1) & 1) * kBlockBytes, k_base + (size_t)blk(m + 1) * kBlockN * k_pitch,
+                                  k_pitch, k_fill_off, wave8);
+            }
             __builtin_amdgcn_sched_barrier(0);
+            return true;
         };
 
         // S^T = K(n) . Q^T
@@ -857,30 +942,32 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
         // the two groups run the same phases one slot apart; written out per group so that the scores
         // (group 0) or the probabilities (group 1) are the only block-sized values that live across
         // an iteration
+        // (a fetch fails when a flag does not come within the time limit or, chained, when a wave's
+        // ranges are not wave 0's: every wavefront is told so at the same fetch, and the program ends)
         if (grp == 0) {
-            fetch(0);                                    // slot 0
+            if (!fetch(0)) return;                       // slot 0
             scores(0);
             end_even();
-            for (int n = 0; n + 1 < nkv; ++n) {
+            for (int n = 0; n + 1 < total; ++n) {
                 softmax();                               // slot 2n + 1
                 end_odd();
-                fetch(n + 1);                            // slot 2n + 2
+                if (!fetch(n + 1)) return;               // slot 2n + 2
                 weighted_values(n);
                 scores(n + 1);
                 end_even();
             }
             softmax();                                   // slot 2N - 1
             end_odd();
-            weighted_values(nkv - 1);                    // slot 2N
+            weighted_values(total - 1);                  // slot 2N
             end_even();
             end_odd();                                   // slot 2N + 1: group 1 finishes
         } else {
-            fetch(0);                                    // slot 0: group 0 starts
+            if (!fetch(0)) return;                       // slot 0: group 0 starts
             end_even();
             scores(0);                                   // slot 1
             end_odd();
-            for (int n = 0; n + 1 < nkv; ++n) {
-                fetch(n + 1);                            // slot 2n + 2
+            for (int n = 0; n + 1 < total; ++n) {
+                if (!fetch(n + 1)) return;               // slot 2n + 2
                 softmax();
                 end_even();
                 weighted_values(n);                      // slot 2n + 3
@@ -889,7 +976,7 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
             }
             softmax();                                   // slot 2N
             end_even();
-            weighted_values(nkv - 1);                    // slot 2N + 1
+            weighted_values(total - 1);                  // slot 2N + 1
             end_odd();
         }
 
@@ -898,6 +985,18 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
         const float lse2 = m_i + fast_log2(l_tot);
         const float inv_l = 1.0f / l_tot;
         const int lock_idx = (int)(head * (p.Sq / kBlockM)) + qb;
+        if constexpr (kChain) {
+            // the only visit that writes these q blocks: nothing to merge with and nobody to exclude
+            merge_rows_through_lds<T>(wave8 < 4 ? k_lds + wave8 * kStageBytes : v_lds + (wave8 - 4) * kStageBytes,
+                                      O + z * p.o_st[0] + h * p.o_st[1] + (int64_t)(qb * kBlockM + wave * 32) * p.o_st[2], p.o_st[2],
+                                      p.lse + head * p.Sq + qb * kBlockM + wave * 32, o_acc, inv_l, lse2, true, lane);
+            __syncthreads();       // the tiles in LDS are free for the next pair's fills
+            if (tid == 0) {
+                __hip_atomic_store(p.first + lock_idx, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(p.first + lock_idx + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            continue;
+        }
         if (tid == 0) {
             // one thread takes both locks, lower q block first: every workgroup that wants this
             // pair of q blocks takes them in the same order
@@ -939,8 +1038,11 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
 }
 
 template <typename T>
-static int launch_attn_pairs(const AttnParams& p, int grid, hipStream_t stream) {
-    hipLaunchKernelGGL((attn_pair_kernel<T>), dim3(grid), dim3(kPairThreads), 0, stream, p);
+static int launch_attn_pairs(const AttnParams& p, int grid, bool chain, hipStream_t stream) {
+    if (chain)
+        hipLaunchKernelGGL((attn_pair_kernel<T, true>), dim3(grid), dim3(kPairThreads), 0, stream, p);
+    else
+        hipLaunchKernelGGL((attn_pair_kernel<T, false>), dim3(grid), dim3(kPairThreads), 0, stream, p);
     return (int)hipGetLastError();
 }
 
@@ -1056,11 +1158,14 @@ int syn_attn_fwd(const syn_attn_desc* d, syn_stream_t stream) {
     if (d->options & SYN_ATTN_PAIR_Q_BLOCKS) {
         // two q blocks per workgroup: the caller vouches for an even number of q blocks in every wave
         if (d->causal || d->counters || d->wait_flags || d->wait_signal_offsets || tiles % 2) return SYN_EINVAL;
+        const bool chain = (d->options & SYN_ATTN_CHAIN_Q_BLOCKS) != 0;
+        if (chain && d->num_programs <= 0) return SYN_EINVAL;
         int grid = d->num_programs > 0 ? d->num_programs : (int)(tiles / 2);
         if (grid > tiles / 2) grid = (int)(tiles / 2);
-        return d->dtype == SYN_DTYPE_BF16 ? launch_attn_pairs<__bf16>(p, grid, s)
-                                          : launch_attn_pairs<_Float16>(p, grid, s);
+        return d->dtype == SYN_DTYPE_BF16 ? launch_attn_pairs<__bf16>(p, grid, chain, s)
+                                          : launch_attn_pairs<_Float16>(p, grid, chain, s);
     }
+    if (d->options & SYN_ATTN_CHAIN_Q_BLOCKS) return SYN_EINVAL;
     int grid = d->num_programs > 0 ? d->num_programs : (int)tiles;
     if (grid > tiles) grid = (int)tiles;
     return d->dtype == SYN_DTYPE_BF16 ? launch_attn<__bf16>(p, grid, s)

@@ -194,6 +194,81 @@ def test_paired_q_blocks_match_sdpa_and_oracle(hip, dtype, num_programs, xcd_rem
         assert sorted(first) == list(range(grid)) and sorted(first.values()) == list(range(grid))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("num_programs,xcd_remap", [(0, False), (12, False), (0, True)])
+def test_chained_q_blocks_match_sdpa_and_oracle(hip, dtype, num_programs, xcd_remap):
+    """Waves that differ in the kv range only, as many programs as a wave has pairs of q blocks: a program
+    walks from one wave's kv range into the next with the sums in registers and writes its q blocks
+    once.  Same tiles on the same programs as the persistent launch of that size (an extension: the
+    reference merges under the q block's lock after every tile)."""
+    from syncopate_amd.computation.attn import attention_forward
+    from syncopate_amd.computation._launch import check_status
+
+    Z, H, Sq, Skv = 2, 3, 512, 1024
+    q, k, v = _qkv(Z, H, Sq, Skv, dtype, seed=6)
+    chunks = [(512, 640), (0, 384), (768, 1024), (384, 512), (640, 768)]     # arrival order, ragged
+    offsets, sizes, cums, signals, total = _kv_waves(Z, H, Sq, chunks, [-1, 0, 1, 2, 1])
+    flags = torch.ones(3, dtype=torch.int64, device="cuda")
+    sm_scale = 128 ** -0.5
+    tiles = total // 128
+    pairs_per_wave = Z * H * Sq // 256
+    log = torch.full((tiles, 8), -1, dtype=torch.int32, device="cuda")
+    o = torch.full((Z, H, Sq, 128), float("nan"), dtype=dtype, device="cuda")
+    _, lse = attention_forward(q.cuda(), k.cuda(), v.cuda(), sm_scale, wave_offsets=offsets,
+                               wave_sizes=sizes, cum_wave_sizes=cums, signal_ptr=flags,
+                               signal_offsets=signals, NUM_WAVES=len(chunks), cum_tiles=total,
+                               num_programs=num_programs, return_lse=True, visit_log=log, out=o,
+                               pair_q_blocks=True, chain_q_blocks=True, xcd_remap=xcd_remap)
+    check_status()
+    assert _rel(o, numerics.sdpa_fp32(q, k, v, sm_scale)) <= REL_TOL
+    want_o, want_lse = numerics.chunked_attention(q, k, v, sm_scale, chunks)
+    assert _rel(o, want_o.float()) <= REL_TOL
+    assert (lse.cpu() - want_lse).abs().max().item() <= 2e-2
+
+    got = log.cpu().tolist()
+    for tile_id, rec in enumerate(got):
+        exp = visit_order.attn_tile_work(tile_id, offsets, sizes, cums, signals)
+        assert rec[:7] == [exp["wave"], exp["z"], exp["h"], exp["q_block"], exp["kv_lo"], exp["kv_hi"], exp["signal"]]
+        assert rec[7] == got[tile_id ^ 1][7]
+    programs = [rec[7] for rec in got[0::2]]
+    if not xcd_remap:
+        # tile t of a persistent launch of that many programs runs on program t % programs
+        assert programs == [pair % pairs_per_wave for pair in range(tiles // 2)]
+    else:
+        assert sorted(programs[:pairs_per_wave]) == list(range(pairs_per_wave))
+        assert programs == programs[:pairs_per_wave] * len(chunks)
+
+
+def test_chained_q_blocks_argument_errors_and_timeout(hip):
+    from syncopate_amd.computation.attn import attention_forward
+    from syncopate_amd.computation._launch import FlagWaitTimeout, check_status
+
+    Z, H, Sq, Skv = 1, 2, 256, 512
+    q, k, v = (t.cuda() for t in _qkv(Z, H, Sq, Skv, torch.bfloat16))
+    flags = torch.ones(2, dtype=torch.int64, device="cuda")
+    offsets, sizes, cums, signals, total = _kv_waves(Z, H, Sq, [(0, 256), (256, 512)], [-1, 0])
+    kw = dict(wave_sizes=sizes, cum_wave_sizes=cums, signal_ptr=flags, signal_offsets=signals, cum_tiles=total)
+    with pytest.raises(ValueError, match="pair_q_blocks"):
+        attention_forward(q, k, v, 0.1, wave_offsets=offsets, chain_q_blocks=True, **kw)
+    with pytest.raises(ValueError, match="num_programs = 2"):
+        attention_forward(q, k, v, 0.1, wave_offsets=offsets, pair_q_blocks=True, chain_q_blocks=True, num_programs=1, **kw)
+    # a wave over other heads than wave 0's
+    shifted = [offsets[0], [0, 1, 0, 256]]
+    narrow = [[Z, 1, Sq, 256], [Z, 1, Sq, 256]]
+    with pytest.raises(ValueError, match="same"):
+        attention_forward(q, k, v, 0.1, wave_offsets=shifted, wave_sizes=narrow, cum_wave_sizes=[Sq, 2 * Sq],
+                          signal_ptr=flags, signal_offsets=signals, cum_tiles=2 * Sq, pair_q_blocks=True,
+                          chain_q_blocks=True)
+
+    # the second wave's flag never comes: every wavefront leaves at that fetch, and the launch says so
+    flags.zero_()
+    attention_forward(q, k, v, 0.1, wave_offsets=offsets, pair_q_blocks=True, chain_q_blocks=True,
+                      spin_timeout_us=20_000, **kw)
+    with pytest.raises(FlagWaitTimeout):
+        check_status()
+    check_status()
+
+
 def test_paired_q_blocks_argument_errors(hip):
     from syncopate_amd.computation.attn import attention_forward
 

@@ -184,11 +184,15 @@ def test_allgather_gemm_reduce_scatter_in_one_kernel(hip, rank):
             assert torch.equal(scatter.comm_buffers["dst"][peer][rank], src[peer * rows:(peer + 1) * rows])
 
 
-@pytest.mark.parametrize("rank,layout", [(1, "bhsd"), (3, "bhsd"), (2, "bshd")])
-def test_allgather_attention_iteration(hip, rank, layout):
+@pytest.mark.parametrize("rank,layout,form", [(1, "bhsd", {}), (3, "bhsd", {}), (2, "bshd", {}),
+                                              (1, "bhsd", dict(pair_q_blocks=True, chain_q_blocks=True)),
+                                              (2, "bshd", dict(pair_q_blocks=True, chain_q_blocks=True, xcd_remap=True))],
+                         ids=lambda x: "+".join(x) if isinstance(x, dict) else str(x))
+def test_allgather_attention_iteration(hip, rank, layout, form):
     """K/V chunks pulled from their owners on a side stream (copy, then flag) while the
     attention kernel walks the waves of the lowered schedule; the local Q attends to the whole
-    sequence."""
+    sequence.  Also in the chained form, where a program goes from one chunk to the next behind its flag
+    without writing its q blocks in between."""
     from syncopate_amd.communication.comm_runtime.communication_context import CommContext
     from syncopate_amd.communication.common_descriptors import build_all_gather_plan_1d_swizzle
     from syncopate_amd.computation._launch import check_status
@@ -226,7 +230,7 @@ def test_allgather_attention_iteration(hip, rank, layout):
                             wave_sizes=tables.wave_sizes, cum_wave_sizes=tables.cum_wave_sizes,
                             signal_ptr=ctx.recv_signal_bufs[rank], signal_offsets=tables.signal_offsets,
                             NUM_WAVES=len(tables.signal_offsets), cum_tiles=tables.cum_tiles, visit_log=log,
-                            layout=layout)
+                            layout=layout, **form)
     ctx.end_before(main)
     check_status()
     ctx.check_status()
