@@ -448,18 +448,22 @@ def run_gemm_rs(device, steps, warmup, gated=True):
     counters = torch.zeros(world, dtype=torch.int32, device=device)
     main = torch.cuda.current_stream()
 
-    def producer(flags, programs=256):
+    def producer(flags, programs=256, xcd_remap=True):
         counters.zero_()
-        # 1024 tiles of 256 x 256: four full rounds of 256 programs
+        # 1024 tiles of 256 x 256: four full rounds of 256 programs.  With the remap an XCD's 32 tiles of a
+        # round are 4 x 8 neighbours (12 panels of A and B through its L2 instead of 18).
         gemm_producer(a, b, src, flags, sizes, offsets, signals, programs, 256, 256, BK, GROUP_M,
-                      cum_tiles=tables.cum_tiles, counter_buffer=counters, xcd_remap=False, eight_waves=EIGHT_WAVES)
+                      cum_tiles=tables.cum_tiles, counter_buffer=counters, xcd_remap=xcd_remap, eight_waves=EIGHT_WAVES)
 
     alone_flags = torch.zeros(world, dtype=torch.int64, device=device)
+    _timed(lambda i: producer(alone_flags), max(3, steps // 4), warmup)        # clocks settle
     producer_ms = _timed(lambda i: producer(alone_flags), steps, warmup)
     assert alone_flags.tolist() == [1] * world
+    no_remap_ms = _timed(lambda i: producer(alone_flags, xcd_remap=False), steps, warmup)
 
     if not gated:
-        return {"launches": steps, "producer_ms": producer_ms, "flop": 2.0 * m * n * k}
+        return {"launches": steps, "producer_ms": producer_ms, "producer_ms_without_xcd_remap": no_remap_ms,
+                "flop": 2.0 * m * n * k}
 
     def fused(programs):
         ctx.reset_signals()
@@ -482,7 +486,8 @@ def run_gemm_rs(device, steps, warmup, gated=True):
         acc = acc + dst[(RANK + i) % world][sample]
     reduce_matches = torch.equal(out[sample], acc)
     pushed = all(torch.equal(ctx.comm_buffers["dst"][p][RANK], src[p * rows:(p + 1) * rows]) for p in (1, 4, 7))
-    return {"launches": steps, "producer_ms": producer_ms, "flop": 2.0 * m * n * k, "fused_step_ms": fused_ms,
+    return {"launches": steps, "producer_ms": producer_ms, "producer_ms_without_xcd_remap": no_remap_ms,
+            "flop": 2.0 * m * n * k, "fused_step_ms": fused_ms,
             "fused_step_ms_by_programs": {str(k_): v for k_, v in fused_by_programs.items()},
             "reduce_matches": bool(reduce_matches), "pushed_chunks_match": bool(pushed)}
 
@@ -945,6 +950,8 @@ def main():
             "producer_tflops": rs["flop"] / (rs["producer_ms"] * 1e-3) / 1e12,
             "producer_pct_bf16_mfma_peak": 100.0 * rs["flop"] / (rs["producer_ms"] * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
             "producer_ms": rs["producer_ms"],
+            "producer_form": "256 programs, xcd_remap",
+            "producer_ms_without_xcd_remap": rs["producer_ms_without_xcd_remap"],
         }
         if gated:
             line["gemm_rs"].update({
