@@ -374,7 +374,7 @@ def run_reduce(device, steps, warmup):
     """GEMM+RS chunked reduce of the headline GEMM+RS configuration: 8 x (1024, 8192) bf16 -> (1024, 8192).
     Launches rotate over three sets of operands (3 x 151 MB, more than the 256 MB of memory-side
     cache) so that every launch streams from HBM; the batch is timed as a whole."""
-    from syncopate_amd.computation.reduce import ring_reduce
+    from syncopate_amd.computation.reduce import padded_receive_buffer, ring_reduce
 
     world, rows, n, sets = 8, 1024, 8192, 3
     torch.manual_seed(1)
@@ -383,7 +383,42 @@ def run_reduce(device, steps, warmup):
     out = [torch.empty(rows, n, dtype=torch.bfloat16, device=device) for _ in range(sets)]
     ms = _timed(lambda i: ring_reduce(recv[i % sets], out[i % sets], local[i % sets], RANK), steps, max(warmup, sets))
     nbytes = (world + 1) * rows * n * 2          # 8 reads + 1 write of a (1024, 8192) bf16 block
-    return ms, nbytes
+    # the same with the eight received blocks 16 MiB + 4 KiB apart (a caller's own receive buffer; the executor's
+    # symmetric buffers keep the reference's contiguous layout, whose byte offsets the op lists carry)
+    padded = [padded_receive_buffer(world, rows, n, torch.bfloat16, device) for _ in range(sets)]
+    for dst, src in zip(padded, recv):
+        dst.copy_(src)
+    padded_ms = _timed(lambda i: ring_reduce(padded[i % sets], out[i % sets], local[i % sets], RANK), steps, max(warmup, sets))
+    return ms, nbytes, padded_ms
+
+
+def run_hbm_read_ceiling(device, launches=30):
+    """What the memory system gives the reduce's READS (`syn_probe_read_streams`: the reduce's loop with an
+    exclusive-or in place of the adds and no result stream, 512 workgroups like the reduce): one linear
+    stream; eight streams 16 MiB apart, which is where the reference's layout [W, rows, N] puts the
+    eight partial blocks of (1024, 8192) bf16; and the same eight streams 16 MiB + 4 KiB apart.  Launches
+    rotate over three regions (3 x 134 MB, more than the memory-side cache)."""
+    from syncopate_amd import _lib
+
+    lib = _lib.load()
+    stream_bytes, sets, blocks = 16 << 20, 3, 512
+    span = 8 * (stream_bytes + 4096)
+    torch.manual_seed(5)
+    pool = torch.randint(0, 2 ** 31 - 1, (sets * span // 4,), dtype=torch.int32, device=device)
+    sink = torch.zeros(4 * blocks, dtype=torch.int32, device=device)
+
+    def probe(region, nbytes, stride, streams):
+        _lib.check("syn_probe_read_streams", lib.syn_probe_read_streams(pool.data_ptr() + region * span, nbytes, stride,
+                                                                         streams, blocks, sink.data_ptr(),
+                                                                         _lib.stream_handle(None)))
+
+    forms = {"one_stream_128MiB": (8 * stream_bytes, 0, 1), "eight_streams_16MiB_apart": (stream_bytes, stream_bytes, 8),
+             "eight_streams_16MiB_plus_4KiB_apart": (stream_bytes, stream_bytes + 4096, 8)}
+    result = {"launches": launches, "bytes_read_per_launch": 8 * stream_bytes}
+    for name, (nbytes, stride, streams) in forms.items():
+        ms = _timed(lambda i: probe(i % sets, nbytes, stride, streams), launches, sets)
+        result[name + "_GBps"] = 8 * stream_bytes / (ms * 1e-3) / 1e9
+    return result
 
 
 def run_box_copies(device, steps, warmup):
@@ -931,13 +966,19 @@ def main():
     if "throttled" in only and gated:
         line["throttled_producer"] = run_throttled(device, 20)
     if "reduce" in only:
-        reduce_ms, reduce_bytes = run_reduce(device, max(args.steps, 30), args.warmup)
+        reduce_ms, reduce_bytes, reduce_padded_ms = run_reduce(device, max(args.steps, 30), args.warmup)
         line.update({
             "rs_reduce_launches": max(args.steps, 30),
             "rs_reduce_GBps": reduce_bytes / (reduce_ms * 1e-3) / 1e9,
             "rs_reduce_us": reduce_ms * 1e3,
             "rs_reduce_pct_hbm_peak": 100.0 * reduce_bytes / (reduce_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "rs_reduce_received_blocks_4KiB_further_apart_GBps": reduce_bytes / (reduce_padded_ms * 1e-3) / 1e9,
         })
+        ceiling_reads = run_hbm_read_ceiling(device)
+        line["hbm_read_ceiling"] = ceiling_reads
+        # the reduce moves its bytes (8/9 of them reads at that placement, 1/9 writes) at this fraction of the
+        # rate at which the same reads alone can be had
+        line["rs_reduce_over_eight_stream_read_ceiling"] = line["rs_reduce_GBps"] / ceiling_reads["eight_streams_16MiB_apart_GBps"]
     if "box_copies" in only:
         boxes = run_box_copies(device, steps_small, args.warmup)
         line["box_copy_launches"] = steps_small

@@ -214,6 +214,14 @@ int syn_gemm_grid(int64_t cum_tiles, int32_t M, int32_t N, int32_t block_m,
 int syn_ring_reduce(const void* recv, const void* local, void* out,
                     int32_t world, int32_t rank, int64_t rows_per_rank, int64_t N,
                     int32_t dtype, int32_t acc_mode, syn_stream_t stream);
+/* The same with the W blocks of recv `recv_block_stride` elements apart (>= Mr*N, a multiple of 8)
+ * instead of back to back: what a [W, Mr, N] view of a padded receive buffer hands over
+ * (torch's input.stride(0) in ring_reduce_tma's call, tests/test_gemm_rs.py:75-121).  Eight
+ * blocks of exactly 16 MiB start in the same DRAM banks and channels; 4 KiB of padding per block
+ * is worth 8 % of read bandwidth. */
+int syn_ring_reduce_strided(const void* recv, int64_t recv_block_stride, const void* local, void* out,
+                            int32_t world, int32_t rank, int64_t rows_per_rank, int64_t N,
+                            int32_t dtype, int32_t acc_mode, syn_stream_t stream);
 
 /*
  * Chunked-KV flash attention forward.  One workgroup per tile id; tile id ->
@@ -407,6 +415,15 @@ int syn_where_async(uint32_t* out, int32_t workgroups, int32_t dwell, syn_stream
  * pipes sustain under the board's power limit when operand bits toggle. */
 int syn_probe_mfma_rate(float* sink, int32_t workgroups, int32_t iters, int32_t pattern,
                         syn_stream_t stream);
+
+/* Measurement aid, no counterpart in the reference: `workgroups` workgroups of 256 lanes read
+ * `streams` (1 or 8) streams of `stream_bytes` each (a multiple of 16384), `stride_bytes` apart
+ * from `base`, in the chunked reduce's access pattern (four 16-byte groups per lane and pass, every
+ * load of a pass issued before the first is used, non-temporal) and write nothing.
+ * bytes read = streams * stream_bytes.  sink: device memory of 16 bytes per workgroup.  The rate is
+ * what the memory system gives the reduce's reads at that placement of its operands. */
+int syn_probe_read_streams(const void* base, int64_t stream_bytes, int64_t stride_bytes, int32_t streams,
+                           int32_t workgroups, void* sink, syn_stream_t stream);
 
 /* Library/ABI version: major*10000 + minor*100 + patch. */
 int syn_version(void);

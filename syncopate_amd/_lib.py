@@ -156,6 +156,10 @@ _SIGNATURES = {
         c_int32,
         [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int64, c_int64, c_int32, c_int32, c_void_p],
     ),
+    "syn_ring_reduce_strided": (
+        c_int32,
+        [c_void_p, c_int64, c_void_p, c_void_p, c_int32, c_int32, c_int64, c_int64, c_int32, c_int32, c_void_p],
+    ),
     "syn_attn_fwd": (c_int32, [POINTER(AttnDesc), c_void_p]),
     "syn_attn_check_waves": (
         c_int32,
@@ -177,6 +181,7 @@ _SIGNATURES = {
     "syn_stream_destroy": (c_int32, [c_void_p]),
     "syn_where_async": (c_int32, [c_void_p, c_int32, c_int32, c_void_p]),
     "syn_probe_mfma_rate": (c_int32, [c_void_p, c_int32, c_int32, c_int32, c_void_p]),
+    "syn_probe_read_streams": (c_int32, [c_void_p, ctypes.c_int64, ctypes.c_int64, c_int32, c_int32, c_void_p, c_void_p]),
     "syn_version": (c_int32, []),
 }
 

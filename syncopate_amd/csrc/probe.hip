@@ -12,6 +12,8 @@
 
 namespace syn {
 
+typedef unsigned int u32x4_probe_t __attribute__((ext_vector_type(4)));
+
 constexpr int kProbeSets = 4;
 
 __device__ __forceinline__ unsigned probe_hash(unsigned x) {
@@ -74,7 +76,55 @@ __global__ void __launch_bounds__(256) mfma_rate_kernel(float* sink, int iters, 
     sink[me] = total;
 }
 
+// HBM read ceiling probe: `STREAMS` read streams `stride_vecs` 16-byte groups apart, walked in the chunked
+// reduce's access pattern - 256 lanes, four groups per lane and pass, every load of a pass issued
+// before the first is used, non-temporal - with an exclusive-or in place of the adds and no result
+// stream.  What it sustains is what the memory system gives that pattern of reads.
+constexpr int kStreamThreads = 256;
+constexpr int kStreamVecs = 4;
+
+template <int STREAMS>
+__global__ void __launch_bounds__(kStreamThreads)
+read_streams_kernel(const u32x4_probe_t* __restrict__ base, int64_t stride_vecs, int64_t stream_vecs,
+                    u32x4_probe_t* __restrict__ sink) {
+    constexpr int64_t kGroup = (int64_t)kStreamThreads * kStreamVecs;
+    u32x4_probe_t mix = {0u, 0u, 0u, 0u};
+    for (int64_t g0 = (int64_t)blockIdx.x * kGroup; g0 + kGroup <= stream_vecs; g0 += (int64_t)gridDim.x * kGroup) {
+        u32x4_probe_t parts[kStreamVecs][STREAMS];
+#pragma unroll
+        for (int u = 0; u < kStreamVecs; ++u)
+#pragma unroll
+            for (int i = 0; i < STREAMS; ++i)
+                parts[u][i] = __builtin_nontemporal_load(base + (int64_t)i * stride_vecs + g0 + threadIdx.x + u * kStreamThreads);
+#pragma unroll
+        for (int u = 0; u < kStreamVecs; ++u)
+#pragma unroll
+            for (int i = 0; i < STREAMS; ++i) mix ^= parts[u][i];
+    }
+    // keeps the loads alive; a lane whose words happen to cancel leaves its note in the sink
+    if ((mix.x ^ mix.y ^ mix.z ^ mix.w) == 0x9e3779b9u) sink[blockIdx.x] = mix;
+}
+
 }  // namespace syn
+
+extern "C" int syn_probe_read_streams(const void* base, int64_t stream_bytes, int64_t stride_bytes, int32_t streams,
+                                      int32_t workgroups, void* sink, syn_stream_t stream) {
+    using namespace syn;
+    if (base == nullptr || sink == nullptr || workgroups <= 0) return SYN_EINVAL;
+    if (stream_bytes <= 0 || stream_bytes % (16 * kStreamThreads * kStreamVecs)) return SYN_EINVAL;
+    if (streams != 1 && streams != 8) return SYN_EINVAL;
+    if (stride_bytes < 0 || stride_bytes % 16 || !aligned16(base) || !aligned16(sink)) return SYN_EALIGN;
+    const u32x4_probe_t* b = reinterpret_cast<const u32x4_probe_t*>(base);
+    u32x4_probe_t* k = reinterpret_cast<u32x4_probe_t*>(sink);
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (streams == 1)
+        hipLaunchKernelGGL(read_streams_kernel<1>, dim3(workgroups), dim3(kStreamThreads), 0, s, b, stride_bytes / 16,
+                           stream_bytes / 16, k);
+    else
+        hipLaunchKernelGGL(read_streams_kernel<8>, dim3(workgroups), dim3(kStreamThreads), 0, s, b, stride_bytes / 16,
+                           stream_bytes / 16, k);
+    return (int)hipGetLastError();
+}
 
 extern "C" int syn_probe_mfma_rate(float* sink, int32_t workgroups, int32_t iters, int32_t pattern,
                                    syn_stream_t stream) {

@@ -46,7 +46,7 @@ constexpr int kVecsPerThread = 4;      // 16-byte groups per lane and pass: 4 x 
 template <typename T, bool ROUND_EACH, int W>
 __global__ void __launch_bounds__(kReduceThreads)
 ring_reduce_kernel(const u32x4_t* __restrict__ recv, const u32x4_t* __restrict__ local,
-                   u32x4_t* __restrict__ out, int world, int rank, int64_t chunk_vecs) {
+                   u32x4_t* __restrict__ out, int world, int rank, int64_t chunk_vecs, int64_t recv_stride_vecs) {
     // W > 0: world known at compile time (fully unrolled loads); W == 0: generic
     constexpr int kParts = W > 0 ? W : kMaxWorld;
     constexpr int64_t kGroup = (int64_t)kReduceThreads * kVecsPerThread;
@@ -66,7 +66,7 @@ ring_reduce_kernel(const u32x4_t* __restrict__ recv, const u32x4_t* __restrict__
                     if (i < w) {
                         int src = rank + i;
                         if (src >= w) src -= w;
-                        parts[u][i] = __builtin_nontemporal_load(recv + (int64_t)src * chunk_vecs + v);
+                        parts[u][i] = __builtin_nontemporal_load(recv + (int64_t)src * recv_stride_vecs + v);
                     }
                 }
             }
@@ -82,7 +82,7 @@ ring_reduce_kernel(const u32x4_t* __restrict__ recv, const u32x4_t* __restrict__
                     if (i < w) {
                         int src = rank + i;
                         if (src >= w) src -= w;
-                        parts[i] = __builtin_nontemporal_load(recv + (int64_t)src * chunk_vecs + v);
+                        parts[i] = __builtin_nontemporal_load(recv + (int64_t)src * recv_stride_vecs + v);
                     }
                 }
                 __builtin_nontemporal_store(add8<T, ROUND_EACH>(parts, w), out + v);
@@ -93,7 +93,7 @@ ring_reduce_kernel(const u32x4_t* __restrict__ recv, const u32x4_t* __restrict__
 
 template <typename T, bool ROUND_EACH>
 static int launch_reduce(const void* recv, const void* local, void* out, int world, int rank,
-                         int64_t chunk_vecs, hipStream_t stream) {
+                         int64_t chunk_vecs, int64_t recv_stride_vecs, hipStream_t stream) {
     // a workgroup takes 1024 16-byte groups per pass; two workgroups per CU, beyond that they loop
     const int64_t group = (int64_t)kReduceThreads * kVecsPerThread;
     int64_t blocks = (chunk_vecs + group - 1) / group;
@@ -105,36 +105,45 @@ static int launch_reduce(const void* recv, const void* local, void* out, int wor
     const u32x4_t* l = reinterpret_cast<const u32x4_t*>(local);
     u32x4_t* o = reinterpret_cast<u32x4_t*>(out);
     switch (world) {
-        case 2: hipLaunchKernelGGL((ring_reduce_kernel<T, ROUND_EACH, 2>), grid, block, 0, stream, r, l, o, world, rank, chunk_vecs); break;
-        case 4: hipLaunchKernelGGL((ring_reduce_kernel<T, ROUND_EACH, 4>), grid, block, 0, stream, r, l, o, world, rank, chunk_vecs); break;
-        case 8: hipLaunchKernelGGL((ring_reduce_kernel<T, ROUND_EACH, 8>), grid, block, 0, stream, r, l, o, world, rank, chunk_vecs); break;
-        default: hipLaunchKernelGGL((ring_reduce_kernel<T, ROUND_EACH, 0>), grid, block, 0, stream, r, l, o, world, rank, chunk_vecs); break;
+        case 2: hipLaunchKernelGGL((ring_reduce_kernel<T, ROUND_EACH, 2>), grid, block, 0, stream, r, l, o, world, rank, chunk_vecs, recv_stride_vecs); break;
+        case 4: hipLaunchKernelGGL((ring_reduce_kernel<T, ROUND_EACH, 4>), grid, block, 0, stream, r, l, o, world, rank, chunk_vecs, recv_stride_vecs); break;
+        case 8: hipLaunchKernelGGL((ring_reduce_kernel<T, ROUND_EACH, 8>), grid, block, 0, stream, r, l, o, world, rank, chunk_vecs, recv_stride_vecs); break;
+        default: hipLaunchKernelGGL((ring_reduce_kernel<T, ROUND_EACH, 0>), grid, block, 0, stream, r, l, o, world, rank, chunk_vecs, recv_stride_vecs); break;
     }
     return (int)hipGetLastError();
 }
 
 }  // namespace syn
 
-extern "C" int syn_ring_reduce(const void* recv, const void* local, void* out, int32_t world,
-                               int32_t rank, int64_t rows_per_rank, int64_t N, int32_t dtype,
-                               int32_t acc_mode, syn_stream_t stream) {
+extern "C" int syn_ring_reduce_strided(const void* recv, int64_t recv_block_stride, const void* local, void* out,
+                                       int32_t world, int32_t rank, int64_t rows_per_rank, int64_t N, int32_t dtype,
+                                       int32_t acc_mode, syn_stream_t stream) {
     using namespace syn;
     if (!recv || !local || !out) return SYN_EINVAL;
     if (world < 1 || world > kMaxWorld || rank < 0 || rank >= world) return SYN_EINVAL;
     if (rows_per_rank <= 0 || N <= 0) return SYN_EINVAL;
     if (acc_mode != 0 && acc_mode != 1) return SYN_EINVAL;
     const int64_t elems = rows_per_rank * N;
-    if (elems % 8) return SYN_EALIGN;
+    if (recv_block_stride < elems) return SYN_EINVAL;
+    if (elems % 8 || recv_block_stride % 8) return SYN_EALIGN;
     if (!aligned16(recv) || !aligned16(local) || !aligned16(out)) return SYN_EALIGN;
-    const int64_t vecs = elems / 8;
+    const int64_t vecs = elems / 8, stride = recv_block_stride / 8;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     if (dtype == SYN_DTYPE_BF16) {
-        return acc_mode == 0 ? launch_reduce<__bf16, true>(recv, local, out, world, rank, vecs, s)
-                             : launch_reduce<__bf16, false>(recv, local, out, world, rank, vecs, s);
+        return acc_mode == 0 ? launch_reduce<__bf16, true>(recv, local, out, world, rank, vecs, stride, s)
+                             : launch_reduce<__bf16, false>(recv, local, out, world, rank, vecs, stride, s);
     }
     if (dtype == SYN_DTYPE_FP16) {
-        return acc_mode == 0 ? launch_reduce<_Float16, true>(recv, local, out, world, rank, vecs, s)
-                             : launch_reduce<_Float16, false>(recv, local, out, world, rank, vecs, s);
+        return acc_mode == 0 ? launch_reduce<_Float16, true>(recv, local, out, world, rank, vecs, stride, s)
+                             : launch_reduce<_Float16, false>(recv, local, out, world, rank, vecs, stride, s);
     }
     return SYN_EINVAL;
+}
+
+extern "C" int syn_ring_reduce(const void* recv, const void* local, void* out, int32_t world,
+                               int32_t rank, int64_t rows_per_rank, int64_t N, int32_t dtype,
+                               int32_t acc_mode, syn_stream_t stream) {
+    if (rows_per_rank <= 0 || N <= 0) return SYN_EINVAL;
+    return syn_ring_reduce_strided(recv, rows_per_rank * N, local, out, world, rank, rows_per_rank, N, dtype, acc_mode,
+                                   stream);
 }

@@ -36,6 +36,33 @@ def test_ring_reduce_bit_exact(hip, dtype, name, world, rows, N, acc_mode):
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
+@pytest.mark.parametrize("world,rows,N", [(8, 128, 512), (3, 40, 72), (1, 16, 64)])
+def test_ring_reduce_over_blocks_that_lie_apart(hip, world, rows, N):
+    """The received blocks as a [W, rows, N] view of a padded buffer (blocks 4 KiB further apart than
+    their size, the gaps poisoned): the same bits as from the contiguous layout."""
+    from syncopate_amd.computation.reduce import padded_receive_buffer, ring_reduce
+
+    rank = world // 2
+    recv, local = _case(world, rows, N, torch.bfloat16, seed=7 * world)
+    want = numerics.ring_reduce(recv.float().numpy(), local.float().numpy(), rank, dtype="bf16", round_each_add=True)
+    padded = padded_receive_buffer(world, rows, N, torch.bfloat16, "cuda")
+    assert padded.shape == recv.shape and (world == 1 or padded.stride(0) == rows * N + 2048)
+    torch.as_strided(padded, (world * (rows * N + 2048),), (1,)).fill_(float("nan"))
+    padded.copy_(recv)
+    padded[rank].fill_(float("nan"))
+    out = torch.empty(rows, N, dtype=torch.bfloat16, device="cuda")
+    ring_reduce(padded, out, local.cuda(), rank)
+    assert np.array_equal(out.float().cpu().numpy().view(np.uint32), want.view(np.uint32))
+    # blocks that are not whole 16-byte groups apart, or that overlap, are refused
+    flat = torch.zeros(world * (rows * N + 4) + 8, dtype=torch.bfloat16, device="cuda")
+    if world > 1:
+        from syncopate_amd import _lib
+        with pytest.raises(_lib.SyncopateHipError):
+            ring_reduce(torch.as_strided(flat, (world, rows, N), (rows * N + 4, N, 1)), out, local.cuda(), rank)
+        with pytest.raises(ValueError):
+            ring_reduce(torch.as_strided(flat, (world, rows, N), (rows * N - 8, N, 1)), out, local.cuda(), rank)
+
+
 def test_ring_reduce_full_size_properties(hip):
     """Benchmark size (8 x (1024, 8192) bf16): integer-valued inputs make every partial sum
     exact, so the result must equal the integer sum whatever the order or rounding."""

@@ -84,6 +84,30 @@ def test_mfma_rate_probe_runs_and_rejects_bad_arguments(hip):
     assert hip.syn_probe_mfma_rate(sink.data_ptr(), 0, 3, 0, stream) == _lib.SYN_EINVAL
 
 
+def test_read_stream_probe_reads_what_it_says(hip):
+    """The benchmark's HBM read probe: eight streams a stride apart, one pass of 1024 groups each.  A marker in
+    the first 256 groups of the last stream reaches every lane once and shows up in the sink; the same
+    marker just past the stream's end is never read."""
+    from syncopate_amd import _lib
+
+    magic, stream_bytes, stride = 0x9E3779B9, 16384, 16384 + 4096
+    stream = _lib.stream_handle(torch.cuda.current_stream())
+    for beyond in (False, True):
+        words = torch.zeros((8 * stride + 16384) // 4, dtype=torch.int32, device="cuda")
+        first = (7 * stride + (stream_bytes if beyond else 0)) // 4
+        words[first:first + 4 * 256:4] = magic - (1 << 32)
+        sink = torch.zeros(4, dtype=torch.int32, device="cuda")
+        _lib.check("syn_probe_read_streams",
+                   hip.syn_probe_read_streams(words.data_ptr(), stream_bytes, stride, 8, 1, sink.data_ptr(), stream))
+        torch.cuda.synchronize()
+        got = [w & 0xFFFFFFFF for w in sink.tolist()]
+        assert got == ([0, 0, 0, 0] if beyond else [magic, 0, 0, 0])
+    assert hip.syn_probe_read_streams(words.data_ptr(), 16000, stride, 8, 1, sink.data_ptr(), stream) == _lib.SYN_EINVAL
+    assert hip.syn_probe_read_streams(words.data_ptr(), stream_bytes, stride, 3, 1, sink.data_ptr(), stream) == _lib.SYN_EINVAL
+    assert hip.syn_probe_read_streams(words.data_ptr(), stream_bytes, stride + 8, 8, 1, sink.data_ptr(), stream) == _lib.SYN_EALIGN
+    assert hip.syn_probe_read_streams(None, stream_bytes, stride, 8, 1, sink.data_ptr(), stream) == _lib.SYN_EINVAL
+
+
 def test_flag_write_as_a_stream_memory_operation(hip):
     """syn_flag_write_value: the flag word is written by the stream itself, in stream order."""
     from syncopate_amd import _lib
