@@ -269,6 +269,58 @@ def test_chained_q_blocks_argument_errors_and_timeout(hip):
     check_status()
 
 
+@pytest.mark.parametrize("seed", list(range(6)))
+def test_random_wave_tables(hip, seed):
+    """Tables drawn at random: heads, q rows and kv rows cut into ragged ranges, every (head range, q range, kv
+    range) one wave, in a random order, with a random program count; odd seeds with two q blocks per
+    workgroup.  The visit log equals the oracle's tile by tile, the result the chunked oracle's."""
+    import numpy as np
+
+    from syncopate_amd.computation.attn import attention_forward
+    from syncopate_amd.computation._launch import check_status
+
+    rng = np.random.default_rng(2000 + seed)
+    pair = bool(seed & 1)
+    Z, H = int(rng.integers(1, 3)), int(rng.integers(1, 4))
+    Sq, Skv = 256 * int(rng.integers(1, 4)), 128 * int(rng.integers(2, 9))
+
+    def cut(extent, block, max_parts):
+        blocks = extent // block
+        parts = int(rng.integers(1, min(max_parts, blocks) + 1))
+        cuts = sorted(rng.choice(range(1, blocks), size=parts - 1, replace=False).tolist()) if parts > 1 else []
+        edges = [0] + cuts + [blocks]
+        return [(lo * block, (hi - lo) * block) for lo, hi in zip(edges, edges[1:])]
+
+    heads, qs, kvs = cut(H, 1, 2), cut(Sq, 256 if pair else 128, 2), cut(Skv, 128, 4)
+    cells = [(h, q_, kv) for h in heads for q_ in qs for kv in kvs]
+    order = rng.permutation(len(cells)).tolist()
+    offsets = [[0, cells[i][0][0], cells[i][1][0], cells[i][2][0]] for i in order]
+    sizes = [[Z, cells[i][0][1], cells[i][1][1], cells[i][2][1]] for i in order]
+    cums, total = [], 0
+    for sz in sizes:
+        total += sz[0] * sz[1] * sz[2]
+        cums.append(total)
+    signals = [int(rng.integers(-1, 2)) for _ in order]
+    tiles = total // 128
+    num_programs = int(rng.choice([0, 1, 3, 7]))
+    q, k, v = _qkv(Z, H, Sq, Skv, torch.bfloat16, seed=seed)
+    flags = torch.ones(2, dtype=torch.int64, device="cuda")
+    log = torch.full((tiles, 8), -1, dtype=torch.int32, device="cuda")
+    sm_scale = 128 ** -0.5
+    o = attention_forward(q.cuda(), k.cuda(), v.cuda(), sm_scale, wave_offsets=offsets, wave_sizes=sizes,
+                          cum_wave_sizes=cums, signal_ptr=flags, signal_offsets=signals, NUM_WAVES=len(order),
+                          cum_tiles=total, num_programs=num_programs, visit_log=log, pair_q_blocks=pair)
+    check_status()
+    assert _rel(o, numerics.sdpa_fp32(q, k, v, sm_scale)) <= REL_TOL
+    got = log.cpu().tolist()
+    units = tiles // 2 if pair else tiles
+    grid = min(num_programs, units) if num_programs else units
+    for tile_id, rec in enumerate(got):
+        exp = visit_order.attn_tile_work(tile_id, offsets, sizes, cums, signals)
+        assert rec[:7] == [exp["wave"], exp["z"], exp["h"], exp["q_block"], exp["kv_lo"], exp["kv_hi"], exp["signal"]]
+        assert rec[7] == ((tile_id // 2) if pair else tile_id) % grid
+
+
 def test_paired_q_blocks_argument_errors(hip):
     from syncopate_amd.computation.attn import attention_forward
 

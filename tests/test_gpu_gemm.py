@@ -119,6 +119,62 @@ def test_consumer_group_size_and_column_waves(hip):
         _check_visits(log, sizes, offsets, signals, M, N, BM, BN, group_m, num_sms, cum, True)
 
 
+def _random_cells(rng, extent, block, max_parts):
+    """`extent` cut into 1..max_parts runs of whole blocks: [(first, length)] in elements."""
+    blocks = extent // block
+    parts = int(rng.integers(1, min(max_parts, blocks) + 1))
+    cuts = sorted(rng.choice(range(1, blocks), size=parts - 1, replace=False).tolist()) if parts > 1 else []
+    edges = [0] + cuts + [blocks]
+    return [(lo * block, (hi - lo) * block) for lo, hi in zip(edges, edges[1:])]
+
+
+@pytest.mark.parametrize("seed", list(range(8)))
+def test_consumer_random_wave_tables(hip, seed):
+    """Wave tables drawn at random - the M x N tile space cut into cells of ragged sizes, visited in a random order,
+    with a random group size, program count, tile shape and flag assignment: the visit log equals the
+    oracle's walk tile by tile and the product is within tolerance."""
+    import numpy as np
+
+    from syncopate_amd.computation.gemm import gemm
+    from syncopate_amd.computation._launch import check_status
+
+    rng = np.random.default_rng(1000 + seed)
+    BM, BN = [(128, 128), (128, 256), (256, 128), (256, 256)][seed % 4]
+    M, N, K = 256 * int(rng.integers(2, 7)), 256 * int(rng.integers(1, 5)), 64 * int(rng.integers(2, 7))
+    rows, cols = _random_cells(rng, M, BM, 4), _random_cells(rng, N, BN, 3)
+    cells = [(r, c) for r in rows for c in cols]
+    order = rng.permutation(len(cells)).tolist()
+    sizes = [[cells[i][0][1], cells[i][1][1]] for i in order]
+    offsets = [[cells[i][0][0], cells[i][1][0]] for i in order]
+    num_flags = 3
+    signals = [int(rng.integers(-1, num_flags)) for _ in order]
+    group_m, num_sms = int(rng.choice([1, 2, 3, 8])), int(rng.integers(1, 48))
+    a, b = _inputs(M, N, K, torch.bfloat16, seed=seed)
+    ref = numerics.gemm_fp32(a, b)
+    flags = torch.ones(num_flags, dtype=torch.int64, device="cuda")
+    c = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    tiles = (M // BM) * (N // BN)
+    log = torch.full((tiles, 4), -1, dtype=torch.int32, device="cuda")
+    gemm(a.cuda(), b.cuda(), c, 1, num_sms, BM, BN, 64, group_m, cur_wave_sizes=sizes, wave_offsets=offsets,
+         signal_ptr=flags, signal_offsets=signals, cum_tiles=M * N, visit_log=log, xcd_remap=bool(seed & 1))
+    check_status()
+    assert _max_rel_err(c, ref) <= REL_TOL
+    want = visit_order.gemm_tile_visits(sizes, offsets, signals, M=M, N=N, BM=BM, BN=BN, group_m=group_m,
+                                        num_sms=num_sms, cum_tiles=M * N)
+    got = log.cpu().tolist()
+    assert len(want) == tiles
+    grid = min(num_sms, tiles)
+    for v in want:
+        pid, wave, pm, pn = got[v["tile_id"]]
+        assert (wave, pm, pn) == (v["wave"], v["pid_m"], v["pid_n"]), v
+        if not seed & 1:
+            assert pid == v["pid"]
+        else:
+            assert 0 <= pid < grid      # with the XCD remap the log holds the logical program id
+    if seed & 1:
+        assert [got[v["tile_id"]][0] for v in want] == [v["pid"] for v in want]
+
+
 def test_consumer_gated_by_side_stream_producer(hip):
     """Chunks land in the symmetric buffer on a side stream (copy, then flag) while the
     consumer is already running; the result must be bitwise the resident one (the flow of
