@@ -530,7 +530,7 @@ def run_gemm_rs(device, steps, warmup, gated=True):
 # ------------------------------------------------------------------------------------ attention
 
 def _gated_attention(q, staged_kv, buf, arrival, chunk, tables, launches, device, causal=False, pair=False,
-                     programs=0, copy_units=32):
+                     programs=0, copy_units=32, xcd_remap=False):
     """Attention over `buf` (stacked K, V of shape [2, B, H, S, D]) while the kv chunks arrive:
     chunk arrival[0] is resident, the others are copied from `staged_kv` by a side-stream
     producer in arrival order - a box copy on `copy_units` compute units, then the chunk's flag.
@@ -555,6 +555,11 @@ def _gated_attention(q, staged_kv, buf, arrival, chunk, tables, launches, device
     def step(i):
         flags.zero_()
         side.wait_stream(main)
+        # The kernel is launched first: its persistent workgroups then hold `programs` compute units and the
+        # copy kernels get the rest.  A copy kernel that starts first spreads its small workgroups over many
+        # compute units, none of which can take an attention workgroup (all registers of a SIMD) until it ends.
+        attention_forward(q, buf[0], buf[1], D ** -0.5, out=out, signal_ptr=flags, causal=causal, pair_q_blocks=pair,
+                          num_programs=programs, xcd_remap=xcd_remap, **tables)
         with torch.cuda.stream(side):
             for wave in range(1, len(arrival)):
                 c = arrival[wave]
@@ -562,8 +567,6 @@ def _gated_attention(q, staged_kv, buf, arrival, chunk, tables, launches, device
                                             buf[:, :, :, c * chunk:(c + 1) * chunk], num_sms=copy_units)
                 _lib.check("syn_flag_set", lib.syn_flag_set(flags.data_ptr() + 8 * signals[wave], 1,
                                                             _lib.stream_handle(side)))
-        attention_forward(q, buf[0], buf[1], D ** -0.5, out=out, signal_ptr=flags, causal=causal, pair_q_blocks=pair,
-                          num_programs=programs, **tables)
         main.wait_stream(side)
 
     ms = _timed(step, launches, 2)
@@ -604,7 +607,7 @@ def run_attention_ag(device, launches=5, gated=True):
     # the reference's protocol: 256 persistent workgroups, every tile merged into the output under its q block's lock
     merged_ms = resident(xcd_remap=True, num_programs=256)
     plain_ms = resident()           # one workgroup per pair of q blocks, dealt round-robin over the XCDs
-    persistent_ms = resident(num_programs=224)
+    persistent_ms = resident(num_programs=224, xcd_remap=True)
     s = (q[0, 7].float() @ kv[0, 0, 7].float().t()) * D ** -0.5
     ref = torch.softmax(s, dim=-1) @ kv[1, 0, 7].float()
     err = ((out[0, 7].float() - ref).abs().max() / ref.abs().max()).item()
@@ -614,11 +617,17 @@ def run_attention_ag(device, launches=5, gated=True):
     if not gated:
         return result
     buf = torch.empty_like(kv)
-    gated_ms, gated_out = _gated_attention(q, kv, buf, arrival, chunk, tables, launches, device, pair=True, programs=224)
+    gated_ms, gated_out = _gated_attention(q, kv, buf, arrival, chunk, tables, launches, device, pair=True, programs=224,
+                                           xcd_remap=True)
     gated_err = ((gated_out[0, 7].float() - ref).abs().max() / ref.abs().max()).item()
+    # the device warms up over these launches (consecutive launches of one kernel get 1 % slower each): the resident
+    # form is timed again behind the gated one and the overhead is quoted against the mean of the two
+    persistent_after_ms = resident(num_programs=224, xcd_remap=True)
+    baseline_ms = 0.5 * (persistent_ms + persistent_after_ms)
     result.update({"ms_gated": gated_ms, "gated_max_rel_err_vs_fp32": gated_err,
                    "gathered_kv_matches": bool(torch.equal(buf, kv)),
-                   "flag_wait_overhead_pct": 100.0 * (gated_ms - persistent_ms) / persistent_ms,
+                   "ms_224_programs_resident_after_gated": persistent_after_ms,
+                   "flag_wait_overhead_pct": 100.0 * (gated_ms - baseline_ms) / baseline_ms,
                    "gated_tflops": result["flop"] / (gated_ms * 1e-3) / 1e12})
     return result
 
@@ -705,9 +714,14 @@ def run_attention_a2a(device, launches=5, gated=True):
     gated_ms = _timed(step, launches, 2)
     check_status()
     gated_err = ((out[0, 1][rows].float() - ref).abs().max() / ref.abs().max()).item()
+    # timed again behind the gated launches: the overhead is quoted against the mean of the two (the device warms up)
+    persistent_after_ms = _timed(lambda i: attention_forward(qkv[0], qkv[1], qkv[2], scale, out=out, signal_ptr=ones,
+                                                             causal=True, num_programs=448, **tables), launches, 2)
+    baseline_ms = 0.5 * (persistent_ms + persistent_after_ms)
     result.update({"ms_causal_448_programs_resident": persistent_ms, "ms_causal_gated": gated_ms,
+                   "ms_causal_448_programs_resident_after_gated": persistent_after_ms,
                    "gated_max_rel_err_vs_fp32": gated_err, "gathered_qkv_matches": bool(torch.equal(buf, qkv)),
-                   "flag_wait_overhead_pct": 100.0 * (gated_ms - persistent_ms) / persistent_ms,
+                   "flag_wait_overhead_pct": 100.0 * (gated_ms - baseline_ms) / baseline_ms,
                    "gated_causal_tflops": result["flop_causal"] / (gated_ms * 1e-3) / 1e12})
     return result
 
