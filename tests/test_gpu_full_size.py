@@ -278,3 +278,76 @@ def test_allgather_attention_full_size_with_chunks_arriving_behind_flags(hip):
     for h in (0, 17, 31):
         s = (q[0, h].float() @ kv[0, 0, h].float().t()) * D ** -0.5
         assert _rel(o[0, h], torch.softmax(s, dim=-1) @ kv[1, 0, h].float()) <= REL_TOL
+
+
+def test_allgather_attention_full_size_chained(hip):
+    """The same configuration in the chained form (512 programs, each walking its two q blocks through the
+    eight chunks with the sums in registers): resident, against fp32 on sampled heads, against the form
+    that merges after every tile, and the visit log of all 8192 tiles against the oracle; then gated on a
+    device split by compute-unit masks - the waiting programs hold their compute units, so the stand-in
+    producer's copy kernels get 32 units of their own - with the rest of the buffer NaN until it is copied."""
+    from oracle import visit_order
+    from syncopate_amd import _lib
+    from syncopate_amd.communication.comm_runtime.cu_partition import split_device_cu_mask
+    from syncopate_amd.communication.comm_runtime.persistent_copy import persistent_copy_last_contig
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.attn import attention_forward
+
+    B, H, Sq, Skv, D, chunks = 1, 32, 4096, 32768, 128, 8
+    g = torch.Generator(device="cuda").manual_seed(2)
+    q = torch.randn(B, H, Sq, D, device="cuda", generator=g).bfloat16()
+    kv = torch.randn(2, B, H, Skv, D, device="cuda", generator=g).bfloat16()
+    chunk = Skv // chunks
+    arrival, signals = [0, 1, 7, 6, 4, 5, 3, 2], [-1, 0, 4, 1, 5, 2, 6, 3]
+    tables = _attn_tables(B, H, Sq, chunk, arrival, signals)
+    ones = torch.ones(chunks, dtype=torch.int64, device="cuda")
+    tiles = tables["cum_tiles"] // 128
+    pairs_per_wave = B * H * Sq // 256
+    log = torch.full((tiles, 8), -1, dtype=torch.int32, device="cuda")
+    o = attention_forward(q, kv[0], kv[1], D ** -0.5, signal_ptr=ones, pair_q_blocks=True, chain_q_blocks=True,
+                          xcd_remap=True, visit_log=log, **tables)
+    check_status()
+    refs = {}
+    for h in (0, 17, 31):
+        s = (q[0, h].float() @ kv[0, 0, h].float().t()) * D ** -0.5
+        refs[h] = torch.softmax(s, dim=-1) @ kv[1, 0, h].float()
+        assert _rel(o[0, h], refs[h]) <= REL_TOL
+        del s
+    merged = attention_forward(q, kv[0], kv[1], D ** -0.5, signal_ptr=ones, pair_q_blocks=True, num_programs=256,
+                               xcd_remap=True, **tables)
+    check_status()
+    assert _rel(merged, o) <= 2 * REL_TOL
+    got = log.cpu().tolist()
+    for tile_id in range(0, tiles, 7):
+        exp = visit_order.attn_tile_work(tile_id, tables["wave_offsets"], tables["wave_sizes"], tables["cum_wave_sizes"],
+                                         signals)
+        assert got[tile_id][:7] == [exp["wave"], exp["z"], exp["h"], exp["q_block"], exp["kv_lo"], exp["kv_hi"],
+                                    exp["signal"]]
+    programs = [rec[7] for rec in got[0::2]]
+    assert sorted(programs[:pairs_per_wave]) == list(range(pairs_per_wave))
+    assert programs == programs[:pairs_per_wave] * chunks            # a program's pair is the same in every wave
+
+    (comm, rest), sizes = split_device_cu_mask(torch.device("cuda", torch.cuda.current_device()), 1, 32)
+    assert sizes == [32, 224]
+    buf = torch.full_like(kv, float("nan"))
+    buf[:, :, :, :chunk].copy_(kv[:, :, :, :chunk])
+    flags = torch.zeros(chunks, dtype=torch.int64, device="cuda")
+    out = torch.empty_like(q)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(comm):
+        for wave in range(1, chunks):
+            c = arrival[wave]
+            _lib.check("syn_delay_us", hip.syn_delay_us(100, _lib.stream_handle(comm)))
+            persistent_copy_last_contig(kv[:, :, :, c * chunk:(c + 1) * chunk], buf[:, :, :, c * chunk:(c + 1) * chunk],
+                                        num_sms=32, stream=comm)
+            _lib.check("syn_flag_set", hip.syn_flag_set(flags.data_ptr() + 8 * signals[wave], 1, _lib.stream_handle(comm)))
+    attention_forward(q, buf[0], buf[1], D ** -0.5, signal_ptr=flags, pair_q_blocks=True, chain_q_blocks=True,
+                      xcd_remap=True, spin_timeout_us=5_000_000, out=out, stream=rest, **tables)
+    torch.cuda.synchronize()
+    check_status()
+    assert flags.tolist()[:7] == [1] * 7
+    assert torch.equal(buf, kv)
+    assert not torch.isnan(out).any()
+    for h, ref in refs.items():
+        assert _rel(out[0, h], ref) <= REL_TOL
+
