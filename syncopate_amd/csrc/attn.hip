@@ -199,6 +199,25 @@ typedef __attribute__((address_space(3))) s16x4_t* lds_s16x4_ptr;
 // s_waitcnt immediate (gfx9 encoding): at most `vm` vector-memory operations outstanding
 constexpr int attn_vmcnt(int vm) { return (vm & 0xF) | ((vm >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
 
+// The wave a tile id falls into: the first w with cum_wave_sizes[w] / block > tile_id (the reference walks
+// the prefix sums one by one, template.py:39-44).  The prefix sums rise over the real waves and zero rows
+// may pad the table's end, so that index is the number of real waves at or below the tile: sixty-four
+// of them are looked at per load, one per lane, instead of one per trip to memory.  Wavefront-uniform;
+// num_waves if the tile lies beyond the table.
+__device__ __forceinline__ int find_wave(const int32_t* __restrict__ cum_wave_sizes, int num_waves, int block, int tile_id,
+                                         int lane) {
+    int w = 0;
+    for (int base = 0; base < num_waves; base += 64) {
+        const int idx = base + lane;
+        const int cum = idx < num_waves ? cum_wave_sizes[idx] : 0;
+        const unsigned long long below = __builtin_amdgcn_ballot_w64(cum != 0 && cum / block <= tile_id);
+        w += __builtin_popcountll(below);
+        if (below != ~0ull) break;
+    }
+    if (w < num_waves && cum_wave_sizes[w] == 0) w = num_waves;        // only padding is left
+    return w;
+}
+
 // One kv block (128 rows of 256 bytes, `pitch` bytes apart in HBM) into LDS.  Wavefront `wave`
 // issues 1 KB fills number wave, wave + 4, ... (4 rows each); lane l lands at byte 16*l of the
 // fill, i.e. row l/16, physical 16-byte chunk l%16, and `lane_off` (row l/16 at the pitch, plus
@@ -278,8 +297,7 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
     const int first_tile = logical_program_id((int)blockIdx.x, (int)gridDim.x, p.xcd_remap != 0);
     for (int tile_id = first_tile; tile_id < p.num_tiles; tile_id += gridDim.x) {
         // ---- tile id -> wave -> (z, h, q block, kv range) ----
-        int w = 0;
-        while (w < p.num_waves && p.cum_wave_sizes[w] / kBlockM <= tile_id) ++w;
+        const int w = find_wave(p.cum_wave_sizes, p.num_waves, kBlockM, tile_id, lane);
         if (w >= p.num_waves) return;
         const int prev = w == 0 ? 0 : p.cum_wave_sizes[w - 1] / kBlockM;
         const int t = tile_id - prev;
@@ -656,8 +674,7 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
     for (int pair = first_pair; pair < num_pairs; pair += gridDim.x) {
         // ---- tile id -> wave -> (z, h, q block, kv range); the two tiles of a pair differ in the q block only ----
         const int tile_id = 2 * pair + grp;
-        int w = 0;
-        while (w < p.num_waves && p.cum_wave_sizes[w] / kBlockM <= tile_id) ++w;
+        const int w = find_wave(p.cum_wave_sizes, p.num_waves, kBlockM, tile_id, lane);
         if (w >= p.num_waves) return;
         const int prev = w == 0 ? 0 : p.cum_wave_sizes[w - 1] / kBlockM;
         const int t = tile_id - prev;
