@@ -27,6 +27,8 @@ import torch
 
 from ... import _lib
 from .._launch import (
+    recall_note,
+    remember_note,
     TableLike,
     already_checked,
     as_device_table,
@@ -42,9 +44,6 @@ from .._launch import (
 BLOCK_M = 128
 BLOCK_N = 128
 DEFAULT_SPIN_TIMEOUT_US = 2_000_000
-
-
-_chain_programs: dict = {}      # ids of a caller's four tables -> pairs of q blocks per wave (chain_q_blocks)
 
 
 @launches_on_stream
@@ -71,6 +70,7 @@ def attention_forward(
     pair_q_blocks: bool = False,
     xcd_remap: bool = False,
     chain_q_blocks: bool = False,
+    form: str = "explicit",
     out: Optional[torch.Tensor] = None,
     return_lse: bool = False,
     visit_log: Optional[torch.Tensor] = None,
@@ -106,6 +106,11 @@ def attention_forward(
     behind its flag) and writes every q block once, without locks or merges.  Programs, tiles and
     their order are those of the persistent launch with that `num_programs`.  A ValueError for
     tables of another shape.
+    `form="auto"` (what `attention()` passes): where none of the three options above, `causal`, `counter_ptr` or
+    `visit_log` is given, the launcher reads the tables and takes the fastest form they allow - two q blocks per
+    workgroup with the XCD remap where every wave holds an even number of q blocks, chained where the waves
+    also share their (z, h, q) ranges and `num_programs` is 0 or the pairs of a wave.  Results are the same
+    to rounding; what differs is which program a tile runs on, which only `visit_log` shows.
     """
     dev = require_cuda(q, k, v, signal_ptr)
     if not (q.dtype == k.dtype == v.dtype):
@@ -148,14 +153,37 @@ def attention_forward(
     if chain_q_blocks and not pair_q_blocks:
         raise ValueError("chain_q_blocks goes with pair_q_blocks")
     num_programs = int(num_programs)
+    host_tables = None
+    if form not in ("explicit", "auto"):
+        raise ValueError("form must be 'explicit' or 'auto'")
+    if form == "auto" and not (pair_q_blocks or chain_q_blocks or xcd_remap or causal or counter_ptr is not None
+                               or consumer_signal_ptr is not None or visit_log is not None):
+        choice = recall_note(tables, "attention form") if caller_owned else None
+        if choice is None:
+            host_tables = (host_copy(offs), host_copy(sizes), host_copy(cums), host_copy(sigs))
+            ho, hs, hc, _ = host_tables
+            real = [i for i in range(num_waves) if int(hc[i]) > 0]
+            even = bool(real) and all(int(hs[i, 2]) % (2 * BLOCK_M) == 0 for i in real)
+            same = even and all(ho[i, :3].tolist() == ho[real[0], :3].tolist() and
+                                hs[i, :3].tolist() == hs[real[0], :3].tolist() for i in real)
+            pairs = int(hs[real[0], 0]) * int(hs[real[0], 1]) * int(hs[real[0], 2]) // (2 * BLOCK_M) if same else 0
+            choice = (even, pairs)
+            if caller_owned:
+                remember_note(tables, "attention form", choice)
+        even, pairs = choice
+        if even:
+            pair_q_blocks = xcd_remap = True
+            if pairs and num_programs in (0, pairs):
+                chain_q_blocks, num_programs = True, pairs
+    given_programs = num_programs
     if chain_q_blocks and num_programs <= 0 and caller_owned:
         # filled in by an earlier call on these tables; `already_checked` below vouches for it
-        num_programs = _chain_programs.get(tuple(id(t) for t in tables), 0)
+        num_programs = recall_note(tables, "chain programs") or 0
     params = (num_waves, Z, H, Sq, Skv, cum_tiles, flags.numel(), bool(pair_q_blocks),
               num_programs if chain_q_blocks else None)
     if cum_tiles is None or (chain_q_blocks and num_programs <= 0) or \
             not (caller_owned and already_checked(tables, params)):
-        ho, hs, hc, hg = host_copy(offs), host_copy(sizes), host_copy(cums), host_copy(sigs)
+        ho, hs, hc, hg = host_tables or (host_copy(offs), host_copy(sizes), host_copy(cums), host_copy(sigs))
         if cum_tiles is None:
             cum_tiles = int(hc[:num_waves].max().item())
         if pair_q_blocks and any(int(hs[i, 2]) % (2 * BLOCK_M) for i in range(num_waves) if int(hc[i]) > 0):
@@ -166,15 +194,13 @@ def attention_forward(
                                hs[i, :3].tolist() != hs[real[0], :3].tolist() for i in real):
                 raise ValueError("chain_q_blocks needs the same (z, h, q) ranges in every wave")
             pairs = int(hs[real[0], 0]) * int(hs[real[0], 1]) * int(hs[real[0], 2]) // (2 * BLOCK_M)
-            if num_programs <= 0:
+            if given_programs <= 0:
                 num_programs = pairs
             elif num_programs != pairs:
                 raise ValueError(f"chain_q_blocks needs num_programs = {pairs}, the pairs of q blocks of one wave")
             params = params[:-1] + (num_programs,)
             if caller_owned:
-                if len(_chain_programs) > 1024:
-                    _chain_programs.clear()
-                _chain_programs[tuple(id(t) for t in tables)] = num_programs
+                remember_note(tables, "chain programs", num_programs)
         _lib.check(
             "syn_attn_check_waves",
             lib.syn_attn_check_waves(host_ptr(ho), host_ptr(hs), host_ptr(hc), host_ptr(hg), num_waves,
@@ -259,7 +285,7 @@ def attention(q, k, v, sm_scale, wave_dicts: Dict, BLOCK_M=128, BLOCK_N=128, NUM
         q, k, v, sm_scale,
         wave_offsets=offs, wave_sizes=sizes, cum_wave_sizes=cums,
         signal_ptr=signal_ptr, signal_offsets=wave_dicts["signal_offsets"],
-        NUM_WAVES=wave_dicts.get("CUM_CHUNK_BLOCK"), **kwargs)
+        NUM_WAVES=wave_dicts.get("CUM_CHUNK_BLOCK"), **{"form": "auto", **kwargs})
 
 
 def build_waves_and_signals_divisible(Z, H, N_CTX_Q, N_CTX_KV, *, BLOCK_M=128, BLOCK_N=128, w=4,

@@ -321,6 +321,49 @@ def test_random_wave_tables(hip, seed):
         assert rec[7] == ((tile_id // 2) if pair else tile_id) % grid
 
 
+def test_auto_form_takes_what_the_tables_allow(hip):
+    """form="auto" (what attention() passes): chained where every wave lists the same (z, h, q) ranges, two q blocks
+    per workgroup where the waves hold even numbers of q blocks, one program per tile otherwise; the same result
+    to rounding every time, and the choice is remembered per table objects."""
+    from syncopate_amd.computation.attn import attention_forward
+    from syncopate_amd.computation._launch import check_status, recall_note
+
+    Z, H, Skv = 1, 2, 512
+    sm_scale = 128 ** -0.5
+    flags = torch.ones(2, dtype=torch.int64, device="cuda")
+
+    def tables_for(Sq, q_cuts):
+        offsets, sizes, cums, total = [], [], [], 0
+        for q_lo, q_len in q_cuts:
+            for kv_lo in (256, 0):
+                offsets.append([0, 0, q_lo, kv_lo])
+                sizes.append([Z, H, q_len, 256])
+                total += Z * H * q_len
+                cums.append(total)
+        dev = lambda rows: torch.tensor(rows, dtype=torch.int32, device="cuda")
+        return dict(wave_offsets=dev(offsets), wave_sizes=dev(sizes), cum_wave_sizes=dev(cums),
+                    signal_offsets=dev([-1, 0, 1, 0][:len(cums)]), cum_tiles=total)
+
+    cases = [(512, [(0, 512)], (True, Z * H * 512 // 256)),            # same q range in both waves: chained
+             (512, [(0, 256), (256, 256)], (True, 0)),                # two q ranges: pairs, merged under locks
+             (384, [(0, 384)], (False, 0))]                           # three q blocks per wave: one program per tile
+    for Sq, q_cuts, want in cases:
+        q, k, v = _qkv(Z, H, Sq, Skv, torch.bfloat16, seed=Sq)
+        t = tables_for(Sq, q_cuts)
+        o = attention_forward(q.cuda(), k.cuda(), v.cuda(), sm_scale, signal_ptr=flags, form="auto", **t)
+        check_status()
+        assert _rel(o, numerics.sdpa_fp32(q, k, v, sm_scale)) <= REL_TOL
+        key = (t["wave_offsets"], t["wave_sizes"], t["cum_wave_sizes"], t["signal_offsets"])
+        assert recall_note(key, "attention form") == want
+        o2 = attention_forward(q.cuda(), k.cuda(), v.cuda(), sm_scale, signal_ptr=flags, form="auto", **t)   # from the note
+        check_status()
+        assert torch.equal(o, o2) or _rel(o2, o.float().cpu()) <= REL_TOL
+        t["wave_sizes"][0, 3] = 256                                   # an in-place write: the note no longer holds
+        assert recall_note(key, "attention form") is None
+    with pytest.raises(ValueError, match="form"):
+        attention_forward(q.cuda(), k.cuda(), v.cuda(), sm_scale, signal_ptr=flags, form="fastest", **t)
+
+
 def test_paired_q_blocks_argument_errors(hip):
     from syncopate_amd.computation.attn import attention_forward
 
