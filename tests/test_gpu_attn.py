@@ -321,6 +321,48 @@ def test_random_wave_tables(hip, seed):
         assert rec[7] == ((tile_id // 2) if pair else tile_id) % grid
 
 
+def test_chained_form_replayed_as_a_graph(hip):
+    """The chained launch (scratch words zeroed by a fill kernel, the kernel itself) captured as a HIP graph and
+    replayed three times on new inputs, with eager work and synchronisation between the replays: every replay
+    gives what the eager launch gives on the same inputs."""
+    from syncopate_amd.computation.attn import attention_forward
+    from syncopate_amd.computation._launch import check_status
+
+    Z, H, Sq, Skv = 1, 2, 512, 768
+    sm_scale = 128 ** -0.5
+    chunks = [(256, 512), (0, 256), (512, 768)]
+    offsets, sizes, cums, signals, total = _kv_waves(Z, H, Sq, chunks, [-1, 0, 1])
+    dev = lambda rows: torch.tensor(rows, dtype=torch.int32, device="cuda")
+    tables = dict(wave_offsets=dev(offsets), wave_sizes=dev(sizes), cum_wave_sizes=dev(cums), signal_offsets=dev(signals),
+                  cum_tiles=total, NUM_WAVES=len(chunks))
+    flags = torch.ones(2, dtype=torch.int64, device="cuda")
+    q, k, v = (t.cuda() for t in _qkv(Z, H, Sq, Skv, torch.bfloat16, seed=30))
+    out = torch.zeros_like(q)
+    kw = dict(signal_ptr=flags, pair_q_blocks=True, chain_q_blocks=True, out=out, **tables)
+    attention_forward(q, k, v, sm_scale, **kw)          # warm-up: tables checked, program count noted
+    check_status()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph):
+            attention_forward(q, k, v, sm_scale, **kw)
+    torch.cuda.current_stream().wait_stream(side)
+    for replay in range(3):
+        nq, nk, nv = _qkv(Z, H, Sq, Skv, torch.bfloat16, seed=40 + replay)
+        q.copy_(nq.cuda()); k.copy_(nk.cuda()); v.copy_(nv.cuda())
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        check_status()
+        got = out.clone()
+        assert _rel(got, numerics.sdpa_fp32(nq, nk, nv, sm_scale)) <= REL_TOL, f"replay {replay}"
+        eager = attention_forward(q, k, v, sm_scale, **{**kw, "out": torch.empty_like(q)})
+        check_status()
+        assert torch.equal(got, eager), f"replay {replay}"
+
+
 def test_auto_form_takes_what_the_tables_allow(hip):
     """form="auto" (what attention() passes): chained where every wave lists the same (z, h, q) ranges, two q blocks
     per workgroup where the waves hold even numbers of q blocks, one program per tile otherwise; the same result
