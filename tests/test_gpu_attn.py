@@ -321,6 +321,39 @@ def test_random_wave_tables(hip, seed):
         assert rec[7] == ((tile_id // 2) if pair else tile_id) % grid
 
 
+@pytest.mark.parametrize("pair", [False, True])
+def test_more_waves_than_a_wavefront_has_lanes(hip, pair):
+    """Eighty waves of one kv block each, padded with zero rows to 128: the wave of a tile id is looked up sixty-four
+    prefix sums at a time, so the table spans two looks and ends in padding."""
+    from syncopate_amd.computation.attn import attention_forward
+    from syncopate_amd.computation._launch import check_status
+
+    Z, H, Sq, waves = 1, 1, 256, 80
+    Skv = waves * 128
+    q, k, v = _qkv(Z, H, Sq, Skv, torch.bfloat16, seed=50)
+    order = torch.randperm(waves, generator=torch.Generator().manual_seed(3)).tolist()
+    chunks = [(o * 128, (o + 1) * 128) for o in order]
+    offsets, sizes, cums, signals, total = _kv_waves(Z, H, Sq, chunks, [-1] * waves)
+    pad = 128 - waves
+    offsets += [[0, 0, 0, 0]] * pad
+    sizes += [[0, 0, 0, 0]] * pad
+    cums += [0] * pad
+    signals += [0] * pad
+    flags = torch.ones(1, dtype=torch.int64, device="cuda")
+    tiles = total // 128
+    log = torch.full((tiles, 8), -1, dtype=torch.int32, device="cuda")
+    sm_scale = 128 ** -0.5
+    o = attention_forward(q.cuda(), k.cuda(), v.cuda(), sm_scale, wave_offsets=offsets, wave_sizes=sizes,
+                          cum_wave_sizes=cums, signal_ptr=flags, signal_offsets=signals, NUM_WAVES=128, cum_tiles=total,
+                          visit_log=log, pair_q_blocks=pair, num_programs=3)
+    check_status()
+    # eighty partial results merged with a rounding each: twice the usual bound
+    assert _rel(o, numerics.sdpa_fp32(q, k, v, sm_scale)) <= 2 * REL_TOL
+    for tile_id, rec in enumerate(log.cpu().tolist()):
+        exp = visit_order.attn_tile_work(tile_id, offsets, sizes, cums, signals)
+        assert rec[:7] == [exp["wave"], exp["z"], exp["h"], exp["q_block"], exp["kv_lo"], exp["kv_hi"], exp["signal"]]
+
+
 def test_chained_form_replayed_as_a_graph(hip):
     """The chained launch (scratch words zeroed by a fill kernel, the kernel itself) captured as a HIP graph and
     replayed three times on new inputs, with eager work and synchronisation between the replays: every replay
