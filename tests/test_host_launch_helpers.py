@@ -1,0 +1,67 @@
+"""Host-side helpers of the launchers (no GPU): what a launcher remembers about a set of tables, and the
+padded receive buffer of the chunked reduce."""
+
+import gc
+
+import torch
+
+from syncopate_amd.computation._launch import already_checked, recall_note, remember_checked, remember_note
+from syncopate_amd.computation.reduce import RECEIVE_BLOCK_PAD_BYTES, padded_receive_buffer
+
+
+def _tables():
+    return tuple(torch.arange(4 * (i + 1), dtype=torch.int32) for i in range(4))
+
+
+def test_notes_are_kept_per_objects_and_versions():
+    tables = _tables()
+    assert recall_note(tables, "form") is None
+    remember_note(tables, "form", (True, 12))
+    remember_note(tables, "programs", 12)
+    assert recall_note(tables, "form") == (True, 12) and recall_note(tables, "programs") == 12
+    # other objects with the same contents: nothing is known about them
+    assert recall_note(_tables(), "form") is None
+    # an in-place write to any of the tables voids every note about the set
+    tables[2][0] = 7
+    assert recall_note(tables, "form") is None and recall_note(tables, "programs") is None
+    remember_note(tables, "form", (False, 0))
+    assert recall_note(tables, "form") == (False, 0)
+
+
+def test_a_note_does_not_outlive_its_tables():
+    """Ids are reused once an object is gone: a note is tied to the objects (weak references), not to their ids."""
+    tables = _tables()
+    remember_note(tables, "form", "old")
+    ids = tuple(id(t) for t in tables)
+    del tables
+    gc.collect()
+    for _ in range(64):                       # give the allocator a chance to hand the ids out again
+        fresh = _tables()
+        if tuple(id(t) for t in fresh) == ids:
+            assert recall_note(fresh, "form") is None
+            break
+        assert recall_note(fresh, "form") is None
+
+
+def test_checked_tables_cache_matches_parameters():
+    tables = _tables()
+    assert not already_checked(tables, (1, 2))
+    remember_checked(tables, (1, 2))
+    assert already_checked(tables, (1, 2)) and not already_checked(tables, (1, 3))
+    tables[0].add_(1)
+    assert not already_checked(tables, (1, 2))
+
+
+def test_padded_receive_buffer_layout():
+    world, rows, n = 8, 16, 64
+    buf = padded_receive_buffer(world, rows, n, torch.bfloat16, "cpu")
+    pad = RECEIVE_BLOCK_PAD_BYTES // 2
+    assert buf.shape == (world, rows, n) and buf.stride() == (rows * n + pad, n, 1)
+    assert buf[3].is_contiguous() and not buf.is_contiguous()
+    # blocks do not overlap: a write to one leaves the others alone
+    buf.zero_()
+    buf[3].fill_(1.0)
+    assert buf.sum().item() == rows * n
+    assert buf[4].data_ptr() - buf[3].data_ptr() == (rows * n + pad) * 2
+    one = padded_receive_buffer(1, rows, n, torch.float16, "cpu")
+    assert one.shape == (1, rows, n)
