@@ -344,16 +344,17 @@ def run_library_baselines(device, state):
     GEMM shapes, torch's scaled_dot_product_attention on the two attention shapes."""
     import torch.nn.functional as F
 
-    out = {"launches": 30}
+    # the board's clock settles over the first ~80 launches after other work (it rises): timed behind as many
+    out = {"launches": 100, "warmup_launches": 80}
     a, b = state["a"], state["b"]
-    ms = _timed(lambda i: torch.matmul(a, b.t()), 30, 10)
+    ms = _timed(lambda i: torch.matmul(a, b.t()), 100, 80)
     out["matmul_8192x8192x3584_tflops"] = 2.0 * M * N * K / ms / 1e9
     a2 = (0.02 * torch.randn(8192, 3584, device=device)).bfloat16()
     b2 = (0.02 * torch.randn(8192, 3584, device=device)).bfloat16()
-    ms = _timed(lambda i: torch.matmul(a2, b2.t()), 30, 10)
+    ms = _timed(lambda i: torch.matmul(a2, b2.t()), 100, 80)
     out["matmul_8192x3584x8192_tflops"] = 2.0 * 8192 * 8192 * 3584 / ms / 1e9
     za, zb = torch.zeros_like(a), torch.zeros_like(b)
-    ms = _timed(lambda i: torch.matmul(za, zb.t()), 30, 10)
+    ms = _timed(lambda i: torch.matmul(za, zb.t()), 100, 80)
     out["matmul_8192x8192x3584_zero_operands_tflops"] = 2.0 * M * N * K / ms / 1e9
     del a2, b2, za, zb
     q = torch.randn(1, 32, 4096, 128, device=device).bfloat16()
@@ -910,7 +911,7 @@ def main():
     flop = 2.0 * M * N * K
     value = flop / (wall_ms * 1e-3) / 1e12
     kernel_tflops = flop / (gated_ms * 1e-3) / 1e12
-    kernel_name = (f"gemm_wave_kernel<bf16, {'EarlyPipe' if (BM, BN) in ((256, 256), (256, 224)) else 'SlabPipe<3 stages>'}, "
+    kernel_name = (f"gemm_wave_kernel<bf16, {'EarlyPipe16' if (BM, BN) in ((256, 256), (256, 224)) else 'SlabPipe<3 stages>'}, "
                    f"{BM}x{BN}, {8 if EIGHT_WAVES else 4} wavefronts, consumer>")
     traffic = _traffic().get("gemm_consumer_256x256_224_programs", {}) if (BM, BN, NUM_SMS) == (256, 256, 224) else {}
     line = {

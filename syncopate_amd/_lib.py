@@ -32,6 +32,7 @@ SYN_GEMM_EIGHT_WAVES = 2
 SYN_GEMM_RING_PIPE = 4
 SYN_GEMM_NO_K_STAGGER = 8
 SYN_GEMM_TWO_STAGE = 16
+SYN_GEMM_MFMA_32X32 = 32
 SYN_ATTN_PAIR_Q_BLOCKS = 1
 SYN_ATTN_XCD_REMAP = 2
 SYN_ATTN_CHAIN_Q_BLOCKS = 4

@@ -62,6 +62,7 @@ def _launch(
     stream: Optional[torch.cuda.Stream],
     wait_signal_buffer: Optional[torch.Tensor] = None,
     wait_signal_offsets: Optional[TableLike] = None,
+    mfma_32x32: bool = False,
 ) -> None:
     # shape/dtype contract of the reference launchers (template.py:177-185)
     assert a.shape[1] == b.shape[1], "Incompatible dimensions"  # b is [N, K]
@@ -154,7 +155,7 @@ def _launch(
         spin_timeout_us=int(spin_timeout_us),
         options=(_lib.SYN_GEMM_XCD_REMAP if xcd_remap else 0) | (_lib.SYN_GEMM_EIGHT_WAVES if eight_waves else 0)
         | (_lib.SYN_GEMM_RING_PIPE if ring_pipe else 0) | (0 if k_stagger else _lib.SYN_GEMM_NO_K_STAGGER)
-        | (_lib.SYN_GEMM_TWO_STAGE if two_stage else 0),
+        | (_lib.SYN_GEMM_TWO_STAGE if two_stage else 0) | (_lib.SYN_GEMM_MFMA_32X32 if mfma_32x32 else 0),
     )
     with torch.cuda.device(dev):
         if wait_flags is not None:
@@ -190,6 +191,7 @@ def gemm_consumer(
     ring_pipe=False,
     k_stagger=True,
     two_stage=False,
+    mfma_32x32=False,
     spin_timeout_us=DEFAULT_SPIN_TIMEOUT_US,
     stream=None,
 ):
@@ -205,7 +207,7 @@ def gemm_consumer(
     assert M_per_rank % BLOCK_SIZE_M == 0
     _launch(False, a, b, c, signal_buffer, cur_wave_size, wave_offset, signal_offsets, num_gemm_sms,
             BLOCK_SIZE_M, BLOCK_SIZE_N, BLOCK_SIZE_K, GROUP_SIZE_M, cum_tiles, None, visit_log,
-            xcd_remap, eight_waves, ring_pipe, k_stagger, two_stage, spin_timeout_us, stream)
+            xcd_remap, eight_waves, ring_pipe, k_stagger, two_stage, spin_timeout_us, stream, mfma_32x32=mfma_32x32)
 
 
 def gemm_producer(
@@ -231,6 +233,7 @@ def gemm_producer(
     ring_pipe=False,
     k_stagger=True,
     two_stage=False,
+    mfma_32x32=False,
     stream=None,
 ):
     """GEMM+RS producer: same GEMM; every finished tile bumps its wave's counter
@@ -240,7 +243,8 @@ def gemm_producer(
     """
     _launch(True, a, b, c, signal_buffer, cur_wave_size, wave_offset, signal_offsets, num_gemm_sms,
             BLOCK_SIZE_M, BLOCK_SIZE_N, BLOCK_SIZE_K, GROUP_SIZE_M, cum_tiles, counter_buffer,
-            visit_log, xcd_remap, eight_waves, ring_pipe, k_stagger, two_stage, DEFAULT_SPIN_TIMEOUT_US, stream)
+            visit_log, xcd_remap, eight_waves, ring_pipe, k_stagger, two_stage, DEFAULT_SPIN_TIMEOUT_US, stream,
+            mfma_32x32=mfma_32x32)
 
 
 def gemm(
@@ -269,6 +273,7 @@ def gemm(
     ring_pipe=False,
     k_stagger=True,
     two_stage=False,
+    mfma_32x32=False,
     spin_timeout_us=DEFAULT_SPIN_TIMEOUT_US,
     stream=None,
 ):
@@ -283,4 +288,4 @@ def gemm(
     _launch(counter_ptr is not None, a, b, c, signal_ptr, cur_wave_sizes, wave_offsets, signal_offsets,
             num_gemm_sms, BLOCK_SIZE_M, BLOCK_SIZE_N, BLOCK_SIZE_K, GROUP_SIZE_M, cum_tiles,
             counter_ptr, visit_log, xcd_remap, eight_waves, ring_pipe, k_stagger, two_stage, spin_timeout_us, stream,
-            consumer_signal_ptr, consumer_signal_offsets)
+            consumer_signal_ptr, consumer_signal_offsets, mfma_32x32=mfma_32x32)

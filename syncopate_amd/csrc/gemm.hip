@@ -87,6 +87,27 @@ struct Mfma32<_Float16> {
     }
 };
 
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+template <typename T>
+struct Mfma16;
+
+template <>
+struct Mfma16<__bf16> {
+    // inline assembly: the accumulator is named as an AGPR tuple that is read and written in place (through the
+    // builtin the register allocator moves accumulators between the two register files inside the K loop)
+    static __device__ __forceinline__ void run(bf16x8_t a, bf16x8_t b, f32x4_t& c) {
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    }
+};
+
+template <>
+struct Mfma16<_Float16> {
+    static __device__ __forceinline__ void run(f16x8_t a, f16x8_t b, f32x4_t& c) {
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    }
+};
+
 template <typename T>
 __device__ __forceinline__ uint2 pack4(float x0, float x1, float x2, float x3) {
     typedef T vec4 __attribute__((ext_vector_type(4)));
@@ -236,6 +257,15 @@ __device__ __forceinline__ void dma_blocks(unsigned char* stage_wave, const unsi
     }
 }
 
+// fill j of the wavefront alone
+template <int BM, int NW, int NV>
+__device__ __forceinline__ void dma_one(int j, unsigned char* stage_wave, const unsigned char* a_k,
+                                        const unsigned char* b_k, const unsigned (&voff)[NV]) {
+    constexpr int kAFills = BM / (8 * NW);
+    const unsigned char* src = j < kAFills ? a_k + voff[j] : b_k + voff[j - kAFills];
+    __builtin_amdgcn_global_load_lds((global_void_ptr)src, (lds_void_ptr)(stage_wave + j * NW * 1024), 16, 0, 0);
+}
+
 // ------------------------------------------------------------------ pipelines
 //
 // Both are split in two: prologue() issues the first fills of a tile from the uniform addresses
@@ -265,6 +295,7 @@ struct SlabPipe {
     static constexpr int LDS_BYTES = NST * STAGE;
     static constexpr int FILLS = (BM + BN) / (8 * NW);
     static constexpr int K_ALIGN = 64;
+    static constexpr bool kMfma16 = false;
     typedef typename Mfma32<T>::frag_t frag_t;
 
     static constexpr int NV = (BM > BN ? BM : BN) / (8 * NW);    // fills per wavefront and operand
@@ -538,6 +569,144 @@ struct EarlyPipe : SlabPipe<T, BM, BN, WGM, WGN, 2> {
     }
 };
 
+// early16: the early-read pipeline on 16x16x32 MFMAs.  A wavefront's 128 x 128 part of the tile is 8 x 8 accumulators
+// of 16 x 16; a slab is two k32 steps of 64 MFMAs, run as four quarters of 32 (row blocks 0-3 or 4-7 of A against all
+// eight column blocks).  A k32 step needs eight fragments of A and eight of B (one 128-bit LDS read each, lane l:
+// row l % 16, 16-byte chunk l / 16 of the step's four), so the fragments of both steps are again 128 VGPRs:
+//     quarter 3 of slab s-1: MFMAs | read the fragments of k32 step 0 of slab s
+//     quarter 0: MFMAs | read the fragments of step 1;  wait for them;  barrier: the stage is free
+//     quarter 1: MFMAs | first third of the fills of slab s+2 into that stage
+//     quarter 2: MFMAs | second third;  wait: own fills of slab s+1 landed;  barrier
+//     quarter 3: MFMAs | last third | read step 0 of slab s+1
+template <typename T, int BM, int BN, int WGM, int WGN>
+struct EarlyPipe16 : SlabPipe<T, BM, BN, WGM, WGN, 2> {
+    typedef SlabPipe<T, BM, BN, WGM, WGN, 2> Base;
+    using Base::TM;
+    using Base::TN;
+    using Base::ROW;
+    using Base::FILLS;
+    using Base::NW;
+    using Base::NV;
+    using Base::BK;
+    using Base::WM;
+    using Base::WN;
+    using Base::A_BYTES;
+    typedef typename Base::frag_t frag_t;
+    typedef typename Base::Lane Lane;
+    static constexpr bool kMfma16 = true;
+    static constexpr int RM = 2 * TM, RN = 2 * TN;          // 16-row blocks of A and of B per wavefront
+    static constexpr int PA = (FILLS + 2) / 3, PB = (FILLS - PA + 1) / 2, PC = FILLS - PA - PB;
+    static_assert(RM % 2 == 0, "two quarters of row blocks");
+
+    struct Lane16 {
+        int a_rd, b_rd, quad, swz;
+    };
+    static __device__ __forceinline__ Lane16 make_lane16(int lane, int wave) {
+        const int wm = wave / WGN, wn = wave % WGN;
+        Lane16 l;
+        l.a_rd = (wm * WM + (lane & 15)) * ROW;
+        l.b_rd = A_BYTES + (wn * WN + (lane & 15)) * ROW;
+        l.quad = lane >> 4;
+        l.swz = (lane >> 1) & 7;
+        return l;
+    }
+
+    // fragment g of a k32 step: 0 .. RM-1 the row blocks of A, then those of B
+    template <int STEP>
+    static __device__ __forceinline__ void read_frag(frag_t (&fa)[RM], frag_t (&fb)[RN], const unsigned char* st,
+                                                     const Lane16& l, int g) {
+        const int chunk = ((4 * STEP + l.quad) ^ l.swz) << 4;
+        if (g < RM) fa[g] = *reinterpret_cast<const frag_t*>(st + l.a_rd + g * 16 * ROW + chunk);
+        else fb[g - RM] = *reinterpret_cast<const frag_t*>(st + l.b_rd + (g - RM) * 16 * ROW + chunk);
+    }
+    template <int STEP>
+    static __device__ __forceinline__ void read_step(frag_t (&fa)[RM], frag_t (&fb)[RN], const unsigned char* st,
+                                                     const Lane16& l) {
+#pragma unroll
+        for (int g = 0; g < RM + RN; ++g) read_frag<STEP>(fa, fb, st, l, g);
+    }
+
+    // One quarter: row blocks HALF * RM/2 .. of A against all column blocks, `between(g)` after MFMA g.  The MFMAs
+    // are volatile assembly, so the memory operations that `between` issues stay where the source puts them.
+    // B is the first operand: acc[i][j] holds D'[n][m] of rows m = 16 i .. and columns n = 16 j .. of the wavefront's
+    // part, lane l the four consecutive n = 4 (l / 16) + 0..3 of row m = l % 16
+    template <int HALF, typename F>
+    static __device__ __forceinline__ void quarter(f32x4_t (&acc)[RM][RN], const frag_t (&fa)[RM], const frag_t (&fb)[RN],
+                                                   F&& between) {
+#pragma unroll
+        for (int i = 0; i < RM / 2; ++i)
+#pragma unroll
+            for (int j = 0; j < RN; ++j) {
+                Mfma16<T>::run(fb[j], fa[HALF * (RM / 2) + i], acc[HALF * (RM / 2) + i][j]);
+                between(i * RN + j);
+            }
+    }
+
+    // fill f of `count` goes out after MFMA g of Q when f * Q / count == g
+    template <int FIRST, int COUNT>
+    static __device__ __forceinline__ void fill_slot(int g, int q, unsigned char* dst, const unsigned char* a_k,
+                                                     const unsigned char* b_k, const Lane& ln) {
+#pragma unroll
+        for (int f = 0; f < COUNT; ++f)
+            if (f * q / COUNT == g) dma_one<BM, NW, NV>(FIRST + f, dst, a_k, b_k, ln.voff);
+    }
+
+    static __device__ __forceinline__ void slab(f32x4_t (&acc)[RM][RN], frag_t (&fa)[2][RM], frag_t (&fb)[2][RN],
+                                                unsigned char* cur, const unsigned char* nxt,
+                                                const unsigned char* a_slab, const unsigned char* b_slab,
+                                                size_t k_refill, const Lane& ln, const Lane16& l16, int wave) {
+        constexpr int Q = RM * RN / 2;                         // MFMAs of a quarter
+        static_assert(RM + RN <= Q, "a fragment read per MFMA");
+        const unsigned char* a_k = a_slab + k_refill;
+        const unsigned char* b_k = b_slab + k_refill;
+        unsigned char* const dst = cur + wave * 1024;
+
+        quarter<0>(acc, fa[0], fb[0], [&](int g) { if (g < RM + RN) read_frag<1>(fa[1], fb[1], cur, l16, g); });
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, true));     // own reads of this stage returned
+        __builtin_amdgcn_s_barrier();                          // everyone's: the stage is free
+
+        quarter<1>(acc, fa[0], fb[0], [&](int g) { fill_slot<0, PA>(g, Q, dst, a_k, b_k, ln); });
+        quarter<0>(acc, fa[1], fb[1], [&](int g) { fill_slot<PA, PB>(g, Q, dst, a_k, b_k, ln); });
+        // own fills of slab s+1 landed (the two thirds of slab s+2 issued since may fly on)
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(PA + PB, false));
+        __builtin_amdgcn_s_barrier();
+
+        quarter<1>(acc, fa[1], fb[1], [&](int g) {
+            if (g < RM + RN) read_frag<0>(fa[0], fb[0], nxt, l16, g);
+            fill_slot<PA + PB, PC>(g, Q, dst, a_k, b_k, ln);
+        });
+    }
+
+    static __device__ __forceinline__ void main(f32x4_t (&acc)[RM][RN], const unsigned char* a_slab,
+                                                const unsigned char* b_slab, size_t row_bytes, int K,
+                                                int k_rot, int lane, int wave) {
+        unsigned char* const stage0 = Base::template stage<0>();
+        unsigned char* const stage1 = Base::template stage<1>();
+        const Lane ln = Base::make_lane(row_bytes, lane, wave);
+        const Lane16 l16 = make_lane16(lane, wave);
+        const int k_steps = K / BK;
+        const int rot = k_rot % k_steps;
+
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(FILLS, true));       // slab 0 landed; slab 1 may fly on
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        frag_t fa[2][RM], fb[2][RN];
+        read_step<0>(fa[0], fb[0], stage0, l16);
+
+        const int pairs = k_steps >> 1;
+        for (int pr = 0; pr < pairs; ++pr) {
+            slab(acc, fa, fb, stage0, stage1, a_slab, b_slab, Base::slab_off(2 * pr + 2, rot, k_steps), ln, l16, wave);
+            slab(acc, fa, fb, stage1, stage0, a_slab, b_slab, Base::slab_off(2 * pr + 3, rot, k_steps), ln, l16, wave);
+        }
+        if (k_steps & 1)
+            slab(acc, fa, fb, stage0, stage1, a_slab, b_slab, Base::slab_off(k_steps + 1, rot, k_steps), ln, l16, wave);
+        // drain the re-fetches of the last slab before anything refills the stages
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, true));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+    }
+};
+
 // the deepest arrangement that fits next to the wave table: three stages, or the early-read form
 // (the kernel's own LDS: up to 4 KB of wave table, 32 rows x 80 bytes of C staging per wavefront)
 template <typename T, int BM, int BN, int WGM, int WGN,
@@ -547,10 +716,23 @@ struct DeepPipeSel {
 };
 template <typename T, int BM, int BN, int WGM, int WGN>
 struct DeepPipeSel<T, BM, BN, WGM, WGN, false> {
-    typedef EarlyPipe<T, BM, BN, WGM, WGN> type;
+    typedef EarlyPipe16<T, BM, BN, WGM, WGN> type;
 };
 template <typename T, int BM, int BN, int WGM, int WGN>
 using DeepPipe = typename DeepPipeSel<T, BM, BN, WGM, WGN>::type;
+
+// the same choice with the early-read form on 32x32x16 MFMAs (SYN_GEMM_MFMA_32X32)
+template <typename T, int BM, int BN, int WGM, int WGN,
+          bool THREE = (3 * (BM + BN) * 128 + WGM * WGN * 32 * 80 + 4096 <= 160 * 1024)>
+struct DeepPipe32Sel {
+    typedef SlabPipe<T, BM, BN, WGM, WGN, 3> type;
+};
+template <typename T, int BM, int BN, int WGM, int WGN>
+struct DeepPipe32Sel<T, BM, BN, WGM, WGN, false> {
+    typedef EarlyPipe<T, BM, BN, WGM, WGN> type;
+};
+template <typename T, int BM, int BN, int WGM, int WGN>
+using DeepPipe32 = typename DeepPipe32Sel<T, BM, BN, WGM, WGN>::type;
 
 // ring: four stages of 32-deep slabs.  LDS row r (64 bytes) keeps logical chunk c at physical
 // chunk c ^ ((r >> 2) & 3): 16 consecutive rows then hit 16 distinct 16-byte bank groups.
@@ -565,6 +747,7 @@ using DeepPipe = typename DeepPipeSel<T, BM, BN, WGM, WGN>::type;
 template <typename T, int BM, int BN, int WGM, int WGN>
 struct RingPipe {
     static constexpr int NW = WGM * WGN;
+    static constexpr bool kMfma16 = false;
     static constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
     static constexpr int BK = 32, ROW = BK * 2;
     static constexpr int A_BYTES = BM * ROW, STAGE = (BM + BN) * ROW;
@@ -893,13 +1076,15 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
     Pipe::prologue(panel_a(tile), panel_b(tile), row_bytes, tile.k_len, tile.k_rot, lane, wave);
 
     for (int it = 0; it < tiles_here; ++it) {
-        f32x16_t acc[TM][TN];
+        constexpr bool M16 = Pipe::kMfma16;                   // 16x16x32 MFMAs: 2 TM x 2 TN accumulators of four floats
+        constexpr int AR = M16 ? 2 * TM : TM, AC = M16 ? 2 * TN : TN, AE = M16 ? 4 : 16;
+        typename std::conditional<M16, f32x4_t, f32x16_t>::type acc[AR][AC];
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < AR; ++i)
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
+            for (int j = 0; j < AC; ++j)
 #pragma unroll
-                for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+                for (int e = 0; e < AE; ++e) acc[i][j][e] = 0.f;
 
         Pipe::main(acc, panel_a(tile), panel_b(tile), row_bytes, tile.k_len, tile.k_rot, lane, wave);
 
@@ -923,6 +1108,22 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
         // D', rows n = 8g + 4*(lane/32) + 0..3: four consecutive elements of one row of C.
         if constexpr (REMOTE) {
             // peer buffers are only 8-byte aligned: one 8-byte store (or two packed atomics) per group
+            if constexpr (M16) {
+                // lane l: row l % 16 of a 16-row block, columns 4 (l / 16) + 0..3 of a 16-column block
+                T* c_row = tile.c_tile + (size_t)(wm * WM + (lane & 15)) * tile.ldc + wn * WN + 4 * (lane >> 4);
+#pragma unroll
+                for (int i = 0; i < AR; ++i)
+#pragma unroll
+                    for (int j = 0; j < AC; ++j) {
+                        const uint2 v = pack4<T>(acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
+                        T* dst = c_row + (size_t)(16 * i) * tile.ldc + 16 * j;
+                        if (p.c_atomic) {
+                            atomic_add4<T>(dst, v);
+                        } else {
+                            *reinterpret_cast<uint2*>(dst) = v;
+                        }
+                    }
+            } else {
             T* c_row = tile.c_tile + (size_t)(wm * WM + (lane & 31)) * tile.ldc + wn * WN + 4 * (lane >> 5);
 #pragma unroll
             for (int i = 0; i < TM; ++i)
@@ -939,6 +1140,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
                             *reinterpret_cast<uint2*>(dst) = v;
                         }
                     }
+            }
         } else {
             // A store instruction of those groups would touch 32 rows with 16 bytes each, and the
             // texture path takes a cycle per cache line touched.  So a strip of 32 rows x CS_COLS
@@ -948,13 +1150,24 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
             constexpr int LPR = CS_COLS / 8;                  // lanes per row on the way out
             constexpr int RPI = 64 / LPR;                     // rows per store instruction
             unsigned char* const cs = s_cstage + wave * (32 * CS_ROW);
-            unsigned char* const cs_wr = cs + (lane & 31) * CS_ROW + 8 * (lane >> 5);
+            unsigned char* const cs_wr = M16 ? cs + (lane & 15) * CS_ROW + 8 * (lane >> 4)
+                                             : cs + (lane & 31) * CS_ROW + 8 * (lane >> 5);
             const unsigned char* const cs_rd = cs + (lane / LPR) * CS_ROW + (lane % LPR) * 16;
             T* const c_out = tile.c_tile + (size_t)(wm * WM + lane / LPR) * tile.ldc + wn * WN + (lane % LPR) * 8;
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int js = 0; js < TN; js += CS_COLS / 32) {
+                    if constexpr (M16) {
+                        // the strip's 32 rows are two 16-row blocks, its columns CS_COLS / 16 blocks of 32 bytes
+#pragma unroll
+                        for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+                            for (int jb = 0; jb < CS_COLS / 16; ++jb)
+                                *reinterpret_cast<uint2*>(cs_wr + rb * 16 * CS_ROW + jb * 32) =
+                                    pack4<T>(acc[2 * i + rb][2 * js + jb][0], acc[2 * i + rb][2 * js + jb][1],
+                                             acc[2 * i + rb][2 * js + jb][2], acc[2 * i + rb][2 * js + jb][3]);
+                    } else {
 #pragma unroll
                     for (int jj = 0; jj < CS_COLS / 32; ++jj)
 #pragma unroll
@@ -962,6 +1175,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
                             *reinterpret_cast<uint2*>(cs_wr + jj * 64 + g * 16) =
                                 pack4<T>(acc[i][js + jj][4 * g], acc[i][js + jj][4 * g + 1],
                                          acc[i][js + jj][4 * g + 2], acc[i][js + jj][4 * g + 3]);
+                    }
 #pragma unroll
                     for (int t = 0; t < 32 / RPI; ++t) {
                         const uint4 v = *reinterpret_cast<const uint4*>(cs_rd + t * RPI * CS_ROW);
@@ -1042,13 +1256,15 @@ static int dispatch_tile(const GemmParams& p, int bm, int bn, bool eight, int gr
 }
 
 template <typename T, int MODE>
-static int dispatch_pipe(const GemmParams& p, int bm, int bn, bool eight, bool ring, bool two_stage, int grid,
-                         hipStream_t stream) {
+static int dispatch_pipe(const GemmParams& p, int bm, int bn, bool eight, bool ring, bool two_stage, bool mfma32,
+                         int grid, hipStream_t stream) {
     // the remote-binding form exists for the default pipeline only
     if (MODE != kRemote) {
         if (ring) return dispatch_tile<T, RingPipe, MODE == kRemote ? kConsumer : MODE>(p, bm, bn, eight, grid, stream);
         if (two_stage) return dispatch_tile<T, PairPipe, MODE == kRemote ? kConsumer : MODE>(p, bm, bn, eight, grid, stream);
     }
+    // tiles of which three stages do not fit have two forms of the early-read pipeline
+    if (mfma32) return dispatch_tile<T, DeepPipe32, MODE>(p, bm, bn, eight, grid, stream);
     return dispatch_tile<T, DeepPipe, MODE>(p, bm, bn, eight, grid, stream);
 }
 
@@ -1125,14 +1341,15 @@ static int gemm_entry(const syn_gemm_desc* d, hipStream_t stream, int mode,
 
     const int bm = d->block_m, bn = d->block_n;
     const bool two = (d->options & SYN_GEMM_TWO_STAGE) != 0;
+    const bool m32 = (d->options & SYN_GEMM_MFMA_32X32) != 0;
     if (d->dtype == SYN_DTYPE_BF16) {
-        if (mode == kRemote) return dispatch_pipe<__bf16, kRemote>(p, bm, bn, eight, false, false, grid, stream);
-        return producer ? dispatch_pipe<__bf16, kProducer>(p, bm, bn, eight, ring, two, grid, stream)
-                        : dispatch_pipe<__bf16, kConsumer>(p, bm, bn, eight, ring, two, grid, stream);
+        if (mode == kRemote) return dispatch_pipe<__bf16, kRemote>(p, bm, bn, eight, false, false, m32, grid, stream);
+        return producer ? dispatch_pipe<__bf16, kProducer>(p, bm, bn, eight, ring, two, m32, grid, stream)
+                        : dispatch_pipe<__bf16, kConsumer>(p, bm, bn, eight, ring, two, m32, grid, stream);
     }
-    if (mode == kRemote) return dispatch_pipe<_Float16, kRemote>(p, bm, bn, eight, false, false, grid, stream);
-    return producer ? dispatch_pipe<_Float16, kProducer>(p, bm, bn, eight, ring, two, grid, stream)
-                    : dispatch_pipe<_Float16, kConsumer>(p, bm, bn, eight, ring, two, grid, stream);
+    if (mode == kRemote) return dispatch_pipe<_Float16, kRemote>(p, bm, bn, eight, false, false, m32, grid, stream);
+    return producer ? dispatch_pipe<_Float16, kProducer>(p, bm, bn, eight, ring, two, m32, grid, stream)
+                    : dispatch_pipe<_Float16, kConsumer>(p, bm, bn, eight, ring, two, m32, grid, stream);
 }
 
 // ---- the producer entry point that allocates nothing ----

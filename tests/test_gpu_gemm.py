@@ -307,6 +307,47 @@ def test_consumer_256x224_tiles(hip, dtype):
         _check_visits(log, sizes, offsets, signals, M, N, 256, 224, 8, num_sms, M * N, True)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("BM,BN,eight", [(256, 256, False), (256, 256, True), (256, 224, False), (128, 256, True),
+                                         (256, 128, True)])
+def test_both_mfma_forms_of_the_early_read_loop(hip, dtype, BM, BN, eight):
+    """Tiles whose K loop runs on two LDS stages with early reads use 16x16x32 MFMAs by default and
+    32x32x16 ones on request: both against fp32, the same visit order, and the same bits (K of one,
+    two, three and eight slabs; consumer and producer)."""
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.gemm import gemm_consumer, gemm_producer
+
+    world, rank = 2, 1
+    M, N = 1024, 2 * BN * (2 if BN < 224 else 1)
+    for K, num_sms in ((64, 5), (128, 256), (192, 3), (512, 16)):
+        a, b = _inputs(M, N, K, dtype, seed=K + BM + BN)
+        sizes, offsets, signals = _row_waves(M, N, world, rank)
+        ref = numerics.gemm_fp32(a, b)
+        ad, bd = a.cuda(), b.cuda()
+        flags = torch.ones(world, dtype=torch.int64, device="cuda")
+        tiles = (M // BM) * (N // BN)
+        results = []
+        for wide in (False, True):
+            c = torch.zeros(M, N, dtype=dtype, device="cuda")
+            log = torch.full((tiles, 4), -1, dtype=torch.int32, device="cuda")
+            gemm_consumer(ad, bd, c, flags, sizes, offsets, signals, world, num_sms, BM, BN, 64, 8, cum_tiles=M * N,
+                          visit_log=log, eight_waves=eight, mfma_32x32=wide)
+            check_status()
+            assert _max_rel_err(c, ref) <= REL_TOL, (K, wide)
+            _check_visits(log, sizes, offsets, signals, M, N, BM, BN, 8, num_sms, M * N, True)
+            results.append(c)
+            p_flags = torch.zeros(world, dtype=torch.int64, device="cuda")
+            counters = torch.zeros(world, dtype=torch.int32, device="cuda")
+            cp = torch.zeros(M, N, dtype=dtype, device="cuda")
+            gemm_producer(ad, bd, cp, p_flags, sizes, offsets, [0, 1], num_sms, BM, BN, cum_tiles=M * N,
+                          counter_buffer=counters, eight_waves=eight, mfma_32x32=wide)
+            check_status()
+            assert p_flags.tolist() == [1, 1]
+            results.append(cp)
+        for other in results[1:]:
+            assert torch.equal(results[0], other), K
+
+
 def test_launch_on_a_stream_that_is_not_current(hip):
     """`stream=` with tables given as lists and no counter buffer: the device tables and the
     zeroed counters the launcher creates must be filled on that stream, ahead of the kernel.
