@@ -322,10 +322,11 @@ def run_mfma_ceiling(device, state, launches=8):
     sink = torch.empty(256 * 256, dtype=torch.float32, device=device)
     stream = _lib.stream_handle(torch.cuda.current_stream())
     iters = 2000
-    out = {"launches": launches, "mfma": "v_mfma_f32_32x32x16_bf16, 4x4 accumulators per wavefront, 64 per round",
+    out = {"launches": launches, "mfma": "v_mfma_f32_16x16x32_bf16, 8x8 accumulators per wavefront, 128 per round (the 256x256 tile's "
+                                          "K loop); mfma_32x32x16_*: v_mfma_f32_32x32x16_bf16, 4x4 accumulators, 64 per round",
            "rounds_per_launch": iters}
     for workgroups in (256, NUM_SMS):
-        for pattern, name in ((1, "constant"), (2, "random")):
+        for pattern, name in ((5, "constant"), (6, "random"), (1, "mfma_32x32x16_constant"), (2, "mfma_32x32x16_random")):
             def probe(i):
                 _lib.check("syn_probe_mfma_rate", lib.syn_probe_mfma_rate(sink.data_ptr(), workgroups, iters, pattern, stream))
             ms = _timed(probe, launches, 3)

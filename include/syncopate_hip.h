@@ -417,7 +417,9 @@ int syn_where_async(uint32_t* out, int32_t workgroups, int32_t dwell, syn_stream
  * accumulator pattern) on register-resident operands - no LDS, no memory.  pattern 0: zero
  * operands, 1: all ones, 2: pseudo-random N(0, 0.02)-like values.  flop = workgroups * 4 * iters *
  * 64 * 32768.  sink: device float[workgroups * 256].  The rate with pattern 2 is what the matrix
- * pipes sustain under the board's power limit when operand bits toggle. */
+ * pipes sustain under the board's power limit when operand bits toggle.  pattern + 4: the same
+ * operands and flop on 128 v_mfma_f32_16x16x32_bf16 per round (8 x 8 accumulators), the form of
+ * the 256x256 tile's K loop. */
 int syn_probe_mfma_rate(float* sink, int32_t workgroups, int32_t iters, int32_t pattern,
                         syn_stream_t stream);
 

@@ -6,13 +6,16 @@
 // straight into LDS stages with global_load_lds_dwordx4 (16 bytes per lane, no register
 // staging); a wavefront-wide load fills 1 KB of consecutive LDS rows, and which 16-byte
 // chunk of its row a lane fetches is XOR-swizzled with the row number so that the 128-bit
-// fragment reads of v_mfma_f32_32x32x16 are bank-conflict free over the 64 LDS banks.
+// fragment reads of the MFMAs (16 rows x four chunks for v_mfma_f32_16x16x32, 32 rows x two for
+// v_mfma_f32_32x32x16) are bank-conflict free over the 64 LDS banks.
 //
 // Pipelines over the same tile walk (the 64 fills of a 256x256 slab take the texture path of a
 // compute unit about 1400 cycles, a k16 step of MFMAs 512: where the fills are issued matters):
 //   early  2 stages of 64-deep slabs, the LDS reads of a slab bunched at its start so that its
-//          stage is refilled during three of the four k16 steps; the default for the tiles of
-//          which only two stages fit the 160 KB of LDS (256x256, 256x224).
+//          stage is refilled during three quarters of the slab's MFMAs; the default for the tiles of
+//          which only two stages fit the 160 KB of LDS (256x256, 256x224), on 16x16x32 MFMAs
+//          (which cost less energy per product on a power-limited board; same bits) or, as an
+//          option, on 32x32x16 ones.
 //   slab   3 stages of 64-deep slabs, a slab's fills spread over the four k16 steps; the default
 //          for the other tiles.  With 2 stages (an option) all fills go out in one step.
 //          Rows are whole 128-byte cache lines; any K % 64 == 0.

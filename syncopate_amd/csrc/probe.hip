@@ -1,8 +1,8 @@
-// Matrix-pipe ceiling probe for gfx950 (MI355X): a loop of nothing but the GEMM kernels' MFMA
-// (v_mfma_f32_32x32x16_bf16), in the GEMM's register pattern - a wavefront owns a 4 x 4 grid of
-// 32x32 accumulators and multiplies four A fragments with four B fragments per k16 step - with
-// every operand held in registers: no LDS, no memory.  One workgroup of four wavefronts per
-// compute unit (one per SIMD), like the 256x256 GEMM tile.
+// Matrix-pipe ceiling probe for gfx950 (MI355X): a loop of nothing but the GEMM kernels' MFMA, in the GEMM's
+// register pattern, with every operand held in registers: no LDS, no memory.  One workgroup of four wavefronts
+// per compute unit (one per SIMD), like the 256x256 GEMM tile.  Two forms: v_mfma_f32_32x32x16_bf16 (a wavefront
+// owns a 4 x 4 grid of 32x32 accumulators and multiplies four A fragments with four B fragments per k16 step) and
+// v_mfma_f32_16x16x32_bf16 (8 x 8 accumulators of 16x16, eight fragments of each operand per k32 step).
 //
 // The operands of consecutive k16 steps rotate over SETS register-resident fragment sets filled
 // with a pattern: zeros, one constant, or N(0, 0.02)-like pseudo-random bf16 values.  The rate
@@ -76,6 +76,41 @@ __global__ void __launch_bounds__(256) mfma_rate_kernel(float* sink, int iters, 
     sink[me] = total;
 }
 
+// the same on 16x16x32 MFMAs: 128 per round, the flop of 64 of the larger ones.  The accumulators are named as AGPR
+// tuples in inline assembly, as in the GEMM's K loop.
+__global__ void __launch_bounds__(256) mfma16_rate_kernel(float* sink, int iters, int pattern) {
+    typedef float f32x4_probe_t __attribute__((ext_vector_type(4)));
+    f32x4_probe_t acc[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[i][j] = f32x4_probe_t{0.f, 0.f, 0.f, 0.f};
+    bf16x8_t fa[2][8], fb[2][8];
+    const unsigned me = blockIdx.x * 256u + threadIdx.x;
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            fa[s][i] = probe_fragment(pattern, (me * 2u + s) * 16u + i);
+            fb[s][i] = probe_fragment(pattern, (me * 2u + s) * 16u + 8u + i);
+        }
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(fb[s][j]), "v"(fa[s][i]));
+    }
+    float total = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) total += acc[i][j][0] + acc[i][j][3];
+    sink[me] = total;
+}
+
 // HBM read ceiling probe: `STREAMS` read streams `stride_vecs` 16-byte groups apart, walked in the chunked
 // reduce's access pattern - 256 lanes, four groups per lane and pass, every load of a pass issued
 // before the first is used, non-temporal - with an exclusive-or in place of the adds and no result
@@ -129,8 +164,12 @@ extern "C" int syn_probe_read_streams(const void* base, int64_t stream_bytes, in
 extern "C" int syn_probe_mfma_rate(float* sink, int32_t workgroups, int32_t iters, int32_t pattern,
                                    syn_stream_t stream) {
     using namespace syn;
-    if (sink == nullptr || workgroups <= 0 || iters <= 0 || pattern < 0 || pattern > 2) return SYN_EINVAL;
-    hipLaunchKernelGGL(mfma_rate_kernel, dim3(workgroups), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), sink,
-                       iters, pattern);
+    if (sink == nullptr || workgroups <= 0 || iters <= 0 || pattern < 0 || (pattern & 3) > 2 || pattern > 6) return SYN_EINVAL;
+    if (pattern & 4)
+        hipLaunchKernelGGL(mfma16_rate_kernel, dim3(workgroups), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
+                           sink, iters, pattern & 3);
+    else
+        hipLaunchKernelGGL(mfma_rate_kernel, dim3(workgroups), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), sink,
+                           iters, pattern);
     return (int)hipGetLastError();
 }

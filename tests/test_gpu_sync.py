@@ -70,16 +70,21 @@ def test_mfma_rate_probe_runs_and_rejects_bad_arguments(hip):
 
     sink = torch.zeros(4 * 256, dtype=torch.float32, device="cuda")
     stream = _lib.stream_handle(torch.cuda.current_stream())
-    for pattern in (0, 1, 2):
+    for pattern in (0, 1, 2, 4, 5, 6):
+        sink.fill_(-1.0)
         _lib.check("syn_probe_mfma_rate", hip.syn_probe_mfma_rate(sink.data_ptr(), 4, 3, pattern, stream))
         torch.cuda.synchronize()
         assert torch.isfinite(sink).all()
-        if pattern == 0:
+        if pattern in (0, 4):
             assert (sink == 0).all()
         if pattern == 1:
             # 3 rounds x 4 fragment sets x 16 (k) ones per accumulator element, two elements of 16 accumulators summed
             assert (sink == 3 * 4 * 16 * 2 * 16).all()
-    assert hip.syn_probe_mfma_rate(sink.data_ptr(), 4, 3, 3, stream) == _lib.SYN_EINVAL
+        if pattern == 5:
+            # the 16x16x32 form: 3 rounds x 2 fragment sets x 32 (k), two elements of 64 accumulators summed
+            assert (sink == 3 * 2 * 32 * 2 * 64).all()
+    for bad in (3, 7, 8, -1):
+        assert hip.syn_probe_mfma_rate(sink.data_ptr(), 4, 3, bad, stream) == _lib.SYN_EINVAL
     assert hip.syn_probe_mfma_rate(None, 4, 3, 0, stream) == _lib.SYN_EINVAL
     assert hip.syn_probe_mfma_rate(sink.data_ptr(), 0, 3, 0, stream) == _lib.SYN_EINVAL
 
