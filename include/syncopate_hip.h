@@ -59,11 +59,9 @@ extern "C" {
                                        the fp32 sums are then taken in rotated order)      */
 #define SYN_GEMM_TWO_STAGE 16u      /* two LDS stages even for tiles of which three fit (every
                                        shape but 256x256): one slab in flight instead of two */
-#define SYN_GEMM_MFMA_32X32 32u     /* tiles whose K loop runs on two LDS stages with early reads
-                                       (256x256, 256x224, the eight-wavefront forms): 32x32x16
-                                       MFMAs instead of the default 16x16x32, which cost less
-                                       energy per product on a power-limited board; same results
-                                       bit for bit                                           */
+#define SYN_GEMM_MFMA_32X32 32u     /* the default K loops on 32x32x16 MFMAs instead of 16x16x32
+                                       ones, which cost less energy per product on a power-limited
+                                       board; same results bit for bit                       */
 
 typedef void* syn_stream_t;        /* hipStream_t */
 

@@ -710,12 +710,111 @@ struct EarlyPipe16 : SlabPipe<T, BM, BN, WGM, WGN, 2> {
     }
 };
 
+// slab16: the three-stage pipeline on 16x16x32 MFMAs, for the tiles of which three stages fit.  The quarters and the
+// fragment reads are those of early16; a slab's fills go out in four parts as in `slab`: part 0 of slab s+3 in quarter 3
+// of slab s (into the stage slab s has left), parts 1-3 in quarters 0-2 of slab s+1; two slabs in flight.
+//     quarter 0: MFMAs (k32 step 0) | read the fragments of step 1 | part 1 of slab s+2
+//     quarter 1: MFMAs (step 0)     | part 2
+//     quarter 2: MFMAs (step 1)     | part 3;  wait: own fills of slab s+1 landed, own reads returned;  barrier
+//     quarter 3: MFMAs (step 1)     | read step 0 of slab s+1 | part 0 of slab s+3 into this slab's stage
+template <typename T, int BM, int BN, int WGM, int WGN>
+struct SlabPipe16 : SlabPipe<T, BM, BN, WGM, WGN, 3> {
+    typedef SlabPipe<T, BM, BN, WGM, WGN, 3> Base;
+    typedef EarlyPipe16<T, BM, BN, WGM, WGN> Ops;            // fragment reads and quarters
+    using Base::TM;
+    using Base::TN;
+    using Base::FILLS;
+    using Base::NW;
+    using Base::NV;
+    using Base::BK;
+    typedef typename Base::frag_t frag_t;
+    typedef typename Base::Lane Lane;
+    typedef typename Ops::Lane16 Lane16;
+    static constexpr bool kMfma16 = true;
+    static constexpr int RM = 2 * TM, RN = 2 * TN;
+
+    template <int PART>
+    static __device__ __forceinline__ void fill_slot(int g, int q, unsigned char* stage_wave, const unsigned char* a_k,
+                                                     const unsigned char* b_k, const Lane& ln) {
+        constexpr int first = Base::part_begin(PART), count = Base::part_begin(PART + 1) - first;
+#pragma unroll
+        for (int f = 0; f < count; ++f)
+            if (f * q / count == g) dma_one<BM, NW, NV>(first + f, stage_wave, a_k, b_k, ln.voff);
+    }
+
+    static __device__ __forceinline__ void slab(f32x4_t (&acc)[RM][RN], frag_t (&fa)[2][RM], frag_t (&fb)[2][RN],
+                                                unsigned char* cur, const unsigned char* nxt, unsigned char* prv,
+                                                const unsigned char* a_slab, const unsigned char* b_slab,
+                                                size_t k_refill, size_t k_prev, const Lane& ln, const Lane16& l16,
+                                                int wave) {
+        constexpr int Q = RM * RN / 2;                         // MFMAs of a quarter
+        static_assert(RM + RN <= Q, "a fragment read per MFMA");
+        unsigned char* const prv_w = prv + wave * 1024;
+        const unsigned char* a_p = a_slab + k_prev;
+        const unsigned char* b_p = b_slab + k_prev;
+
+        Ops::template quarter<0>(acc, fa[0], fb[0], [&](int g) {
+            if (g < RM + RN) Ops::template read_frag<1>(fa[1], fb[1], cur, l16, g);
+            fill_slot<1>(g, Q, prv_w, a_p, b_p, ln);
+        });
+        Ops::template quarter<1>(acc, fa[0], fb[0], [&](int g) { fill_slot<2>(g, Q, prv_w, a_p, b_p, ln); });
+        Ops::template quarter<0>(acc, fa[1], fb[1], [&](int g) { fill_slot<3>(g, Q, prv_w, a_p, b_p, ln); });
+        // own fills of slab s+1 landed (those of slab s+2, all younger, may fly on)
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(FILLS, true));
+        __builtin_amdgcn_s_barrier();
+
+        Ops::template quarter<1>(acc, fa[1], fb[1], [&](int g) {
+            if (g < RM + RN) Ops::template read_frag<0>(fa[0], fb[0], nxt, l16, g);
+            fill_slot<0>(g, Q, cur + wave * 1024, a_slab + k_refill, b_slab + k_refill, ln);
+        });
+    }
+
+    static __device__ __forceinline__ void main(f32x4_t (&acc)[RM][RN], const unsigned char* a_slab,
+                                                const unsigned char* b_slab, size_t row_bytes, int K,
+                                                int k_rot, int lane, int wave) {
+        unsigned char* const stage0 = Base::template stage<0>();
+        unsigned char* const stage1 = Base::template stage<1>();
+        unsigned char* const stage2 = Base::template stage<2>();
+        const Lane ln = Base::make_lane(row_bytes, lane, wave);
+        const Lane16 l16 = Ops::make_lane16(lane, wave);
+        const int k_steps = K / BK;
+        const int rot = k_rot % k_steps;
+
+        // slab 0 landed; slab 1 and part 0 of slab 2 may fly on
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(FILLS + Base::template part_size<0>(), true));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        frag_t fa[2][RM], fb[2][RN];
+        Ops::template read_step<0>(fa[0], fb[0], stage0, l16);
+
+        auto run = [&](unsigned char* cur, const unsigned char* nxt, unsigned char* prv, int s) {
+            slab(acc, fa, fb, cur, nxt, prv, a_slab, b_slab, Base::slab_off(s + 3, rot, k_steps),
+                 Base::slab_off(s + 2, rot, k_steps), ln, l16, wave);
+        };
+        const int triples = k_steps / 3, rest = k_steps - 3 * triples;
+        for (int tr = 0; tr < triples; ++tr) {
+            run(stage0, stage1, stage2, 3 * tr);
+            run(stage1, stage2, stage0, 3 * tr + 1);
+            run(stage2, stage0, stage1, 3 * tr + 2);
+        }
+        if (rest >= 1) run(stage0, stage1, stage2, 3 * triples);
+        if (rest == 2) run(stage1, stage2, stage0, 3 * triples + 1);
+        // drain the re-fetches of the last slab before anything refills the stages
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, true));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+    }
+};
+
 // the deepest arrangement that fits next to the wave table: three stages, or the early-read form
 // (the kernel's own LDS: up to 4 KB of wave table, 32 rows x 80 bytes of C staging per wavefront)
 template <typename T, int BM, int BN, int WGM, int WGN,
           bool THREE = (3 * (BM + BN) * 128 + WGM * WGN * 32 * 80 + 4096 <= 160 * 1024)>
 struct DeepPipeSel {
-    typedef SlabPipe<T, BM, BN, WGM, WGN, 3> type;
+    // a wavefront part of 64 x 64 (the 128x128 tile) is 2 % faster on 32x32x16 MFMAs: eight MFMAs per quarter
+    // leave no room beside the fragment reads
+    typedef typename std::conditional<(BM / WGM) * (BN / WGN) <= 64 * 64, SlabPipe<T, BM, BN, WGM, WGN, 3>,
+                                      SlabPipe16<T, BM, BN, WGM, WGN>>::type type;
 };
 template <typename T, int BM, int BN, int WGM, int WGN>
 struct DeepPipeSel<T, BM, BN, WGM, WGN, false> {
@@ -724,7 +823,7 @@ struct DeepPipeSel<T, BM, BN, WGM, WGN, false> {
 template <typename T, int BM, int BN, int WGM, int WGN>
 using DeepPipe = typename DeepPipeSel<T, BM, BN, WGM, WGN>::type;
 
-// the same choice with the early-read form on 32x32x16 MFMAs (SYN_GEMM_MFMA_32X32)
+// the same choice on 32x32x16 MFMAs (SYN_GEMM_MFMA_32X32)
 template <typename T, int BM, int BN, int WGM, int WGN,
           bool THREE = (3 * (BM + BN) * 128 + WGM * WGN * 32 * 80 + 4096 <= 160 * 1024)>
 struct DeepPipe32Sel {

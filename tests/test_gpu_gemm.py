@@ -309,9 +309,9 @@ def test_consumer_256x224_tiles(hip, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("BM,BN,eight", [(256, 256, False), (256, 256, True), (256, 224, False), (128, 256, True),
-                                         (256, 128, True)])
-def test_both_mfma_forms_of_the_early_read_loop(hip, dtype, BM, BN, eight):
-    """Tiles whose K loop runs on two LDS stages with early reads use 16x16x32 MFMAs by default and
+                                         (256, 128, True), (128, 256, False), (256, 128, False), (128, 128, False)])
+def test_both_mfma_forms_of_the_k_loop(hip, dtype, BM, BN, eight):
+    """The default K loops (two LDS stages with early reads, or three stages) run on 16x16x32 MFMAs and on
     32x32x16 ones on request: both against fp32, the same visit order, and the same bits (K of one,
     two, three and eight slabs; consumer and producer)."""
     from syncopate_amd.computation._launch import check_status
