@@ -523,10 +523,28 @@ def run_gemm_rs(device, steps, warmup, gated=True):
         acc = acc + dst[(RANK + i) % world][sample]
     reduce_matches = torch.equal(out[sample], acc)
     pushed = all(torch.equal(ctx.comm_buffers["dst"][p][RANK], src[p * rows:(p + 1) * rows]) for p in (1, 4, 7))
+    # The reference's other GEMM+RS form (template_rs.py:212-290, tests/test_gemm_rs_direct_reduce.py): no pushes and no
+    # reduce kernel - the GEMM's epilogue adds every tile into its owner's (1024, 8192) result with packed 16-bit
+    # float atomics.  This rank's launch alone, all 256 compute units (the peers' atomics would arrive beside it);
+    # the owners' buffers are eight local allocations here and keep accumulating over the timed launches.
+    from syncopate_amd.computation.gemm import gemm_rs_producer_persistent
+    owners = [torch.zeros(rows, n, dtype=torch.bfloat16, device=device) for _ in range(world)]
+    targets = [row // rows for row, _ in tables.block_offsets]
+    def direct():
+        gemm_rs_producer_persistent(a, b, owners, sizes, offsets, targets, world, world, 256, 256, 256, BK, GROUP_M)
+    direct()
+    torch.cuda.synchronize()
+    direct_matches = True
+    for p in (1, 4, RANK):
+        ref = a[p * rows + 5:p * rows + 6].float() @ b.float().t()
+        direct_matches = direct_matches and bool(((owners[p][5:6].float() - ref).abs().max() / ref.abs().max()) < 1e-2)
+    direct_ms = _timed(lambda i: direct(), steps, max(3, warmup // 4))
+    check_status()
     return {"launches": steps, "producer_ms": producer_ms, "producer_ms_without_xcd_remap": no_remap_ms,
             "flop": 2.0 * m * n * k, "fused_step_ms": fused_ms,
             "fused_step_ms_by_programs": {str(k_): v for k_, v in fused_by_programs.items()},
-            "reduce_matches": bool(reduce_matches), "pushed_chunks_match": bool(pushed)}
+            "reduce_matches": bool(reduce_matches), "pushed_chunks_match": bool(pushed),
+            "direct_reduce_form_ms": direct_ms, "direct_reduce_form_matches": direct_matches}
 
 
 # ------------------------------------------------------------------------------------ attention
@@ -1016,6 +1034,9 @@ def main():
                 "fused_step_ms_by_programs": rs["fused_step_ms_by_programs"],
                 "fused_step_tflops": rs["flop"] / (rs["fused_step_ms"] * 1e-3) / 1e12,
                 "fused_step_over_producer_pct": 100.0 * (rs["fused_step_ms"] - rs["producer_ms"]) / rs["producer_ms"],
+                "direct_reduce_form_ms": rs["direct_reduce_form_ms"],
+                "direct_reduce_form_tflops": rs["flop"] / (rs["direct_reduce_form_ms"] * 1e-3) / 1e12,
+                "direct_reduce_form_matches": rs["direct_reduce_form_matches"],
                 "reduce_matches": rs["reduce_matches"],
                 "pushed_chunks_match": rs["pushed_chunks_match"],
             })

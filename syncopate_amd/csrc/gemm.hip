@@ -958,24 +958,22 @@ struct RingPipe {
 
 // ------------------------------------------------------------------ kernel
 
-// C += v (four consecutive elements) with two packed 16-bit atomic adds
+// C += v (two consecutive elements) with one packed 16-bit atomic add
 template <typename T>
-__device__ __forceinline__ void atomic_add4(T* dst, uint2 v);
+__device__ __forceinline__ void atomic_add2(T* dst, unsigned v);
 
 template <>
-__device__ __forceinline__ void atomic_add4<__bf16>(__bf16* dst, uint2 v) {
+__device__ __forceinline__ void atomic_add2<__bf16>(__bf16* dst, unsigned v) {
     typedef __bf16 v2 __attribute__((ext_vector_type(2)));
     typedef __attribute__((address_space(1))) v2* gptr;
-    __builtin_amdgcn_global_atomic_fadd_v2bf16((gptr)dst, __builtin_bit_cast(v2, v.x));
-    __builtin_amdgcn_global_atomic_fadd_v2bf16((gptr)(dst + 2), __builtin_bit_cast(v2, v.y));
+    __builtin_amdgcn_global_atomic_fadd_v2bf16((gptr)dst, __builtin_bit_cast(v2, v));
 }
 
 template <>
-__device__ __forceinline__ void atomic_add4<_Float16>(_Float16* dst, uint2 v) {
+__device__ __forceinline__ void atomic_add2<_Float16>(_Float16* dst, unsigned v) {
     typedef _Float16 v2 __attribute__((ext_vector_type(2)));
     typedef __attribute__((address_space(1))) v2* gptr;
-    __builtin_amdgcn_global_atomic_fadd_v2f16((gptr)dst, __builtin_bit_cast(v2, v.x));
-    __builtin_amdgcn_global_atomic_fadd_v2f16((gptr)(dst + 2), __builtin_bit_cast(v2, v.y));
+    __builtin_amdgcn_global_atomic_fadd_v2f16((gptr)dst, __builtin_bit_cast(v2, v));
 }
 
 // 16 bytes stored through the XCD's L2 to memory (the agent-scope form of a store: what a relaxed
@@ -1000,9 +998,9 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
     __shared__ int s_spun;
     // C staging of the epilogue: 32 rows x CS_COLS columns per wavefront, 64 columns where LDS allows
     constexpr int NWAVES = WGM * WGN;
-    constexpr int CS_COLS = (!REMOTE && (BN / WGN / 32) % 2 == 0 &&
+    constexpr int CS_COLS = ((BN / WGN / 32) % 2 == 0 &&
                              Pipe::LDS_BYTES + NWAVES * 32 * (64 * 2 + 16) + 4096 <= 160 * 1024) ? 64 : 32;
-    __shared__ __attribute__((aligned(16))) unsigned char s_cstage[REMOTE ? 16 : NWAVES * 32 * (CS_COLS * 2 + 16)];
+    __shared__ __attribute__((aligned(16))) unsigned char s_cstage[NWAVES * 32 * (CS_COLS * 2 + 16)];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -1208,42 +1206,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
 
         // Epilogue.  With B as the first MFMA operand a lane holds, for column m = lane % 32 of
         // D', rows n = 8g + 4*(lane/32) + 0..3: four consecutive elements of one row of C.
-        if constexpr (REMOTE) {
-            // peer buffers are only 8-byte aligned: one 8-byte store (or two packed atomics) per group
-            if constexpr (M16) {
-                // lane l: row l % 16 of a 16-row block, columns 4 (l / 16) + 0..3 of a 16-column block
-                T* c_row = tile.c_tile + (size_t)(wm * WM + (lane & 15)) * tile.ldc + wn * WN + 4 * (lane >> 4);
-#pragma unroll
-                for (int i = 0; i < AR; ++i)
-#pragma unroll
-                    for (int j = 0; j < AC; ++j) {
-                        const uint2 v = pack4<T>(acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
-                        T* dst = c_row + (size_t)(16 * i) * tile.ldc + 16 * j;
-                        if (p.c_atomic) {
-                            atomic_add4<T>(dst, v);
-                        } else {
-                            *reinterpret_cast<uint2*>(dst) = v;
-                        }
-                    }
-            } else {
-            T* c_row = tile.c_tile + (size_t)(wm * WM + (lane & 31)) * tile.ldc + wn * WN + 4 * (lane >> 5);
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        const uint2 v = pack4<T>(acc[i][j][4 * g], acc[i][j][4 * g + 1],
-                                                 acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
-                        T* dst = c_row + (size_t)(32 * i) * tile.ldc + 32 * j + 8 * g;
-                        if (p.c_atomic) {
-                            atomic_add4<T>(dst, v);
-                        } else {
-                            *reinterpret_cast<uint2*>(dst) = v;
-                        }
-                    }
-            }
-        } else {
+        {
             // A store instruction of those groups would touch 32 rows with 16 bytes each, and the
             // texture path takes a cycle per cache line touched.  So a strip of 32 rows x CS_COLS
             // columns goes through a private piece of LDS (rows padded by 16 bytes) and leaves as
@@ -1278,11 +1241,34 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
                                 pack4<T>(acc[i][js + jj][4 * g], acc[i][js + jj][4 * g + 1],
                                          acc[i][js + jj][4 * g + 2], acc[i][js + jj][4 * g + 3]);
                     }
+                    if constexpr (REMOTE) {
+                        if (p.c_atomic) {
+                            // one packed atomic per lane, the lanes of an instruction side by side in a row: every
+                            // instruction adds into whole cache lines.  (Issued as 8 or 16 bytes per lane - four
+                            // instructions that each touch a quarter of every line - the atomic form of the
+                            // 8192 x 8192 x 3584 GEMM took 0.82-0.86 ms against 0.33 for the stores.)
+                            constexpr int DPR = CS_COLS / 2;          // dwords of a staged row
+                            constexpr int RPA = 64 / DPR;             // rows per atomic instruction
+#pragma unroll
+                            for (int t = 0; t < 32 / RPA; ++t) {
+                                const int row = t * RPA + lane / DPR;
+                                const unsigned v = *reinterpret_cast<const unsigned*>(cs + row * CS_ROW + (lane % DPR) * 4);
+                                atomic_add2<T>(tile.c_tile + (size_t)(wm * WM + 32 * i + row) * tile.ldc + wn * WN + 32 * js +
+                                                   (lane % DPR) * 2, v);
+                            }
+                            continue;
+                        }
+                    }
 #pragma unroll
                     for (int t = 0; t < 32 / RPI; ++t) {
                         const uint4 v = *reinterpret_cast<const uint4*>(cs_rd + t * RPI * CS_ROW);
                         T* dst = c_out + (size_t)(32 * i + t * RPI) * tile.ldc + 32 * js;
-                        if (PRODUCER) {
+                        if constexpr (REMOTE) {
+                            // peer buffers are only 8-byte aligned: two 8-byte stores per lane
+                            const uint2 lo = {v.x, v.y}, hi = {v.z, v.w};
+                            *reinterpret_cast<uint2*>(dst) = lo;
+                            *reinterpret_cast<uint2*>(dst + 4) = hi;
+                        } else if (PRODUCER) {
                             // written through the XCD's L2: the release below then has nothing
                             // of this tile left to write back
                             store16_write_through(dst, v);
