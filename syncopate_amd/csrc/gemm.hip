@@ -98,7 +98,11 @@ struct Mfma16;
 template <>
 struct Mfma16<__bf16> {
     // inline assembly: the accumulator is named as an AGPR tuple that is read and written in place (through the
-    // builtin the register allocator moves accumulators between the two register files inside the K loop)
+    // builtin the register allocator moves accumulators between the two register files inside the K loop).
+    // The compiler does not know that the statement is an MFMA and adds no wait states behind it: the pipelines
+    // touch an accumulator once per quarter (at least eight MFMAs apart), and vector instructions read the
+    // accumulators only after the K loop's closing wait and barrier, and write them (zeros) only before its
+    // opening ones.
     static __device__ __forceinline__ void run(bf16x8_t a, bf16x8_t b, f32x4_t& c) {
         asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
     }
