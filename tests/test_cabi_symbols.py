@@ -38,6 +38,22 @@ def test_header_and_library_agree(lib):
     assert lib.syn_version() >= 100
 
 
+def test_constants_match_the_header():
+    """Every numeric SYN_* constant the Python binding mirrors has the header's value, and every option
+    bit of the header is mirrored (a launcher that set a stale bit would silently run another form)."""
+    from syncopate_amd import _lib
+
+    text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    header = {name: int(value.rstrip("uU"), 0)
+              for name, value in re.findall(r"#define\s+(SYN_[A-Z0-9_]+)\s+\(?(-?(?:0x[0-9a-fA-F]+|\d+)[uU]?)\)?\s*$", text, flags=re.M)}
+    assert len(header) > 20
+    mirrored = {name: getattr(_lib, name) for name in header if hasattr(_lib, name)}
+    assert mirrored == {name: header[name] for name in mirrored}
+    for name in header:
+        if name.startswith(("SYN_GEMM_", "SYN_ATTN_", "SYN_E")):
+            assert name in mirrored, name
+
+
 def test_struct_layouts_match_the_header():
     """Field order and count of the ctypes mirrors follow the header's structs."""
     from syncopate_amd import _lib
