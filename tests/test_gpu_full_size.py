@@ -45,21 +45,24 @@ def test_ag_gemm_8192x8192x3584(hip):
     ref = a[sample].float() @ b.float().t()
 
     outputs = []
-    # (BM, BN, programs, 8 wavefronts, ring pipeline)
-    for BM, BN, num_sms, eight, ring in [(256, 256, 224, False, False), (256, 256, 256, True, False),
-                                         (256, 256, 131, True, True), (128, 256, 224, False, False)]:
+    # (BM, BN, programs, 8 wavefronts, ring pipeline, 32x32x16 MFMAs in the default pipelines)
+    for BM, BN, num_sms, eight, ring, wide in [(256, 256, 224, False, False, False), (256, 256, 256, True, False, False),
+                                               (256, 256, 131, True, True, False), (256, 256, 224, False, False, True),
+                                               (128, 256, 224, False, False, False), (128, 256, 97, False, False, True)]:
         c = torch.zeros(M, N, dtype=torch.bfloat16, device="cuda")
         log = torch.full(((M // BM) * (N // BN), 4), -1, dtype=torch.int32, device="cuda")
         gemm_consumer(a, b, c, flags, sizes, offsets, signals, world, num_sms, BM, BN, 64, 8,
-                      cum_tiles=M * N, visit_log=log, xcd_remap=False, eight_waves=eight, ring_pipe=ring)
+                      cum_tiles=M * N, visit_log=log, xcd_remap=False, eight_waves=eight, ring_pipe=ring, mfma_32x32=wide)
         check_status()
         assert _rel(c[sample], ref) <= REL_TOL
         _check_visit_log(log, sizes, offsets, signals, M, N, BM, BN, num_sms)
         outputs.append((BM, BN, c))
-    # one tile shape -> one order of the fp32 sums, whatever the grid, workgroup shape or pipeline
-    same_tile = [c for BM, BN, c in outputs if (BM, BN) == (256, 256)]
-    for other in same_tile[1:]:
-        assert torch.equal(same_tile[0], other)
+    # one tile shape -> one order of the fp32 sums, whatever the grid, workgroup shape, pipeline or MFMA form
+    for shape in ((256, 256), (128, 256)):
+        same_tile = [c for BM, BN, c in outputs if (BM, BN) == shape]
+        assert len(same_tile) >= 2
+        for other in same_tile[1:]:
+            assert torch.equal(same_tile[0], other)
     # other tile shapes rotate the K walk differently: equal to rounding
     assert _rel(outputs[-1][2], outputs[0][2]) <= 2e-2
 
