@@ -44,7 +44,9 @@ extern "C" {
 #define SYN_STATUS_BAD_PAIRING 2    /* SYN_ATTN_PAIR_Q_BLOCKS on a wave with an odd number of q blocks:
                                        [1]=wave index, [2]=program id, [3]=q blocks of the wave */
 #define SYN_STATUS_BAD_CHAIN 3      /* SYN_ATTN_CHAIN_Q_BLOCKS: [1]=wave whose (z, h, q) ranges differ from wave 0's, or 0
-                                       and [3]=pairs per wave when the grid is not that many programs */
+                                       and [3]=pairs per wave when the grid is not that many programs;
+                                       SYN_ATTN_WORK_LIST: [1]=wave, [3]=tile id of an entry that cannot continue
+                                       its segment (other q blocks, or nothing below the diagonal) */
 
 /* gemm option bits */
 #define SYN_GEMM_XCD_REMAP 1u       /* permute hardware workgroup ids so that consecutive
@@ -62,6 +64,17 @@ extern "C" {
 #define SYN_GEMM_MFMA_32X32 32u     /* the default K loops on 32x32x16 MFMAs instead of 16x16x32
                                        ones, which cost less energy per product on a power-limited
                                        board; same results bit for bit                       */
+
+#define SYN_GEMM_ACQUIRE_ALWAYS 64u  /* take the agent-scope acquire fence behind EVERY flag wait.  Without
+                                       it a program whose flag is already up when it looks reads the chunk
+                                       without a fence (the fence empties the XCD's L2 of the operand panels
+                                       its neighbours reuse), which is safe only if the caller sees to it that
+                                       (1) nothing on the device - an earlier iteration still running, another
+                                       kernel - reads the gathered buffer between the start of this kernel and
+                                       a chunk's flag, and (2) no flag word is raised more than once during
+                                       the launch.  The reference always acquires (dl.wait,
+                                       gemm/template.py:92-97,121-128); callers that cannot promise (1) and (2)
+                                       set this bit. */
 
 typedef void* syn_stream_t;        /* hipStream_t */
 
@@ -129,6 +142,10 @@ int syn_gemm_producer(const syn_gemm_desc* desc, syn_stream_t stream);
  * call outside stream capture.
  */
 int syn_gemm_producer_static(const syn_gemm_desc* desc, syn_stream_t stream);
+
+/* Test hook of syn_gemm_producer_static: copies the first `count` words of the current device's static counter
+ * array to host memory (a synchronous hipMemcpy; allocates nothing).  No counterpart in the reference. */
+int syn_gemm_static_counters_peek(int32_t* host_out, int32_t count);
 
 /*
  * A GEMM in both roles: the producer above that, before the first tile of a wave, also waits
@@ -288,14 +305,16 @@ typedef struct syn_attn_desc {
                                        (consumer_signal_ptr / consumer_signal_offsets beside the
                                        producer's, transformer.py:1077-1123,
                                        tests/test_all2all_attn_all2all.py:192-210)                    */
+    const int32_t* work_list;       /* with SYN_ATTN_WORK_LIST, else NULL: device int32: num_programs + 1 entry
+                                       offsets, then the entries (see SYN_ATTN_WORK_LIST)              */
 } syn_attn_desc;
 
 /* syn_attn_desc.options: one workgroup of eight wavefronts takes two consecutive q blocks (tiles
  * 2i and 2i + 1) and runs them half a kv block apart, so that the softmax of one overlaps the
  * matrix products of the other and both read K and V from the same LDS blocks.  No counterpart in
  * the reference (one program per tile there); results and merge protocol are the same.  The
- * caller vouches that every wave holds an even number of q blocks; not with `causal` or
- * `counters`. */
+ * caller vouches that every wave holds an even number of q blocks (and, with `causal`, that every wave's q and
+ * kv ranges begin at even blocks); not with `counters`. */
 #define SYN_ATTN_PAIR_Q_BLOCKS 1u
 /* workgroup b takes tile (b % 8) * (grid / 8) + b / 8 instead of tile b: the workgroups of one XCD
  * then work on consecutive tiles - the q blocks of one head - and that head's K and V pass through
@@ -310,6 +329,36 @@ typedef struct syn_attn_desc {
  * neither `lock` nor a stored partial result is read.  A table or grid that is not of that shape
  * ends the launch with SYN_STATUS_BAD_CHAIN in `status`.  No counterpart in the reference. */
 #define SYN_ATTN_CHAIN_Q_BLOCKS 4u
+/* the attention kernels' form of SYN_GEMM_ACQUIRE_ALWAYS: the acquire fence behind every flag wait, for callers
+ * who cannot promise that K and V are not read on the device before a chunk's flag and that no flag is raised
+ * twice during the launch (the reference always acquires: dl.wait, attn/template.py:90-96) */
+#define SYN_ATTN_ACQUIRE_ALWAYS 8u
+/* with SYN_ATTN_PAIR_Q_BLOCKS: `work_list` says which program visits which tiles, in which order.  The tile ->
+ * (wave, z, h, q block, kv range) mapping stays the table's (and the reference's); what the list chooses is the
+ * part the reference leaves to the hardware scheduler - which program runs a tile - and, beyond it, that a
+ * program which visits the same pair of q blocks several times in a row keeps the running maxima, sums and output
+ * in registers from one visit to the next (a SEGMENT) and merges into the output once.  Layout: words
+ * [0, num_programs] are offsets into the entries that follow at work_list + num_programs + 1; program b makes the
+ * visits entries[offset[b]] .. entries[offset[b + 1] - 1] in that order.  An entry is a pair index (tiles 2 * pair and
+ * 2 * pair + 1 of the table) in SYN_ATTN_WORK_PAIR_MASK, SYN_ATTN_WORK_CONTINUES when the next entry visits the same
+ * (z, h, q blocks) and continues the segment, and - on a segment's first entry - SYN_ATTN_WORK_SOLE_WRITER when no
+ * other segment of the launch writes these q blocks (they are then stored without taking their locks).  Every
+ * visit of the table appears exactly once; under `causal` the visits that lie wholly above the diagonal may be
+ * left out (they add nothing; listed, they are logged in the visit log and skipped) and must not be part of a
+ * segment, and every wave's q and kv ranges begin at even blocks.  num_programs is the grid.  Flags are waited for
+ * visit by visit, in list order: a program's entries should follow the order in which their waves arrive.
+ * syn_attn_check_work_list (HOST pointers) checks all of this; the kernel trusts a list that passed and ends a
+ * launch whose list breaks a segment's promise with SYN_STATUS_BAD_CHAIN.  No counterpart in the reference. */
+#define SYN_ATTN_WORK_LIST 16u
+#define SYN_ATTN_WORK_PAIR_MASK 0x0fffffff
+#define SYN_ATTN_WORK_CONTINUES 0x10000000
+#define SYN_ATTN_WORK_SOLE_WRITER 0x20000000
+int syn_attn_check_work_list(const int32_t* wave_offsets, const int32_t* wave_sizes, const int32_t* cum_wave_sizes,
+                             int32_t num_waves, int32_t block_m, int32_t block_n, int32_t causal,
+                             const int32_t* work_list, int64_t work_list_words, int32_t num_programs,
+                             int32_t require_masked_visits);
+/* syn_attn_fwd trusts its tables: pass them through syn_attn_check_waves first.  (A real wave behind a zero
+ * row of padding, which the check rejects, would never be selected by the wave lookup.) */
 int syn_attn_fwd(const syn_attn_desc* desc, syn_stream_t stream);
 
 /* Host-only check of an attention wave table (HOST pointers). */

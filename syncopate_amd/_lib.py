@@ -33,9 +33,15 @@ SYN_GEMM_RING_PIPE = 4
 SYN_GEMM_NO_K_STAGGER = 8
 SYN_GEMM_TWO_STAGE = 16
 SYN_GEMM_MFMA_32X32 = 32
+SYN_GEMM_ACQUIRE_ALWAYS = 64
 SYN_ATTN_PAIR_Q_BLOCKS = 1
 SYN_ATTN_XCD_REMAP = 2
 SYN_ATTN_CHAIN_Q_BLOCKS = 4
+SYN_ATTN_ACQUIRE_ALWAYS = 8
+SYN_ATTN_WORK_LIST = 16
+SYN_ATTN_WORK_PAIR_MASK = 0x0FFFFFFF
+SYN_ATTN_WORK_CONTINUES = 0x10000000
+SYN_ATTN_WORK_SOLE_WRITER = 0x20000000
 SYN_STATUS_BAD_PAIRING = 2
 SYN_STATUS_BAD_CHAIN = 3
 SYN_BOX_COPY, SYN_BOX_ADD_ATOMIC, SYN_BOX_ADD_EXCLUSIVE = range(3)
@@ -137,6 +143,7 @@ class AttnDesc(ctypes.Structure):
         ("options", c_int32),
         ("wait_flags", c_void_p),
         ("wait_signal_offsets", c_void_p),
+        ("work_list", c_void_p),
     ]
 
 
@@ -145,6 +152,7 @@ _SIGNATURES = {
     "syn_gemm_consumer": (c_int32, [POINTER(GemmDesc), c_void_p]),
     "syn_gemm_producer": (c_int32, [POINTER(GemmDesc), c_void_p]),
     "syn_gemm_producer_static": (c_int32, [POINTER(GemmDesc), c_void_p]),
+    "syn_gemm_static_counters_peek": (c_int32, [c_void_p, c_int32]),
     "syn_gemm_consumer_producer": (c_int32, [POINTER(GemmDesc), c_void_p, c_void_p, c_void_p]),
     "syn_gemm_remote_binding": (c_int32, [POINTER(GemmDesc), POINTER(GemmRemote), c_void_p]),
     "syn_gemm_check_waves": (
@@ -162,6 +170,10 @@ _SIGNATURES = {
         [c_void_p, c_int64, c_void_p, c_void_p, c_int32, c_int32, c_int64, c_int64, c_int32, c_int32, c_void_p],
     ),
     "syn_attn_fwd": (c_int32, [POINTER(AttnDesc), c_void_p]),
+    "syn_attn_check_work_list": (
+        c_int32,
+        [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_void_p, c_int64, c_int32, c_int32],
+    ),
     "syn_attn_check_waves": (
         c_int32,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32,

@@ -37,6 +37,7 @@ from .operations import (
     SMCopyOp,
     WaitIntraNodeSignal,
 )
+from ...computation._launch import trust_flags
 from .cu_partition import split_device_cu_mask
 from .persistent_copy import persistent_copy_last_contig
 from .streams import pick_side_streams
@@ -91,7 +92,7 @@ class CommContext:
         # lead_copy_blocks workgroups if given, and the rest).  No kernel starts or ends on the device while
         # the consumer runs, so nothing writes back or invalidates the L2s its operands are cached in.
         self.list_blocks = int(list_blocks)
-        self._list_records: Dict[tuple, torch.Tensor] = {}
+        self._list_records: Dict[tuple, tuple] = {}
         self._list_tickets: Dict[int, torch.Tensor] = {}
         self._lib = _lib.load()
         world = info.local_world_size
@@ -113,6 +114,11 @@ class CommContext:
              flag_arrays(info.compute_signal_num))
             for _ in range(flag_sets)
         ]
+        # this executor's copies are the only writers of its buffers and its flags are reset between iterations:
+        # kernels that wait on these arrays may skip the acquire fence when a flag is already up
+        for flag_set in self._flag_sets:
+            for group in flag_set:
+                trust_flags(*group)
         self._cur_set = 0
         self._stale_set: Optional[int] = None
         self._stale_whole_mesh = False
@@ -253,8 +259,13 @@ class CommContext:
         world = self.info.local_world_size
         if len(ops) == 0 or len(ops) % 2:
             return False
+        # the records hold addresses and sizes: they are good for exactly this op list, these buffers and this delay
         key = (lane, self._cur_set, neglect_local)
-        records = self._list_records.get(key)
+        stamp = (tuple(map(id, ops)), self.link_delay_us,
+                 tuple(t.data_ptr() for name in sorted(self.comm_buffers) for t in self.comm_buffers[name]),
+                 tuple(t.data_ptr() for t in self.recv_signal_bufs))
+        cached = self._list_records.get(key)
+        records = cached[1] if cached is not None and cached[0] == stamp else None
         if records is None:
             rows = []
             for i in range(0, len(ops), 2):
@@ -277,7 +288,7 @@ class CommContext:
                 delay = self.link_delay_us * 100 if (self.link_delay_us and op.src_rank != op.dst_rank) else 0
                 rows.append([dst_ptr, src_ptr, 0 if skip else op.size // 16, flags.data_ptr() + 8 * flag_op.offset, 1, delay])
             records = torch.tensor(rows, dtype=torch.int64, device=self.device)
-            self._list_records[key] = records
+            self._list_records[key] = (stamp, records)
         tickets = self._list_tickets.get(lane)
         if tickets is None or tickets.numel() < records.shape[0]:
             tickets = torch.zeros(records.shape[0], dtype=torch.int32, device=self.device)

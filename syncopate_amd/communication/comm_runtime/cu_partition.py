@@ -11,6 +11,7 @@ engines, and the kernels on the remaining ones still see eight equal XCDs.
 
 from __future__ import annotations
 
+import atexit
 import ctypes
 from typing import List, Tuple
 
@@ -20,7 +21,23 @@ from ... import _lib
 
 XCDS = 8
 
-_live_streams: List[Tuple[int, torch.cuda.Stream]] = []     # masked streams live as long as the process
+# Masked streams are handed out for the life of the process (a CommContext keeps using them), and are destroyed
+# before the interpreter goes: a process that ended with such streams still alive has crashed inside the HIP
+# runtime's own exit handlers.  `atexit` runs this hook while torch and the library are still loaded.
+_live_streams: List[Tuple[int, torch.cuda.Stream]] = []
+_exit_hook_registered = False
+
+
+def destroy_masked_streams() -> None:
+    """Wait for and destroy every stream `masked_stream` created; they must not be used afterwards."""
+    lib = _lib.load()
+    while _live_streams:
+        handle, stream = _live_streams.pop()
+        try:
+            stream.synchronize()
+        except Exception:       # a device already in an error state: still hand the stream back
+            pass
+        lib.syn_stream_destroy(ctypes.c_void_p(handle))
 
 
 def cu_mask_words(first: int, count: int, total: int) -> List[int]:
@@ -53,6 +70,10 @@ def masked_stream(words: List[int], device: torch.device) -> torch.cuda.Stream:
                    lib.syn_stream_create_cu_mask(arr, len(words), ctypes.byref(handle)))
     stream = torch.cuda.ExternalStream(handle.value, device=device)
     _live_streams.append((handle.value, stream))
+    global _exit_hook_registered
+    if not _exit_hook_registered:
+        atexit.register(destroy_masked_streams)
+        _exit_hook_registered = True
     return stream
 
 

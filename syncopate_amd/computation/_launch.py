@@ -154,6 +154,26 @@ def remember_note(tensors: Sequence[torch.Tensor], slot: str, value) -> None:
     )
 
 
+# Flag arrays whose owner promises what the kernels' fast flag wait needs (include/syncopate_hip.h,
+# SYN_GEMM_ACQUIRE_ALWAYS): nothing on the device reads the gathered buffer between the start of a consumer
+# kernel and a chunk's flag, and no flag word is raised twice during a launch.  CommContext registers the arrays
+# it allocates (its copies are the only writers of its buffers, its flags are reset between iterations); a
+# launch on any other flag tensor takes the acquire fence behind every flag wait, like the reference.
+_trusted_flags: "weakref.WeakValueDictionary[int, torch.Tensor]" = weakref.WeakValueDictionary()
+
+
+def trust_flags(*tensors: torch.Tensor) -> None:
+    """Declare that the caller upholds the precondition above for these flag arrays (the tensor objects given,
+    not views of them made later)."""
+    for t in tensors:
+        _trusted_flags[id(t)] = t
+
+
+def acquire_always(signal_buffer: torch.Tensor) -> bool:
+    """Whether a launch that waits on `signal_buffer` must fence behind every flag wait."""
+    return _trusted_flags.get(id(signal_buffer)) is not signal_buffer
+
+
 def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
     return None if t is None else t.data_ptr()
 

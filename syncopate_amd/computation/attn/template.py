@@ -27,6 +27,7 @@ import torch
 
 from ... import _lib
 from .._launch import (
+    acquire_always,
     recall_note,
     remember_note,
     TableLike,
@@ -41,9 +42,13 @@ from .._launch import (
     status_words,
 )
 
+from .work_plan import WorkPlan, plan_attention_work
+
 BLOCK_M = 128
 BLOCK_N = 128
 DEFAULT_SPIN_TIMEOUT_US = 2_000_000
+# longest segment of an automatic plan, in visits (see work_plan.plan_attention_work)
+DEFAULT_PLAN_MAX_VISITS = 2
 
 
 @launches_on_stream
@@ -70,6 +75,7 @@ def attention_forward(
     pair_q_blocks: bool = False,
     xcd_remap: bool = False,
     chain_q_blocks: bool = False,
+    work_plan: Optional[WorkPlan] = None,
     form: str = "explicit",
     out: Optional[torch.Tensor] = None,
     return_lse: bool = False,
@@ -106,6 +112,10 @@ def attention_forward(
     behind its flag) and writes every q block once, without locks or merges.  Programs, tiles and
     their order are those of the persistent launch with that `num_programs`.  A ValueError for
     tables of another shape.
+    `work_plan` (an extension, with `pair_q_blocks`; `plan_attention_work` makes one): which program visits which
+    tiles, in which order, and which consecutive visits to the same q blocks are one segment whose sums stay in
+    registers (include/syncopate_hip.h, SYN_ATTN_WORK_LIST).  `num_programs` is the plan's.  The tile -> work
+    mapping is the tables'; the visit log shows on which program each tile ran.
     `form="auto"` (what `attention()` passes): where none of the three options above, `causal`, `counter_ptr` or
     `visit_log` is given, the launcher reads the tables and takes the fastest form they allow - two q blocks per
     workgroup with the XCD remap where every wave holds an even number of q blocks, chained where the waves
@@ -148,14 +158,42 @@ def attention_forward(
     tables = (wave_offsets, wave_sizes, cum_wave_sizes, signal_offsets)   # the caller's objects
     caller_owned = all(isinstance(t, torch.Tensor) and t.is_cuda
                        for t in (wave_offsets, wave_sizes, cum_wave_sizes, signal_offsets))
-    if pair_q_blocks and (causal or counter_ptr is not None):
-        raise ValueError("pair_q_blocks goes with neither causal nor counter_ptr")
+    if pair_q_blocks and counter_ptr is not None:
+        raise ValueError("pair_q_blocks does not go with counter_ptr")
     if chain_q_blocks and not pair_q_blocks:
         raise ValueError("chain_q_blocks goes with pair_q_blocks")
+    if chain_q_blocks and causal:
+        raise ValueError("chain_q_blocks does not go with causal: plan the visits with plan_attention_work")
+    if work_plan is not None and (not pair_q_blocks or chain_q_blocks):
+        raise ValueError("work_plan goes with pair_q_blocks and without chain_q_blocks")
     num_programs = int(num_programs)
+    if work_plan is not None:
+        if num_programs not in (0, work_plan.num_programs):
+            raise ValueError(f"the work plan is for {work_plan.num_programs} programs")
+        num_programs = work_plan.num_programs
     host_tables = None
     if form not in ("explicit", "auto"):
         raise ValueError("form must be 'explicit' or 'auto'")
+    if form == "auto" and causal and not (pair_q_blocks or chain_q_blocks or xcd_remap or counter_ptr is not None
+                                          or consumer_signal_ptr is not None or visit_log is not None
+                                          or work_plan is not None):
+        # under a causal mask the visits differ in cost and many cost nothing: a planned launch of one program per
+        # compute unit where the tables pair up, the one-tile-per-program kernel where they do not
+        units = num_programs or torch.cuda.get_device_properties(dev).multi_processor_count
+        plan = recall_note(tables, f"causal work plan {units}") if caller_owned else None
+        if plan is None:
+            host_tables = (host_copy(offs), host_copy(sizes), host_copy(cums), host_copy(sigs))
+            try:
+                plan = plan_attention_work(host_tables[0][:num_waves].tolist(), host_tables[1][:num_waves].tolist(),
+                                           host_tables[2][:num_waves].tolist(), causal=True, num_programs=units,
+                                           max_visits=DEFAULT_PLAN_MAX_VISITS)
+            except ValueError:
+                plan = False
+            if caller_owned:
+                remember_note(tables, f"causal work plan {units}", plan)
+        if plan:
+            pair_q_blocks = xcd_remap = True
+            work_plan, num_programs = plan, plan.num_programs
     if form == "auto" and not (pair_q_blocks or chain_q_blocks or xcd_remap or causal or counter_ptr is not None
                                or consumer_signal_ptr is not None or visit_log is not None):
         choice = recall_note(tables, "attention form") if caller_owned else None
@@ -179,8 +217,8 @@ def attention_forward(
     if chain_q_blocks and num_programs <= 0 and caller_owned:
         # filled in by an earlier call on these tables; `already_checked` below vouches for it
         num_programs = recall_note(tables, "chain programs") or 0
-    params = (num_waves, Z, H, Sq, Skv, cum_tiles, flags.numel(), bool(pair_q_blocks),
-              num_programs if chain_q_blocks else None)
+    params = (num_waves, Z, H, Sq, Skv, cum_tiles, flags.numel(), bool(pair_q_blocks), bool(causal),
+              None if work_plan is None else id(work_plan), num_programs if chain_q_blocks else None)
     if cum_tiles is None or (chain_q_blocks and num_programs <= 0) or \
             not (caller_owned and already_checked(tables, params)):
         ho, hs, hc, hg = host_tables or (host_copy(offs), host_copy(sizes), host_copy(cums), host_copy(sigs))
@@ -188,6 +226,17 @@ def attention_forward(
             cum_tiles = int(hc[:num_waves].max().item())
         if pair_q_blocks and any(int(hs[i, 2]) % (2 * BLOCK_M) for i in range(num_waves) if int(hc[i]) > 0):
             raise ValueError("pair_q_blocks needs an even number of q blocks in every wave")
+        if pair_q_blocks and causal and any(int(ho[i, 2]) % (2 * BLOCK_M) or int(ho[i, 3]) % (2 * BLOCK_N)
+                                            for i in range(num_waves) if int(hc[i]) > 0):
+            raise ValueError("pair_q_blocks with causal needs q and kv ranges that begin at even blocks")
+        if work_plan is not None:
+            words = torch.tensor(work_plan.words, dtype=torch.int32)
+            _lib.check(
+                "syn_attn_check_work_list",
+                lib.syn_attn_check_work_list(host_ptr(ho), host_ptr(hs), host_ptr(hc), num_waves, BLOCK_M, BLOCK_N,
+                                             1 if causal else 0, host_ptr(words), words.numel(),
+                                             work_plan.num_programs, 1 if visit_log is not None and causal else 0),
+            )
         if chain_q_blocks:
             real = [i for i in range(num_waves) if int(hc[i]) > 0]
             if not real or any(ho[i, :3].tolist() != ho[real[0], :3].tolist() or
@@ -254,13 +303,31 @@ def attention_forward(
         q_strides=strides(q), k_strides=strides(k), v_strides=strides(v), o_strides=strides(o),
         counters=None if counter_ptr is None else counter_ptr.data_ptr(),
         options=(_lib.SYN_ATTN_PAIR_Q_BLOCKS if pair_q_blocks else 0) | (_lib.SYN_ATTN_XCD_REMAP if xcd_remap else 0)
-        | (_lib.SYN_ATTN_CHAIN_Q_BLOCKS if chain_q_blocks else 0),
+        | (_lib.SYN_ATTN_CHAIN_Q_BLOCKS if chain_q_blocks else 0) | (_lib.SYN_ATTN_WORK_LIST if work_plan is not None else 0)
+        | (_lib.SYN_ATTN_ACQUIRE_ALWAYS
+           if acquire_always(consumer_signal_ptr if consumer_signal_ptr is not None else signal_ptr) else 0),
         wait_flags=None if wait_flags is None else wait_flags.data_ptr(),
         wait_signal_offsets=None if wait_sigs is None else wait_sigs.data_ptr(),
+        work_list=None if work_plan is None else _device_words(work_plan, dev).data_ptr(),
     )
     with torch.cuda.device(dev):
         _lib.check("syn_attn_fwd", lib.syn_attn_fwd(ctypes.byref(desc), _lib.stream_handle(stream)))
     return (o, lse) if return_lse else o
+
+
+# a plan's words on a device, kept with the plan object
+_plan_words: Dict[tuple, tuple] = {}
+
+
+def _device_words(plan: WorkPlan, dev: torch.device) -> torch.Tensor:
+    key = (id(plan), dev.index)
+    entry = _plan_words.get(key)
+    if entry is None or entry[0] is not plan:
+        if len(_plan_words) > 256:
+            _plan_words.clear()
+        entry = (plan, torch.tensor(plan.words, dtype=torch.int32, device=dev))
+        _plan_words[key] = entry
+    return entry[1]
 
 
 def attention(q, k, v, sm_scale, wave_dicts: Dict, BLOCK_M=128, BLOCK_N=128, NUM_BUFFERS=2,

@@ -27,6 +27,7 @@ from .._launch import (
     host_copy,
     host_ptr,
     launches_on_stream,
+    acquire_always,
     remember_checked,
     require_cuda,
     status_words,
@@ -155,7 +156,9 @@ def _launch(
         spin_timeout_us=int(spin_timeout_us),
         options=(_lib.SYN_GEMM_XCD_REMAP if xcd_remap else 0) | (_lib.SYN_GEMM_EIGHT_WAVES if eight_waves else 0)
         | (_lib.SYN_GEMM_RING_PIPE if ring_pipe else 0) | (0 if k_stagger else _lib.SYN_GEMM_NO_K_STAGGER)
-        | (_lib.SYN_GEMM_TWO_STAGE if two_stage else 0) | (_lib.SYN_GEMM_MFMA_32X32 if mfma_32x32 else 0),
+        | (_lib.SYN_GEMM_TWO_STAGE if two_stage else 0) | (_lib.SYN_GEMM_MFMA_32X32 if mfma_32x32 else 0)
+        | (_lib.SYN_GEMM_ACQUIRE_ALWAYS
+           if acquire_always(wait_signal_buffer if wait_signal_buffer is not None else signal_buffer) else 0),
     )
     with torch.cuda.device(dev):
         if wait_flags is not None:

@@ -25,7 +25,7 @@ from typing import Optional, Sequence
 import torch
 
 from ... import _lib
-from .._launch import (TableLike, as_device_table, host_copy, host_ptr, launches_on_stream, require_cuda,
+from .._launch import (TableLike, acquire_always, as_device_table, host_copy, host_ptr, launches_on_stream, require_cuda,
                        status_words)
 
 _pointer_tables: dict = {}
@@ -195,7 +195,8 @@ def gemm_remote(
         status=status_words(dev).data_ptr(), num_waves=num_waves, M=M, N=N, K=K,
         dtype=_lib.dtype_code(b.dtype), block_m=BLOCK_SIZE_M, block_n=BLOCK_SIZE_N, block_k=BLOCK_SIZE_K,
         group_m=GROUP_SIZE_M, num_sms=num_gemm_sms, cum_tiles=int(cum_tiles), spin_timeout_us=0,
-        options=(_lib.SYN_GEMM_XCD_REMAP if xcd_remap else 0) | (_lib.SYN_GEMM_EIGHT_WAVES if eight_waves else 0),
+        options=(_lib.SYN_GEMM_XCD_REMAP if xcd_remap else 0) | (_lib.SYN_GEMM_EIGHT_WAVES if eight_waves else 0)
+        | (_lib.SYN_GEMM_ACQUIRE_ALWAYS if signal_ptr is not None and acquire_always(signal_ptr) else 0),
     )
     with torch.cuda.device(dev):
         _lib.check("syn_gemm_remote_binding",

@@ -24,7 +24,10 @@
 // wavefront is never held at the vector-memory queue.
 // The kernel stays under 256 registers and 80 KB of LDS, so two workgroups share a compute
 // unit and one's exponentials overlap the other's matrix work.
+#include <array>
+#include <map>
 #include <type_traits>
+#include <vector>
 
 #include "common.h"
 
@@ -56,6 +59,8 @@ struct AttnParams {
     int32_t causal;
     int32_t num_tiles;
     int32_t xcd_remap;    // workgroups of one XCD take consecutive tiles (see logical_program_id)
+    int32_t acquire_always;   // SYN_ATTN_ACQUIRE_ALWAYS: fence behind every flag wait, not only behind a spin
+    const int32_t* work_list; // SYN_ATTN_WORK_LIST: [grid + 1] entry offsets, then the entries
     float qk_scale;       // sm_scale * 1.44269504 (template.py:178-179)
     // element strides {batch, head, row}
     int64_t q_st[3], k_st[3], v_st[3], o_st[3];
@@ -113,6 +118,15 @@ __device__ __forceinline__ void store_f32_through(float* ptr, float value) {
     __hip_atomic_store(reinterpret_cast<uint32_t*>(ptr), __builtin_bit_cast(uint32_t, value), __ATOMIC_RELAXED,
                        __HIP_MEMORY_SCOPE_AGENT);
 }
+
+// The hand-over of a q block's lock.  What orders it in hardware: every lane's stores of O and lse are
+// write-through stores whose acknowledgement (s_waitcnt vmcnt(0)) means they have reached memory, the
+// barrier collects all lanes, and thread 0's `first` store is acknowledged the same way before the lock word
+// goes out; the next holder reads past its L2.  These two fences add nothing to that on this part (at
+// workgroup scope they write back and invalidate nothing): they tell the COMPILER that the relaxed atomics
+// around them may not change places.
+__device__ __forceinline__ void lock_release_fence() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup"); }
+__device__ __forceinline__ void lock_taken_fence() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup"); }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
@@ -353,8 +367,9 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
             // Nothing reads a chunk's lines before its flag is up, so this XCD's L2 cannot hold a stale one
             // (it was emptied when the kernel began); the fence - it drops every clean line of the L2, the K
             // and V blocks other workgroups are about to reuse among them - is kept for the workgroup that
-            // really had to wait.
-            if (s_spun) acquire_fence_agent();
+            // really had to wait.  (The caller's part: nothing on the device reads a chunk before its flag during
+            // the launch and no flag is raised twice; SYN_ATTN_ACQUIRE_ALWAYS otherwise.)
+            if (s_spun || p.acquire_always) acquire_fence_agent();
             if (s_abort) return;
         }
 
@@ -559,6 +574,7 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
                 report_status(p.status, SYN_STATUS_SPIN_TIMEOUT, w, (int)blockIdx.x, -2);
                 s_abort = 1;
             }
+            lock_taken_fence();
         }
         __syncthreads();
         if (s_abort) return;
@@ -574,8 +590,10 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
         __builtin_amdgcn_s_waitcnt(attn_vmcnt(0));
         __syncthreads();
         if (tid == 0) {
+            lock_release_fence();
             __hip_atomic_store(p.first + lock_idx, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __builtin_amdgcn_s_waitcnt(attn_vmcnt(0));
+            lock_release_fence();
             __hip_atomic_store(p.lock + lock_idx, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             count_tile();
         }
@@ -615,15 +633,24 @@ __device__ __forceinline__ void dma_kv_block8(unsigned char* lds, const unsigned
 }
 
 //
-// kChain (SYN_ATTN_CHAIN_Q_BLOCKS): every wave lists the same (z, h, q) ranges and there are as many
-// programs as a wave has pairs, so program b's tiles are pair b of wave 0, of wave 1, ...: the
-// same two q blocks against one kv range after the other.  The walk over kv blocks then simply
-// continues into the next wave's range (after that wave's flag), the running maxima, sums and
-// output stay in registers, and the q blocks are written once, at the end, without locks.
-template <typename T, bool kChain>
+// The visits of a program come in SEGMENTS: one or more visits to the same pair of q blocks, walked as one run of
+// kv blocks with the running maxima, sums and output in registers, and written (or merged) once, at the end.
+//   kPairTiles       a segment is one visit; pair b, b + grid, ... of the table; merged under the q blocks' locks.
+//   kPairChainWaves  (SYN_ATTN_CHAIN_Q_BLOCKS) every wave lists the same (z, h, q) ranges and there are as many
+//                    programs as a wave has pairs: program b's segment is pair b of wave 0, of wave 1, ...; each
+//                    wave's kv range behind that wave's flag; the q blocks are written once, without locks.
+//   kPairWorkList    (SYN_ATTN_WORK_LIST) the caller's list says which visits a program makes, in which order, which
+//                    of them continue a segment, and whether a segment is the only one that writes its q blocks.
+// CAUSAL: kv blocks above a q block's diagonal contribute nothing - a visit ends at the diagonal of its higher q
+// block, the lower q block sits the last block out, and each masks its own diagonal block.
+constexpr int kPairTiles = 0, kPairChainWaves = 1, kPairWorkList = 2;
+constexpr int32_t kWorkPairMask = SYN_ATTN_WORK_PAIR_MASK;
+
+template <typename T, int MODE, bool CAUSAL>
 __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnParams p) {
     typedef typename AttnMfma<T>::frag_t frag_t;
     typedef T vec4_t __attribute__((ext_vector_type(4)));
+    static_assert(!(CAUSAL && MODE == kPairChainWaves), "the waves of a causal table do not share their kv extent");
 
     __shared__ __attribute__((aligned(1024))) unsigned char k_lds[2 * kBlockBytes];
     __shared__ __attribute__((aligned(1024))) unsigned char v_lds[2 * kBlockBytes];
@@ -655,9 +682,9 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
 #pragma unroll
     for (int i = 0; i < 4; ++i)
         v_rd[i] = v_row * kRowBytes + ((((4 * i + (v_col_bytes >> 4)) ^ v_swz) << 4) | (v_col_bytes & 15));
-    int k_chunk[8];
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) k_chunk[ks] = ((2 * ks + half) ^ (r & 15)) << 4;
+    // logical chunk 2 ks + half of row r sits at physical chunk (2 ks + half) ^ (r & 15) = 2 ks ^ (half ^ (r & 15)): one
+    // register, and an exclusive-or with a constant per step (see `scores`)
+    const int k_swz = (half ^ (r & 15)) << 4;
 
     const T* __restrict__ Q = reinterpret_cast<const T*>(p.q);
     const unsigned char* __restrict__ K = reinterpret_cast<const unsigned char*>(p.k);
@@ -665,29 +692,70 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
     T* __restrict__ O = reinterpret_cast<T*>(p.o);
 
     const int pairs_per_wave = p.cum_wave_sizes[0] / kBlockM / 2;
-    const int num_pairs = kChain ? pairs_per_wave : p.num_tiles / 2;
-    if (kChain && (int)gridDim.x != pairs_per_wave) {
+    const int num_pairs = MODE == kPairChainWaves ? pairs_per_wave : p.num_tiles / 2;
+    if (MODE == kPairChainWaves && (int)gridDim.x != pairs_per_wave) {
         if (tid == 0) report_status(p.status, SYN_STATUS_BAD_CHAIN, 0, (int)blockIdx.x, pairs_per_wave);
         return;
     }
-    const int first_pair = logical_program_id((int)blockIdx.x, (int)gridDim.x, p.xcd_remap != 0);
-    for (int pair = first_pair; pair < num_pairs; pair += gridDim.x) {
-        // ---- tile id -> wave -> (z, h, q block, kv range); the two tiles of a pair differ in the q block only ----
-        const int tile_id = 2 * pair + grp;
+    const int program = logical_program_id((int)blockIdx.x, (int)gridDim.x, p.xcd_remap != 0);
+
+    // where the program stands: the next pair of the table (kPairTiles, kPairChainWaves) or the entry of its list
+    int pair = program;
+    int e = 0, e_end = 0;
+    const int32_t* entries = nullptr;
+    if constexpr (MODE == kPairWorkList) {
+        e = __builtin_amdgcn_readfirstlane(p.work_list[program]);
+        e_end = __builtin_amdgcn_readfirstlane(p.work_list[program + 1]);
+        entries = p.work_list + gridDim.x + 1;
+    }
+    auto advance = [&]() __attribute__((always_inline)) {
+        if constexpr (MODE == kPairWorkList) ++e;
+        else pair += gridDim.x;
+    };
+    auto pending = [&]() __attribute__((always_inline)) { return MODE == kPairWorkList ? e < e_end : pair < num_pairs; };
+
+    // wait for flag `sg` of the wave `wv` that is being entered; false when the wait gave up
+    auto wait_for_flag = [&](const int sg, const int wv) __attribute__((always_inline)) -> bool {
+        if (tid == 0) {
+            s_spun = __hip_atomic_load(p.flags + sg, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 1ull;
+            if (s_spun && !spin_until_equal(p.flags + sg, 1ull, p.timeout_ticks)) {
+                report_status(p.status, SYN_STATUS_SPIN_TIMEOUT, wv, (int)blockIdx.x, sg);
+                s_abort = 1;
+            }
+        }
+        __syncthreads();
+        // (both words are the same for every lane: read as scalars, so that what depends on them - whether the
+        // walk goes on - stays wavefront-uniform for the compiler too)
+        if (__builtin_amdgcn_readfirstlane(s_spun) || p.acquire_always) acquire_fence_agent();       // see attn_fwd_kernel
+        const bool ok = __builtin_amdgcn_readfirstlane(s_abort) == 0;
+        __syncthreads();       // s_spun may be written again only when everyone has read it
+        return ok;
+    };
+
+    for (; pending(); advance()) {
+        // ---- the segment's first visit: tile id -> wave -> (z, h, q block, kv range); the two tiles of a pair
+        //      differ in the q block only ----
+        int entry = 0;
+        if constexpr (MODE == kPairWorkList) entry = __builtin_amdgcn_readfirstlane(entries[e]);
+        const int pair_id = MODE == kPairWorkList ? (entry & kWorkPairMask) : pair;
+        const bool sole_writer = MODE == kPairChainWaves || (MODE == kPairWorkList && (entry & SYN_ATTN_WORK_SOLE_WRITER));
+        const int tile_id = 2 * pair_id + grp;
         const int w = find_wave(p.cum_wave_sizes, p.num_waves, kBlockM, tile_id, lane);
         if (w >= p.num_waves) return;
         const int prev = w == 0 ? 0 : p.cum_wave_sizes[w - 1] / kBlockM;
         const int t = tile_id - prev;
         const int size_h = p.wave_sizes[w * 4 + 1];
         const int nq = p.wave_sizes[w * 4 + 2] / kBlockM;
-        const int nkv = p.wave_sizes[w * 4 + 3] / kBlockN;
         const int z = t / (nq * size_h) + p.wave_offsets[w * 4 + 0];
         const int h = (t / nq) % size_h + p.wave_offsets[w * 4 + 1];
         const int qb = t % nq + p.wave_offsets[w * 4 + 2] / kBlockM;
         const int kv_lo = p.wave_offsets[w * 4 + 3] / kBlockN;
+        const int kv_len = p.wave_sizes[w * 4 + 3] / kBlockN;
         const int sig = p.signal_offsets[w];
-        if ((nq & 1) || (prev & 1)) {
-            // the caller promised an even number of q blocks per wave; leave a note instead of wrong results
+        // the caller promised an even number of q blocks per wave (and, under a causal mask, q ranges and kv
+        // ranges that begin at even blocks: the lower q block of a pair then never finds its whole visit masked
+        // while the higher one has work); leave a note instead of wrong results
+        if ((nq & 1) || (prev & 1) || (CAUSAL && ((kv_lo | (qb - grp)) & 1))) {
             if (lane == 0 && wave8 == 0) report_status(p.status, SYN_STATUS_BAD_PAIRING, w, (int)blockIdx.x, nq);
             return;
         }
@@ -695,99 +763,119 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
         if (p.visit_log != nullptr && lane == 0 && wave == 0) {
             int4* rec = reinterpret_cast<int4*>(p.visit_log) + 2 * (size_t)tile_id;
             rec[0] = make_int4(w, z, h, qb);
-            rec[1] = make_int4(kv_lo, kv_lo + nkv, sig, (int)blockIdx.x);
+            rec[1] = make_int4(kv_lo, kv_lo + kv_len, sig, (int)blockIdx.x);
         }
 
-        if (sig >= 0) {
-            if (tid == 0) {
-                s_spun = __hip_atomic_load(p.flags + sig, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 1ull;
-                if (s_spun && !spin_until_equal(p.flags + sig, 1ull, p.timeout_ticks)) {
-                    report_status(p.status, SYN_STATUS_SPIN_TIMEOUT, w, (int)blockIdx.x, sig);
-                    s_abort = 1;
-                }
-            }
-            __syncthreads();
-            if (s_spun) acquire_fence_agent();       // see attn_fwd_kernel
-            if (s_abort) return;
-        }
+        // kv blocks the pair walks in this visit: under a causal mask, up to the diagonal of its higher q block
+        const int diag_hi = qb | 1;                     // the higher q block of the pair
+        const int nkv = CAUSAL ? min(kv_len, diag_hi + 1 - kv_lo) : kv_len;
+        if (CAUSAL && nkv <= 0) continue;               // wholly above the diagonal: visited, nothing to add
+
+        if (sig >= 0 && !wait_for_flag(sig, w)) return;
 
         const size_t head = (size_t)z * p.H + h;
         const int q_row = qb * kBlockM + wave * 32 + r;
         const T* q_src = Q + z * p.q_st[0] + h * p.q_st[1] + q_row * p.q_st[2] + 8 * half;
-        const unsigned char* k_base = K + (z * p.k_st[0] + h * p.k_st[1]) * (int64_t)sizeof(T) +
-                                      (size_t)kv_lo * kBlockN * k_pitch;
-        const unsigned char* v_base = V + (z * p.v_st[0] + h * p.v_st[1]) * (int64_t)sizeof(T) +
-                                      (size_t)kv_lo * kBlockN * v_pitch;
+        const unsigned char* const k_head = K + (z * p.k_st[0] + h * p.k_st[1]) * (int64_t)sizeof(T);
+        const unsigned char* const v_head = V + (z * p.v_st[0] + h * p.v_st[1]) * (int64_t)sizeof(T);
 
         // With the XCD remap the workgroups of an XCD work on the q blocks of one or two heads at the
-        // same time and read the same K and V: each pair starts its walk over the wave's kv blocks
+        // same time and read the same K and V: each pair starts its walk over a visit's kv blocks
         // one block after its neighbour's and wraps around, so that they ask the L2 for different
         // lines at any moment while staying within a window of blocks that the L2 holds (the sum
-        // over kv blocks is order-free up to rounding).
-        const int rot = p.xcd_remap ? (int)((unsigned)pair % (unsigned)nkv) : 0;
-        auto blk = [&](const int m) {
-            const int b = m + rot;
-            return b >= nkv ? b - nkv : b;
+        // over kv blocks is order-free up to rounding).  A visit that reaches a diagonal is walked from its
+        // first block: every row's first block then has an unmasked position, and the masked blocks come last.
+        auto rotation = [&](const int lo, const int len, const int walked) __attribute__((always_inline)) {
+            if (!p.xcd_remap || (CAUSAL && lo + len > (qb & ~1))) return 0;
+            return (int)((unsigned)pair_id % (unsigned)walked);
+        };
+        // what a kv block is to THIS group's q block: how far it lies beyond the block before the diagonal - 0 or less
+        // below the diagonal (nothing masked), 1 the diagonal block, 2 the block after it (everything masked)
+        auto beyond = [&](const int kv_block) __attribute__((always_inline)) { return kv_block - qb + 1; };
+
+        // ---- the walk: the K fills run one block ahead of the V fills; both step through the visit's blocks
+        //      (rotated) and the K walk enters the segment's next visit when its own is used up ----
+        int k_lo = kv_lo, k_nkv = nkv, k_next = 1, k_rot = rotation(kv_lo, kv_len, nkv);
+        int v_nkv = nkv, v_next = 0, v_rot = k_rot;
+        const unsigned char* k_walk = k_head + (size_t)kv_lo * kBlockN * k_pitch;
+        const unsigned char* v_walk = v_head + (size_t)kv_lo * kBlockN * v_pitch;
+        int k_wave = w;                                  // kPairChainWaves: the wave the K walk is in
+        // `beyond` of the blocks whose softmax is still to come: block n (the next one), n + 1 and n + 2
+        int m0 = CAUSAL ? beyond(kv_lo + k_rot) : 0, m1 = 0, m2 = 0;
+        // (The chained forms without a causal mask keep the masking block of `softmax`, which they never enter, and
+        // get their zeros here from behind an opaque statement: with the block in place the register allocator finds
+        // the assignment it finds for the causal forms - 237 registers, nothing spilled; without it, 256 and 53
+        // registers spilled inside the loop over kv blocks.)
+        if constexpr (!CAUSAL && MODE != kPairTiles) {
+            asm volatile("s_mov_b32 %0, 0" : "=s"(m0));
+            m2 = m0;
+        }
+
+        // the K walk enters the segment's next visit: 1 entered, 0 the segment ends here, -1 give up
+        auto enter_next_visit = [&]() __attribute__((always_inline)) -> int {
+            int wv;
+            int next_tile;
+            if constexpr (MODE == kPairTiles) {
+                return 0;
+            } else if constexpr (MODE == kPairChainWaves) {
+                if (k_wave + 1 >= p.num_waves || p.cum_wave_sizes[k_wave + 1] == 0) return 0;
+                wv = ++k_wave;
+                bool same = true;
+#pragma unroll
+                for (int a = 0; a < 3; ++a)
+                    same = same && p.wave_offsets[wv * 4 + a] == p.wave_offsets[a] && p.wave_sizes[wv * 4 + a] == p.wave_sizes[a];
+                if (!same) {
+                    if (tid == 0) report_status(p.status, SYN_STATUS_BAD_CHAIN, wv, (int)blockIdx.x, -1);
+                    return -1;
+                }
+                next_tile = tile_id + 2 * wv * pairs_per_wave;
+            } else {
+                if (!(entry & SYN_ATTN_WORK_CONTINUES) || e + 1 >= e_end) return 0;
+                ++e;
+                entry = __builtin_amdgcn_readfirstlane(entries[e]);
+                next_tile = 2 * (entry & kWorkPairMask) + grp;
+                wv = find_wave(p.cum_wave_sizes, p.num_waves, kBlockM, next_tile, lane);
+                bool same = wv < p.num_waves;
+                if (same) {
+                    const int pv = wv == 0 ? 0 : p.cum_wave_sizes[wv - 1] / kBlockM;
+                    const int tt = next_tile - pv;
+                    const int sh = p.wave_sizes[wv * 4 + 1];
+                    const int nn = p.wave_sizes[wv * 4 + 2] / kBlockM;
+                    same = !(nn & 1) && !(pv & 1) && tt / (nn * sh) + p.wave_offsets[wv * 4 + 0] == z &&
+                           (tt / nn) % sh + p.wave_offsets[wv * 4 + 1] == h &&
+                           tt % nn + p.wave_offsets[wv * 4 + 2] / kBlockM == qb;
+                }
+                if (!same) {
+                    // the entry does not continue on this segment's q blocks
+                    if (tid == 0) report_status(p.status, SYN_STATUS_BAD_CHAIN, wv, (int)blockIdx.x, next_tile);
+                    return -1;
+                }
+            }
+            const int lo = p.wave_offsets[wv * 4 + 3] / kBlockN;
+            const int len = p.wave_sizes[wv * 4 + 3] / kBlockN;
+            const int sg = p.signal_offsets[wv];
+            const int walked = CAUSAL ? min(len, diag_hi + 1 - lo) : len;
+            if (CAUSAL && (walked <= 0 || (lo & 1))) {
+                // a visit with nothing below the diagonal cannot continue a segment
+                if (tid == 0) report_status(p.status, SYN_STATUS_BAD_CHAIN, wv, (int)blockIdx.x, next_tile);
+                return -1;
+            }
+            if (p.visit_log != nullptr && lane == 0 && wave == 0) {
+                int4* rec = reinterpret_cast<int4*>(p.visit_log) + 2 * (size_t)next_tile;
+                rec[0] = make_int4(wv, z, h, qb);
+                rec[1] = make_int4(lo, lo + len, sg, (int)blockIdx.x);
+            }
+            if (sg >= 0 && !wait_for_flag(sg, wv)) return -1;
+            k_lo = lo;
+            k_nkv = walked;
+            k_rot = rotation(lo, len, walked);
+            k_next = 0;
+            k_walk = k_head + (size_t)lo * kBlockN * k_pitch;
+            return 1;
         };
 
-        // kChain: where the walk stands, for the K fills (one block ahead) and for the V fills: wave,
-        // kv blocks of it, next block, rotation and base address.  `total` counts the kv blocks of all waves.
-        int total = nkv;
-        int k_wave = 0, k_nkv = nkv, k_next = 1, k_rot = rot;
-        int v_wave = 0, v_nkv = nkv, v_next = 0, v_rot = rot;
-        const unsigned char* k_walk = k_base;
-        const unsigned char* v_walk = v_base;
-        if (kChain) {
-            for (int x = 1; x < p.num_waves && p.cum_wave_sizes[x] != 0; ++x) total += p.wave_sizes[x * 4 + 3] / kBlockN;
-        }
-        // the K fills enter the next wave: its tile is visited now - log, the (z, h, q) ranges promised to
-        // be wave 0's, its flag - and then its first K block may be asked for
-        auto enter_wave_k = [&]() -> bool {
-            ++k_wave;
-            bool same = true;
-#pragma unroll
-            for (int a = 0; a < 3; ++a)
-                same = same && p.wave_offsets[k_wave * 4 + a] == p.wave_offsets[a] && p.wave_sizes[k_wave * 4 + a] == p.wave_sizes[a];
-            if (!same) {
-                if (tid == 0) report_status(p.status, SYN_STATUS_BAD_CHAIN, k_wave, (int)blockIdx.x, -1);
-                return false;
-            }
-            k_nkv = p.wave_sizes[k_wave * 4 + 3] / kBlockN;
-            const int lo = p.wave_offsets[k_wave * 4 + 3] / kBlockN;
-            const int sg = p.signal_offsets[k_wave];
-            if (p.visit_log != nullptr && lane == 0 && wave == 0) {
-                int4* rec = reinterpret_cast<int4*>(p.visit_log) + 2 * ((size_t)tile_id + 2 * (size_t)k_wave * pairs_per_wave);
-                rec[0] = make_int4(k_wave, z, h, qb);
-                rec[1] = make_int4(lo, lo + k_nkv, sg, (int)blockIdx.x);
-            }
-            if (sg >= 0) {
-                if (tid == 0) {
-                    s_spun = __hip_atomic_load(p.flags + sg, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 1ull;
-                    if (s_spun && !spin_until_equal(p.flags + sg, 1ull, p.timeout_ticks)) {
-                        report_status(p.status, SYN_STATUS_SPIN_TIMEOUT, k_wave, (int)blockIdx.x, sg);
-                        s_abort = 1;
-                    }
-                }
-                __syncthreads();
-                if (s_spun) acquire_fence_agent();
-                if (s_abort) return false;
-                __syncthreads();       // s_spun may be written again only when everyone has read it
-            }
-            k_walk = K + (z * p.k_st[0] + h * p.k_st[1]) * (int64_t)sizeof(T) + (size_t)lo * kBlockN * k_pitch;
-            k_rot = p.xcd_remap ? (int)((unsigned)pair % (unsigned)k_nkv) : 0;
-            k_next = 0;
-            return true;
-        };
-        auto enter_wave_v = [&]() {
-            ++v_wave;
-            v_nkv = p.wave_sizes[v_wave * 4 + 3] / kBlockN;
-            v_walk = V + (z * p.v_st[0] + h * p.v_st[1]) * (int64_t)sizeof(T) +
-                     (size_t)(p.wave_offsets[v_wave * 4 + 3] / kBlockN) * kBlockN * v_pitch;
-            v_rot = p.xcd_remap ? (int)((unsigned)pair % (unsigned)v_nkv) : 0;
-            v_next = 0;
-        };
-        // every wavefront has passed the barrier that ended the previous pair: all four buffers are free
-        dma_kv_block8(k_lds, k_base + (size_t)blk(0) * kBlockN * k_pitch, k_pitch, k_fill_off, wave8);
+        // every wavefront has passed the barrier that ended the previous segment: all four buffers are free
+        dma_kv_block8(k_lds, k_walk + (size_t)k_rot * kBlockN * k_pitch, k_pitch, k_fill_off, wave8);
 
         frag_t qf[8];
 #pragma unroll
@@ -796,7 +884,7 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) o_acc[i][e] = 0.f;
+            for (int e2 = 0; e2 < 16; ++e2) o_acc[i][e2] = 0.f;
         float m_i = -INFINITY;
         float l_i = 0.f;
         f32x16_t s[4];
@@ -811,46 +899,55 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
         // slot 2m + 2; their buffers were last read in slot 2m - 1.  (Spreading the fills between the
         // products or the exponentials, or leaving them all to the group that is in its softmax,
         // measured 1-6 % slower: a wavefront stalls at every fill wherever it is placed.)
-        auto fetch = [&](const int m) -> bool {
+        // Returns 1 when K(m+1) was asked for, 0 when block m is the segment's last, -1 to give up (a flag did
+        // not come within the time limit, or the next visit is not one of this segment's: every wavefront is
+        // told so at the same fetch, and the program ends).
+        auto fetch = [&](const int m) __attribute__((always_inline)) -> int {
             __builtin_amdgcn_sched_barrier(0);
-            if constexpr (kChain) {
-                if (v_next == v_nkv) enter_wave_v();
-                int b = v_next + v_rot;
-                b = b >= v_nkv ? b - v_nkv : b;
-                dma_kv_block8(v_lds + (m & 1) * kBlockBytes, v_walk + (size_t)b * kBlockN * v_pitch, v_pitch, v_fill_off, wave8);
-                ++v_next;
-                if (m + 1 < total) {
-                    if (k_next == k_nkv && !enter_wave_k()) return false;
-                    b = k_next + k_rot;
-                    b = b >= k_nkv ? b - k_nkv : b;
-                    dma_kv_block8(k_lds + ((m + 1) & 1) * kBlockBytes, k_walk + (size_t)b * kBlockN * k_pitch, k_pitch, k_fill_off,
-                                  wave8);
-                    ++k_next;
-                }
-            } else {
-                dma_kv_block8(v_lds + (m & 1) * kBlockBytes, v_base + (size_t)blk(m) * kBlockN * v_pitch, v_pitch, v_fill_off,
+            // block m is the first of a new visit exactly when the V walk has used its visit up; the K walk
+            // entered that visit when it fetched K(m) and has not moved since
+            if (v_next == v_nkv) {
+                v_nkv = k_nkv;
+                v_rot = k_rot;
+                v_walk = v_head + (size_t)k_lo * kBlockN * v_pitch;
+                v_next = 0;
+            }
+            int b = v_next + v_rot;
+            b = b >= v_nkv ? b - v_nkv : b;
+            dma_kv_block8(v_lds + (m & 1) * kBlockBytes, v_walk + (size_t)b * kBlockN * v_pitch, v_pitch, v_fill_off, wave8);
+            ++v_next;
+            int more = 1;
+            if (k_next == k_nkv) more = enter_next_visit();
+            if (more > 0) {
+                b = k_next + k_rot;
+                b = b >= k_nkv ? b - k_nkv : b;
+                dma_kv_block8(k_lds + ((m + 1) & 1) * kBlockBytes, k_walk + (size_t)b * kBlockN * k_pitch, k_pitch, k_fill_off,
                               wave8);
-                if (m + 1 < nkv)
-                    dma_kv_block8(k_lds + ((m + 1) & 1) * kBlockBytes, k_base + (size_t)blk(m + 1) * kBlockN * k_pitch,
-                                  k_pitch, k_fill_off, wave8);
+                ++k_next;
+                if constexpr (CAUSAL) m2 = beyond(k_lo + b);
             }
             __builtin_amdgcn_sched_barrier(0);
-            return true;
+            return __builtin_amdgcn_readfirstlane(more);       // the same in every lane: a scalar for the compiler too
         };
 
         // S^T = K(n) . Q^T
-        auto scores = [&](const int n) {
+        auto scores = [&](const int n) __attribute__((always_inline)) {
             const f32x16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
             // fragments of steps ks and ks + 1 are in registers; the register a product has just
             // consumed is refilled with the fragment of step ks + 2, so a read has almost two steps
             // (256 MFMA cycles) to come back
             frag_t kf[2][4];
             const unsigned char* k_row = k_lds + (n & 1) * kBlockBytes + k_rd;
+            // (opaque to the compiler, which would otherwise carry the eight chunk offsets in eight registers around
+            // the loop over kv blocks - registers this kernel does not have)
+            int swz = k_swz;
+            asm volatile("" : "+v"(swz));
+            auto k_chunk = [&](const int ks) __attribute__((always_inline)) { return swz ^ (32 * ks); };
 #pragma unroll
             for (int b = 0; b < 2; ++b)
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
-                    kf[b][j] = *reinterpret_cast<const frag_t*>(k_row + 32 * j * kRowBytes + k_chunk[b]);
+                    kf[b][j] = *reinterpret_cast<const frag_t*>(k_row + 32 * j * kRowBytes + k_chunk(b));
             __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
 #pragma unroll
             for (int ks = 0; ks < 8; ++ks) {
@@ -858,7 +955,7 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
                 for (int j = 0; j < 4; ++j) {
                     s[j] = AttnMfma<T>::run(kf[ks & 1][j], qf[ks], ks == 0 ? zero : s[j]);
                     if (ks + 2 < 8)
-                        kf[ks & 1][j] = *reinterpret_cast<const frag_t*>(k_row + 32 * j * kRowBytes + k_chunk[ks + 2]);
+                        kf[ks & 1][j] = *reinterpret_cast<const frag_t*>(k_row + 32 * j * kRowBytes + k_chunk(ks + 2));
                 }
                 if (ks + 2 < 8) {
 #pragma unroll
@@ -872,13 +969,25 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
             }
         };
 
-        // online softmax in base 2 over the scores in s; leaves P^T in pf
-        auto softmax = [&]() {
+        // online softmax in base 2 over the scores in s; leaves P^T in pf.  `past` > 0 (CAUSAL): the block reaches
+        // the q block's diagonal (1) or lies wholly behind it (2) - positions beyond a row's own are masked.  A row
+        // has seen an unmasked position by then (a visit that reaches the diagonal is walked from its first block,
+        // which is at or below the lower q block), so its running maximum is finite and a wholly masked block adds
+        // exact zeros.
+        auto softmax = [&](const int past) __attribute__((always_inline)) {
+            if ((CAUSAL || MODE != kPairTiles) && past > 0) {
+                const int lim = wave * 32 + r - 4 * half - (past - 1) * kBlockN;     // mask where 32j + 8(e/4) + e%4 > lim
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int e2 = 0; e2 < 16; ++e2)
+                        if (32 * j + 8 * (e2 >> 2) + (e2 & 3) > lim) s[j][e2] = -INFINITY;
+            }
             float mx = -INFINITY;
 #pragma unroll
             for (int j = 0; j < 4; ++j)
 #pragma unroll
-                for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s[j][e]);
+                for (int e2 = 0; e2 < 16; ++e2) mx = fmaxf(mx, s[j][e2]);
             mx = fmaxf(mx, __shfl_xor(mx, 32));
             const float m_new = fmaxf(m_i, mx * p.qk_scale);
             const float alpha = fast_exp2(m_i - m_new);
@@ -886,23 +995,23 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
 #pragma unroll
-                    for (int e = 0; e < 16; ++e) o_acc[i][e] *= alpha;
+                    for (int e2 = 0; e2 < 16; ++e2) o_acc[i][e2] *= alpha;
             }
             float row_sum = 0.f;
 #pragma unroll
             for (int j = 0; j < 4; ++j)
 #pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    const float pe = fast_exp2(s[j][e] * p.qk_scale - m_new);
+                for (int e2 = 0; e2 < 16; ++e2) {
+                    const float pe = fast_exp2(s[j][e2] * p.qk_scale - m_new);
                     row_sum += pe;
-                    pf[2 * j + (e >> 3)][e & 7] = (T)pe;
+                    pf[2 * j + (e2 >> 3)][e2 & 7] = (T)pe;
                 }
             l_i = l_i * alpha + row_sum;
             m_i = m_new;
         };
 
         // O^T += V(n)^T . P^T
-        auto weighted_values = [&](const int n) {
+        auto weighted_values = [&](const int n) __attribute__((always_inline)) {
             typedef short s16x8_t __attribute__((ext_vector_type(8)));
             const unsigned char* v_blk = v_lds + (n & 1) * kBlockBytes;
             s16x4_t vlo[2][4], vhi[2][4];
@@ -940,16 +1049,15 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
             }
         };
 
-
         // a slot ends when every wavefront's LDS reads have returned; at the end of an odd slot the
         // blocks fetched one slot earlier have landed as well
-        auto end_even = [&]() {
+        auto end_even = [&]() __attribute__((always_inline)) {
             __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_waitcnt(0xc07f);
             __builtin_amdgcn_s_barrier();
             __builtin_amdgcn_sched_barrier(0);
         };
-        auto end_odd = [&]() {
+        auto end_odd = [&]() __attribute__((always_inline)) {
             __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_waitcnt(0x0070);
             __builtin_amdgcn_s_barrier();
@@ -958,42 +1066,50 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
 
         // the two groups run the same phases one slot apart; written out per group so that the scores
         // (group 0) or the probabilities (group 1) are the only block-sized values that live across
-        // an iteration
-        // (a fetch fails when a flag does not come within the time limit or, chained, when a wave's
-        // ranges are not wave 0's: every wavefront is told so at the same fetch, and the program ends)
+        // an iteration.  `more`: block n + 1 exists and its K block has been asked for.
+        int n = 0;
+        int more = fetch(0);                             // slot 0; m2 = mode of block 1
+        if (more < 0) return;
+        m1 = m2;
         if (grp == 0) {
-            if (!fetch(0)) return;                       // slot 0
             scores(0);
             end_even();
-            for (int n = 0; n + 1 < total; ++n) {
-                softmax();                               // slot 2n + 1
+            while (more > 0) {
+                softmax(m0);                          // slot 2n + 1
                 end_odd();
-                if (!fetch(n + 1)) return;               // slot 2n + 2
+                more = fetch(n + 1);                     // slot 2n + 2
+                if (more < 0) return;
                 weighted_values(n);
                 scores(n + 1);
                 end_even();
+                ++n;
+                m0 = m1;
+                m1 = m2;
             }
-            softmax();                                   // slot 2N - 1
+            softmax(m0);                              // slot 2N - 1
             end_odd();
-            weighted_values(total - 1);                  // slot 2N
+            weighted_values(n);                   // slot 2N
             end_even();
             end_odd();                                   // slot 2N + 1: group 1 finishes
         } else {
-            if (!fetch(0)) return;                       // slot 0: group 0 starts
-            end_even();
-            scores(0);                                   // slot 1
+            end_even();                                  // slot 0: group 0 starts
+            scores(0);                            // slot 1
             end_odd();
-            for (int n = 0; n + 1 < total; ++n) {
-                if (!fetch(n + 1)) return;               // slot 2n + 2
-                softmax();
+            while (more > 0) {
+                more = fetch(n + 1);                     // slot 2n + 2
+                if (more < 0) return;
+                softmax(m0);
                 end_even();
-                weighted_values(n);                      // slot 2n + 3
+                weighted_values(n);               // slot 2n + 3
                 scores(n + 1);
                 end_odd();
+                ++n;
+                m0 = m1;
+                m1 = m2;
             }
-            softmax();                                   // slot 2N
+            softmax(m0);                              // slot 2N
             end_even();
-            weighted_values(total - 1);                  // slot 2N + 1
+            weighted_values(n);                   // slot 2N + 1
             end_odd();
         }
 
@@ -1002,12 +1118,12 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
         const float lse2 = m_i + fast_log2(l_tot);
         const float inv_l = 1.0f / l_tot;
         const int lock_idx = (int)(head * (p.Sq / kBlockM)) + qb;
-        if constexpr (kChain) {
-            // the only visit that writes these q blocks: nothing to merge with and nobody to exclude
+        if (sole_writer) {
+            // the only segment that writes these q blocks: nothing to merge with and nobody to exclude
             merge_rows_through_lds<T>(wave8 < 4 ? k_lds + wave8 * kStageBytes : v_lds + (wave8 - 4) * kStageBytes,
                                       O + z * p.o_st[0] + h * p.o_st[1] + (int64_t)(qb * kBlockM + wave * 32) * p.o_st[2], p.o_st[2],
                                       p.lse + head * p.Sq + qb * kBlockM + wave * 32, o_acc, inv_l, lse2, true, lane);
-            __syncthreads();       // the tiles in LDS are free for the next pair's fills
+            __syncthreads();       // the tiles in LDS are free for the next segment's fills
             if (tid == 0) {
                 __hip_atomic_store(p.first + lock_idx, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 __hip_atomic_store(p.first + lock_idx + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1030,6 +1146,7 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
                 report_status(p.status, SYN_STATUS_SPIN_TIMEOUT, w, (int)blockIdx.x, -2);
                 s_abort = 1;
             }
+            lock_taken_fence();
         }
         __syncthreads();
         if (s_abort) return;
@@ -1045,9 +1162,11 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
         __syncthreads();
         if (tid == 0) {
             // tid 0 is in group 0: its lock_idx is the lower q block of the pair
+            lock_release_fence();
             __hip_atomic_store(p.first + lock_idx, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __hip_atomic_store(p.first + lock_idx + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __builtin_amdgcn_s_waitcnt(attn_vmcnt(0));
+            lock_release_fence();
             __hip_atomic_store(p.lock + lock_idx + 1, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __hip_atomic_store(p.lock + lock_idx, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
@@ -1055,11 +1174,18 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
 }
 
 template <typename T>
-static int launch_attn_pairs(const AttnParams& p, int grid, bool chain, hipStream_t stream) {
-    if (chain)
-        hipLaunchKernelGGL((attn_pair_kernel<T, true>), dim3(grid), dim3(kPairThreads), 0, stream, p);
+static int launch_attn_pairs(const AttnParams& p, int grid, int mode, bool causal, hipStream_t stream) {
+    const dim3 g(grid), b(kPairThreads);
+    if (mode == kPairChainWaves)
+        hipLaunchKernelGGL((attn_pair_kernel<T, kPairChainWaves, false>), g, b, 0, stream, p);
+    else if (mode == kPairWorkList && causal)
+        hipLaunchKernelGGL((attn_pair_kernel<T, kPairWorkList, true>), g, b, 0, stream, p);
+    else if (mode == kPairWorkList)
+        hipLaunchKernelGGL((attn_pair_kernel<T, kPairWorkList, false>), g, b, 0, stream, p);
+    else if (causal)
+        hipLaunchKernelGGL((attn_pair_kernel<T, kPairTiles, true>), g, b, 0, stream, p);
     else
-        hipLaunchKernelGGL((attn_pair_kernel<T, false>), dim3(grid), dim3(kPairThreads), 0, stream, p);
+        hipLaunchKernelGGL((attn_pair_kernel<T, kPairTiles, false>), g, b, 0, stream, p);
     return (int)hipGetLastError();
 }
 
@@ -1102,6 +1228,87 @@ int syn_attn_check_waves(const int32_t* wave_offsets, const int32_t* wave_sizes,
         if (sig >= 0 && num_flags >= 0 && sig >= num_flags) return SYN_ERANGE;
     }
     if (running <= 0 || running != cum_tiles) return SYN_EINVAL;
+    return 0;
+}
+
+int syn_attn_check_work_list(const int32_t* wave_offsets, const int32_t* wave_sizes, const int32_t* cum_wave_sizes,
+                             int32_t num_waves, int32_t block_m, int32_t block_n, int32_t causal,
+                             const int32_t* work_list, int64_t work_list_words, int32_t num_programs,
+                             int32_t require_masked_visits) {
+    if (!wave_offsets || !wave_sizes || !cum_wave_sizes || !work_list) return SYN_EINVAL;
+    if (num_waves <= 0 || block_m <= 0 || block_n <= 0 || num_programs <= 0) return SYN_EINVAL;
+    if (work_list_words < (int64_t)num_programs + 1) return SYN_EINVAL;
+    const int32_t* entries = work_list + num_programs + 1;
+    const int64_t num_entries = work_list_words - num_programs - 1;
+    if (work_list[0] != 0 || work_list[num_programs] != num_entries) return SYN_EINVAL;
+    for (int b = 0; b < num_programs; ++b)
+        if (work_list[b + 1] < work_list[b]) return SYN_EINVAL;
+    int real_waves = 0;
+    while (real_waves < num_waves && cum_wave_sizes[real_waves] != 0) ++real_waves;
+    if (real_waves == 0 || cum_wave_sizes[real_waves - 1] % (2 * block_m)) return SYN_EINVAL;
+    const int64_t pairs = cum_wave_sizes[real_waves - 1] / block_m / 2;
+
+    struct Visit { int z, h, qb, walked; };
+    auto visit_of = [&](int64_t pair, Visit* v) -> bool {
+        int w = 0;
+        while (w < real_waves && cum_wave_sizes[w] / block_m <= 2 * pair) ++w;
+        if (w >= real_waves) return false;
+        const int prev = w == 0 ? 0 : cum_wave_sizes[w - 1] / block_m;
+        const int t = (int)(2 * pair) - prev;
+        const int sh = wave_sizes[4 * w + 1], nq = wave_sizes[4 * w + 2] / block_m;
+        if (sh <= 0 || nq <= 0 || (nq & 1) || (prev & 1)) return false;
+        v->z = t / (nq * sh) + wave_offsets[4 * w];
+        v->h = (t / nq) % sh + wave_offsets[4 * w + 1];
+        v->qb = t % nq + wave_offsets[4 * w + 2] / block_m;
+        const int lo = wave_offsets[4 * w + 3] / block_n, len = wave_sizes[4 * w + 3] / block_n;
+        v->walked = len;
+        if (causal) {
+            if ((lo & 1) || (v->qb & 1)) return false;
+            v->walked = len < v->qb + 2 - lo ? len : v->qb + 2 - lo;
+        }
+        return true;
+    };
+
+    std::vector<unsigned char> seen((size_t)pairs, 0);
+    // per pair of q blocks: segments that write it, and whether one of them claims to be the only one
+    std::map<std::array<int, 3>, std::pair<int, int>> writers;
+    for (int b = 0; b < num_programs; ++b) {
+        bool continued = false;
+        Visit first{};
+        for (int64_t i = work_list[b]; i < work_list[b + 1]; ++i) {
+            const int32_t entry = entries[i];
+            if (entry & ~(SYN_ATTN_WORK_PAIR_MASK | SYN_ATTN_WORK_CONTINUES | SYN_ATTN_WORK_SOLE_WRITER)) return SYN_EINVAL;
+            const int64_t pair = entry & SYN_ATTN_WORK_PAIR_MASK;
+            if (pair >= pairs || seen[(size_t)pair]) return SYN_EINVAL;       // every visit at most once
+            seen[(size_t)pair] = 1;
+            Visit v;
+            if (!visit_of(pair, &v)) return SYN_EINVAL;
+            const bool continues = (entry & SYN_ATTN_WORK_CONTINUES) != 0;
+            if (v.walked <= 0) {
+                // wholly above the diagonal: logged, nothing else; never part of a segment
+                if (continued || continues) return SYN_EINVAL;
+                continue;
+            }
+            if (continued) {
+                if (v.z != first.z || v.h != first.h || v.qb != first.qb) return SYN_EINVAL;
+            } else {
+                first = v;
+                auto& wr = writers[{v.z, v.h, v.qb}];
+                wr.first += 1;
+                wr.second += (entry & SYN_ATTN_WORK_SOLE_WRITER) ? 1 : 0;
+            }
+            if (continues && i + 1 >= work_list[b + 1]) return SYN_EINVAL;    // nothing to continue with
+            continued = continues;
+        }
+    }
+    for (const auto& kv : writers)
+        if (kv.second.second && kv.second.first != 1) return SYN_EINVAL;      // "only writer" beside another segment
+    for (int64_t pair = 0; pair < pairs; ++pair) {
+        if (seen[(size_t)pair]) continue;
+        Visit v;
+        if (!visit_of(pair, &v)) return SYN_EINVAL;
+        if (v.walked > 0 || require_masked_visits) return SYN_EINVAL;         // a visit with work is missing
+    }
     return 0;
 }
 
@@ -1152,6 +1359,8 @@ int syn_attn_fwd(const syn_attn_desc* d, syn_stream_t stream) {
     p.causal = d->causal ? 1 : 0;
     p.num_tiles = (int)tiles;
     p.xcd_remap = (d->options & SYN_ATTN_XCD_REMAP) ? 1 : 0;
+    p.acquire_always = (d->options & SYN_ATTN_ACQUIRE_ALWAYS) ? 1 : 0;
+    p.work_list = d->work_list;
     p.qk_scale = d->sm_scale * 1.44269504f;
     {
         // all-zero strides: contiguous [Z, H, S, D]
@@ -1174,15 +1383,20 @@ int syn_attn_fwd(const syn_attn_desc* d, syn_stream_t stream) {
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     if (d->options & SYN_ATTN_PAIR_Q_BLOCKS) {
         // two q blocks per workgroup: the caller vouches for an even number of q blocks in every wave
-        if (d->causal || d->counters || d->wait_flags || d->wait_signal_offsets || tiles % 2) return SYN_EINVAL;
+        if (d->counters || d->wait_flags || d->wait_signal_offsets || tiles % 2) return SYN_EINVAL;
         const bool chain = (d->options & SYN_ATTN_CHAIN_Q_BLOCKS) != 0;
-        if (chain && d->num_programs <= 0) return SYN_EINVAL;
+        const bool list = (d->options & SYN_ATTN_WORK_LIST) != 0;
+        if (chain && (list || d->causal)) return SYN_EINVAL;
+        if ((chain || list) && d->num_programs <= 0) return SYN_EINVAL;
+        if (list != (d->work_list != nullptr)) return SYN_EINVAL;
         int grid = d->num_programs > 0 ? d->num_programs : (int)(tiles / 2);
-        if (grid > tiles / 2) grid = (int)(tiles / 2);
-        return d->dtype == SYN_DTYPE_BF16 ? launch_attn_pairs<__bf16>(p, grid, chain, s)
-                                          : launch_attn_pairs<_Float16>(p, grid, chain, s);
+        if (!list && grid > tiles / 2) grid = (int)(tiles / 2);      // a list names its programs' visits itself
+        const int mode = chain ? kPairChainWaves : (list ? kPairWorkList : kPairTiles);
+        return d->dtype == SYN_DTYPE_BF16 ? launch_attn_pairs<__bf16>(p, grid, mode, d->causal != 0, s)
+                                          : launch_attn_pairs<_Float16>(p, grid, mode, d->causal != 0, s);
     }
-    if (d->options & SYN_ATTN_CHAIN_Q_BLOCKS) return SYN_EINVAL;
+    if (d->options & (SYN_ATTN_CHAIN_Q_BLOCKS | SYN_ATTN_WORK_LIST)) return SYN_EINVAL;
+    if (d->work_list != nullptr) return SYN_EINVAL;
     int grid = d->num_programs > 0 ? d->num_programs : (int)tiles;
     if (grid > tiles) grid = (int)tiles;
     return d->dtype == SYN_DTYPE_BF16 ? launch_attn<__bf16>(p, grid, s)

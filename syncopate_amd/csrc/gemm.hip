@@ -55,6 +55,7 @@ struct GemmParams {
     int32_t num_tiles;
     int32_t xcd_remap;
     int32_t k_stagger;
+    int32_t acquire_always;      // SYN_GEMM_ACQUIRE_ALWAYS: fence behind every flag wait, not only behind a spin
     // remote bindings (kernel mode 2): per-wave peer tables for A and / or C
     const void* const* a_peers;
     const int32_t* a_target;
@@ -99,10 +100,15 @@ template <>
 struct Mfma16<__bf16> {
     // inline assembly: the accumulator is named as an AGPR tuple that is read and written in place (through the
     // builtin the register allocator moves accumulators between the two register files inside the K loop).
-    // The compiler does not know that the statement is an MFMA and adds no wait states behind it: the pipelines
-    // touch an accumulator once per quarter (at least eight MFMAs apart), and vector instructions read the
-    // accumulators only after the K loop's closing wait and barrier, and write them (zeros) only before its
-    // opening ones.
+    // The compiler does not know that the statement is an MFMA and adds no wait states behind it, so the
+    // hazards are covered by hand:
+    //  - MFMA result -> MFMA accumulator input: the pipelines touch an accumulator once per quarter, at least
+    //    eight MFMAs (128 cycles) apart, and always as the same whole tuple;
+    //  - MFMA result -> vector ALU read or overwrite: a matrix op of N passes needs N + 3 wait states before a
+    //    vector instruction may read or write its result registers (7 for the four passes of 16x16x32, 11 for
+    //    eight, 19 for sixteen).  Every K loop ends in mfma_result_wait_states() below, which idles 24 - more
+    //    than the longest form needs - before the epilogue reads the accumulators and before the next tile's
+    //    zeros are written.
     static __device__ __forceinline__ void run(bf16x8_t a, bf16x8_t b, f32x4_t& c) {
         asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
     }
@@ -114,6 +120,12 @@ struct Mfma16<_Float16> {
         asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
     }
 };
+
+// Wait states between the last assembly MFMA of a K loop and the first vector instruction that touches an
+// accumulator (see Mfma16): 16 + 8 idle issue slots, once per tile.
+__device__ __forceinline__ void mfma_result_wait_states() {
+    asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
+}
 
 template <typename T>
 __device__ __forceinline__ uint2 pack4(float x0, float x1, float x2, float x3) {
@@ -710,6 +722,7 @@ struct EarlyPipe16 : SlabPipe<T, BM, BN, WGM, WGN, 2> {
         // drain the re-fetches of the last slab before anything refills the stages
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, true));
         __builtin_amdgcn_s_barrier();
+        mfma_result_wait_states();      // the accumulators are read by vector instructions from here on
         __builtin_amdgcn_sched_barrier(0);
     }
 };
@@ -806,6 +819,7 @@ struct SlabPipe16 : SlabPipe<T, BM, BN, WGM, WGN, 3> {
         // drain the re-fetches of the last slab before anything refills the stages
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, true));
         __builtin_amdgcn_s_barrier();
+        mfma_result_wait_states();      // the accumulators are read by vector instructions from here on
         __builtin_amdgcn_sched_barrier(0);
     }
 };
@@ -1087,8 +1101,10 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
         // No program reads a chunk's rows before its flag is up, so the XCD's L2 (emptied when the kernel
         // began) cannot hold a stale line of it.  The acquire fence drops every clean line of that L2 -
         // the panels of A and B its 28 other programs are reusing - so only a program that really had
-        // to wait takes it.
-        if (s_spun) acquire_fence_agent();
+        // to wait takes it.  That rests on the caller: nothing on the device reads the gathered buffer
+        // between the start of this kernel and a chunk's flag, and no flag is raised twice during the
+        // launch.  SYN_GEMM_ACQUIRE_ALWAYS is for callers that cannot promise that.
+        if (s_spun || p.acquire_always) acquire_fence_agent();
         return s_abort == 0;
     };
 
@@ -1360,9 +1376,19 @@ static int dispatch_pipe(const GemmParams& p, int bm, int bn, bool eight, bool r
     return dispatch_tile<T, DeepPipe, MODE>(p, bm, bn, eight, grid, stream);
 }
 
+__global__ void __launch_bounds__(256) clear_words_kernel(int32_t* words, int n);
+
+// the tile shapes dispatch_tile has kernels for
+static bool gemm_tile_shape_built(int bm, int bn, bool eight) {
+    const bool common = (bm == 256 && bn == 256) || (bm == 128 && bn == 256) || (bm == 256 && bn == 128);
+    return common || (!eight && ((bm == 256 && bn == 224) || (bm == 128 && bn == 128)));
+}
+
+// clear_counters > 0: the first that many words of `counters` are zeroed on the stream in front of the kernel,
+// once every check has passed (a rejected call must not touch counters a running launch may own).
 static int gemm_entry(const syn_gemm_desc* d, hipStream_t stream, int mode,
                       const syn_gemm_remote* remote = nullptr, const uint64_t* wait_flags = nullptr,
-                      const int32_t* wait_signal_offsets = nullptr) {
+                      const int32_t* wait_signal_offsets = nullptr, int clear_counters = 0) {
     if (d == nullptr) return SYN_EINVAL;
     const bool producer = mode == kProducer;
     if ((wait_flags == nullptr) != (wait_signal_offsets == nullptr)) return SYN_EINVAL;
@@ -1419,6 +1445,7 @@ static int gemm_entry(const syn_gemm_desc* d, hipStream_t stream, int mode,
     p.num_tiles = (int)tiles;
     p.xcd_remap = (d->options & SYN_GEMM_XCD_REMAP) ? 1 : 0;
     p.k_stagger = (d->options & SYN_GEMM_NO_K_STAGGER) ? 0 : 1;
+    p.acquire_always = (d->options & SYN_GEMM_ACQUIRE_ALWAYS) ? 1 : 0;
     p.a_peers = a_remote ? remote->a_peers : nullptr;
     p.a_target = a_remote ? remote->a_target_rank : nullptr;
     p.c_peers = c_remote ? remote->c_peers : nullptr;
@@ -1434,6 +1461,13 @@ static int gemm_entry(const syn_gemm_desc* d, hipStream_t stream, int mode,
     const int bm = d->block_m, bn = d->block_n;
     const bool two = (d->options & SYN_GEMM_TWO_STAGE) != 0;
     const bool m32 = (d->options & SYN_GEMM_MFMA_32X32) != 0;
+    if (!gemm_tile_shape_built(bm, bn, eight)) return SYN_EINVAL;
+    if (clear_counters > 0) {
+        hipLaunchKernelGGL(clear_words_kernel, dim3((clear_counters + 255) / 256), dim3(256), 0, stream, d->counters,
+                           clear_counters);
+        const hipError_t err = hipGetLastError();
+        if (err != hipSuccess) return (int)err;
+    }
     if (d->dtype == SYN_DTYPE_BF16) {
         if (mode == kRemote) return dispatch_pipe<__bf16, kRemote>(p, bm, bn, eight, false, false, m32, grid, stream);
         return producer ? dispatch_pipe<__bf16, kProducer>(p, bm, bn, eight, ring, two, m32, grid, stream)
@@ -1494,14 +1528,20 @@ int syn_gemm_producer_static(const syn_gemm_desc* desc, syn_stream_t stream) {
     const int rc = scratch_address(&counters);
     if (rc != 0) return rc;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-    // the array keeps the last call's counts: the words this launch uses start at zero
-    hipLaunchKernelGGL(clear_words_kernel, dim3((desc->num_waves + 255) / 256), dim3(256), 0, s, counters,
-                       desc->num_waves);
-    const hipError_t err = hipGetLastError();
-    if (err != hipSuccess) return (int)err;
     syn_gemm_desc d = *desc;
     d.counters = counters;
-    return gemm_entry(&d, s, kProducer);
+    // the array keeps the last call's counts: the words this launch uses are zeroed in front of the kernel,
+    // behind every check of the descriptor
+    return gemm_entry(&d, s, kProducer, nullptr, nullptr, nullptr, desc->num_waves);
+}
+
+int syn_gemm_static_counters_peek(int32_t* host_out, int32_t count) {
+    using namespace syn;
+    if (host_out == nullptr || count <= 0 || count > kStaticCounterWords) return SYN_EINVAL;
+    int32_t* counters = nullptr;
+    const int rc = scratch_address(&counters);
+    if (rc != 0) return rc;
+    return (int)hipMemcpy(host_out, counters, sizeof(int32_t) * (size_t)count, hipMemcpyDeviceToHost);
 }
 
 int syn_gemm_consumer(const syn_gemm_desc* desc, syn_stream_t stream) {

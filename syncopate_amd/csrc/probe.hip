@@ -103,6 +103,9 @@ __global__ void __launch_bounds__(256) mfma16_rate_kernel(float* sink, int iters
                 for (int j = 0; j < 8; ++j)
                     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(fb[s][j]), "v"(fa[s][i]));
     }
+    // the compiler adds no wait states behind assembly MFMAs: a matrix op of N passes needs N + 3 of them (at
+    // most 19) before a vector instruction may read its result
+    asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
     float total = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i)

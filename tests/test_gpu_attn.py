@@ -453,11 +453,18 @@ def test_paired_q_blocks_argument_errors(hip):
     offsets, sizes, cums, signals, total = _kv_waves(1, 1, 256, [(0, 256)], [-1])
     kw = dict(wave_offsets=offsets, wave_sizes=sizes, cum_wave_sizes=cums, signal_ptr=flags, signal_offsets=signals,
               cum_tiles=total)
-    with pytest.raises(ValueError):
-        attention_forward(q2, k2, v2, 0.1, pair_q_blocks=True, causal=True, **kw)
+    with pytest.raises(ValueError, match="chain_q_blocks does not go with causal"):
+        attention_forward(q2, k2, v2, 0.1, pair_q_blocks=True, chain_q_blocks=True, causal=True, **kw)
     with pytest.raises(ValueError):
         attention_forward(q2, k2, v2, 0.1, pair_q_blocks=True,
                           counter_ptr=torch.zeros(1, dtype=torch.int32, device="cuda"), **kw)
+    # under a causal mask the pairs' kv ranges have to begin at even blocks
+    q3, k3, v3 = (t.cuda() for t in _qkv(1, 1, 512, 512, torch.bfloat16))
+    offsets, sizes, cums, signals, total = _kv_waves(1, 1, 512, [(0, 128), (128, 512)], [-1, -1])
+    kw = dict(wave_offsets=offsets, wave_sizes=sizes, cum_wave_sizes=cums, signal_ptr=flags, signal_offsets=signals,
+              cum_tiles=total)
+    with pytest.raises(ValueError, match="even blocks"):
+        attention_forward(q3, k3, v3, 0.1, pair_q_blocks=True, causal=True, **kw)
 
 
 def test_producer_form_that_also_waits(hip):

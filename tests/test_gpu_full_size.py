@@ -174,6 +174,66 @@ def test_all2all_attention_16384_causal(hip):
             del s, ref
 
 
+def test_all2all_attention_16384_on_the_64_wave_table(hip):
+    """The table the benchmark times: 8 arrivals of (Q, K, V) chunks of 2048 rows expanded to 64 waves
+    (tests/test_all2all_attn_transform.py:58-117), 4 local heads, causal and not.  The planned launch (one
+    program per compute unit, segments of visits to the same q blocks) and the launcher's automatic choice, both
+    against torch's attention in fp32 on every head; the visit log of the planned launch against the oracle's
+    tile -> work mapping, all 4096 tiles."""
+    from oracle import visit_order
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.attn import attention_forward, plan_attention_work
+    from syncopate_amd.communication.code_gen import CommGenerator
+    from syncopate_amd.communication.common_descriptors import build_all_to_all_plan_dim
+    from syncopate_amd.interface import lower_comm_plan_to_raw_schedules
+    from syncopate_amd.interface.wave_tables import all2all_attn_tables
+
+    world, H, chunk, D = 8, 4, 2048, 128
+    S = world * chunk
+    # rank 0's tables from the plan, as the reference's test derives them
+    plans = {r: build_all_to_all_plan_dim(shape=(3, 1, H * world, chunk, D), dtype=torch.bfloat16, mesh_size=world,
+                                          rank=r, src_buffer="src", dst_buffer="dst", src_split_axis=3,
+                                          dst_split_axis=2, transfer_kind="pull", compute_producer=False)
+             for r in range(world)}
+    gen = CommGenerator(plans)
+    gen.plan_signals()
+    host = all2all_attn_tables(lower_comm_plan_to_raw_schedules(gen)[0]["dst"], {"batch": 1, "head": 2, "seq": 3})
+    offsets, sizes, cums, signals, total = (host.wave_offsets, host.wave_sizes, host.cum_wave_sizes,
+                                            host.signal_offsets, host.cum_tiles)
+    assert len(cums) == 64 and total // 128 == 4096 and max(signals) + 1 == world
+    g = torch.Generator(device="cuda").manual_seed(0)
+    q, k, v = (torch.randn(1, H, S, D, device="cuda", generator=g).bfloat16() for _ in range(3))
+    flags = torch.ones(world, dtype=torch.int64, device="cuda")
+    tables = dict(wave_offsets=offsets, wave_sizes=sizes, cum_wave_sizes=cums, signal_offsets=signals, cum_tiles=total)
+    refs = {}
+    for causal in (True, False):
+        for h in range(H):
+            s = (q[0, h].float() @ k[0, h].float().t()) * D ** -0.5
+            if causal:
+                s = s.masked_fill(torch.ones(S, S, dtype=torch.bool, device="cuda").triu(1), float("-inf"))
+            refs[causal, h] = torch.softmax(s, dim=-1) @ v[0, h].float()
+            del s
+    log = torch.full((total // 128, 8), -1, dtype=torch.int32, device="cuda")
+    for causal in (True, False):
+        for max_visits in (2, None):
+            plan = plan_attention_work(offsets, sizes, cums, causal=causal, num_programs=256, max_visits=max_visits,
+                                       list_masked_visits=True)
+            log.fill_(-1)
+            o = attention_forward(q, k, v, D ** -0.5, signal_ptr=flags, causal=causal, pair_q_blocks=True,
+                                  xcd_remap=True, work_plan=plan, visit_log=log, **tables)
+            check_status()
+            for h in range(H):
+                assert _rel(o[0, h], refs[causal, h]) <= REL_TOL, (causal, max_visits, h)
+            for t, got in enumerate(log.cpu().tolist()):
+                w = visit_order.attn_tile_work(t, offsets, sizes, cums, signals)
+                assert got[:7] == [w["wave"], w["z"], w["h"], w["q_block"], w["kv_lo"], w["kv_hi"], w["signal"]], t
+        # what attention() and form="auto" pick for these tables
+        o = attention_forward(q, k, v, D ** -0.5, signal_ptr=flags, causal=causal, form="auto", **tables)
+        check_status()
+        for h in range(H):
+            assert _rel(o[0, h], refs[causal, h]) <= REL_TOL, (causal, "auto", h)
+
+
 def test_c1_mesh4_fp16_gathered_4096x512_times_512x1024(hip):
     """The reference's own CPU-runnable case on the HIP consumer: mesh of 4, 1-D swizzle pull,
     per-rank A (1024, 512) fp16 gathered to (4096, 512), B (512, 1024), seed 0; every rank's wave
