@@ -251,9 +251,10 @@ def run_throttled(device, steps):
     """The same fused step with the producer throttled to one link's rate: a delay in front of
     every chunk copy brings a chunk to ~LINK_CHUNK_US, the time 16.8 MB take over one xGMI link.
     Seven chunks in sequence then take longer than the GEMM: the step is bound by the producer,
-    and what the wave order buys is that only the last chunk's tiles are left when it lands."""
+    and what the wave order buys is that only the last chunk's tiles are left when it lands - if
+    the tile shape lets that chunk fill the machine.  Every shape is timed; `choose_tile` picks."""
     from syncopate_amd.computation._launch import check_status
-    from syncopate_amd.computation.gemm import gemm
+    from syncopate_amd.computation.gemm import choose_tile, gemm
 
     delay = LINK_CHUNK_US - 28          # a chunk copy beside the running GEMM takes ~28 us
     state = build_ag_gemm(device, link_delay_us=delay)
@@ -261,17 +262,16 @@ def run_throttled(device, steps):
     symm = ctx.comm_buffers["a"][RANK]
     stream = torch.cuda.current_stream()
 
-    def step(i):
-        ctx.reset_signals()
-        ctx.start_after(stream)
-        ctx.execute()
-        gemm(symm, b, c, WORLD, NUM_SMS, BM, BN, BK, GROUP_M, signal_ptr=ctx.recv_signal_bufs[RANK],
-             xcd_remap=XCD_REMAP, eight_waves=EIGHT_WAVES, **tables)
-        ctx.end_before(stream)
+    def step_for(bm, bn):
+        def step(i):
+            ctx.reset_signals()
+            ctx.start_after(stream)
+            ctx.execute()
+            gemm(symm, b, c, WORLD, NUM_SMS, bm, bn, BK, GROUP_M, signal_ptr=ctx.recv_signal_bufs[RANK],
+                 xcd_remap=XCD_REMAP, eight_waves=EIGHT_WAVES, **tables)
+            ctx.end_before(stream)
+        return step
 
-    ms = _timed(step, steps, 5, stream)
-    check_status()
-    ctx.check_status()
     # the producer alone: the same op list with nothing to overlap
     def comm_only(i):
         ctx.reset_signals()
@@ -279,9 +279,23 @@ def run_throttled(device, steps):
         ctx.execute()
         ctx.end_before(stream)
     comm_ms = _timed(comm_only, steps, 3, stream)
+    by_shape = {}
+    for bm, bn in ((256, 256), (128, 256), (256, 128), (128, 128)):
+        ms = _timed(step_for(bm, bn), steps, 5, stream)
+        check_status()
+        ctx.check_status()
+        rows = torch.arange(0, M, 257, device=device)
+        ref = state["a"][rows].float() @ b.float().t()
+        err = ((c[rows].float() - ref).abs().max() / ref.abs().max()).item()
+        by_shape[f"{bm}x{bn}"] = {"ms_per_step": ms, "exposed_compute_ms": ms - comm_ms, "max_rel_err_vs_fp32": err}
+    comm_after_ms = _timed(comm_only, steps, 3, stream)
+    bm, bn = choose_tile(M // WORLD, N, NUM_SMS, producer_bound=True)
+    chosen = by_shape[f"{bm}x{bn}"]
     del state
-    return {"launches": steps, "link_delay_us_per_chunk": delay, "ms_per_step": ms, "producer_alone_ms": comm_ms,
-            "exposed_compute_ms": ms - comm_ms}
+    return {"launches": steps, "link_delay_us_per_chunk": delay, "tile": f"{bm}x{bn}",
+            "tile_choice": "choose_tile(chunk rows, N, programs, producer_bound=True): fewest rounds x tile time for the last chunk",
+            "ms_per_step": chosen["ms_per_step"], "producer_alone_ms": comm_ms, "producer_alone_after_ms": comm_after_ms,
+            "exposed_compute_ms": chosen["exposed_compute_ms"], "by_tile": by_shape}
 
 
 def traffic_calibration(device):
@@ -652,15 +666,20 @@ def run_attention_ag(device, launches=5, gated=True):
     return result
 
 
-def run_attention_a2a(device, launches=5, gated=True):
+def run_attention_a2a(device, launches=10, gated=True):
     """All-to-all (Ulysses) attention of rank 0 of 8: the whole sequence of 16384, 4 local heads, head
     dim 128, causal; Q, K and V arrive as 8 sequence chunks of 2048 (the rank's own first), and
     arrival w unlocks (Q_w x KV_w), (Q_p x KV_w) and (Q_w x KV_p) for every earlier p: 64 waves.
+    The launch is planned (work_plan.plan_attention_work): one program per compute unit, every head's visits on
+    two XCDs, visits to the same q blocks in a row as one segment, segments cut to a program's fair share.
     Resident, and with the chunks copied in behind flags.  flop counts the causal half."""
+    from syncopate_amd import _lib
     from syncopate_amd.communication.code_gen import CommGenerator
     from syncopate_amd.communication.common_descriptors import build_all_to_all_plan_dim
-    from syncopate_amd.computation._launch import check_status
-    from syncopate_amd.computation.attn import attention_forward
+    from syncopate_amd.communication.comm_runtime.persistent_copy import persistent_copy_last_contig
+    from syncopate_amd.communication.comm_runtime.streams import pick_side_streams
+    from syncopate_amd.computation._launch import check_status, trust_flags
+    from syncopate_amd.computation.attn import attention_forward, plan_attention_work
     from syncopate_amd.interface import lower_comm_plan_to_raw_schedules
     from syncopate_amd.interface.wave_tables import all2all_attn_tables
 
@@ -679,70 +698,127 @@ def run_attention_a2a(device, launches=5, gated=True):
     torch.manual_seed(4)
     qkv = torch.randn(3, B, H_local, S, D, device=device).bfloat16()
     scale = D ** -0.5
+    # the benchmark owns these flag arrays and keeps the kernels' precondition: nothing reads a chunk before its flag
     ones = torch.ones(num_flags, dtype=torch.int64, device=device)
+    flags = torch.zeros(num_flags, dtype=torch.int64, device=device)
+    trust_flags(ones, flags)
     out = torch.empty_like(qkv[0])
-    ms = _timed(lambda i: attention_forward(qkv[0], qkv[1], qkv[2], scale, out=out, signal_ptr=ones, causal=True,
-                                            **tables), launches, 2)
+
+    def plan_for(causal, programs, **limits):
+        return plan_attention_work(host.wave_offsets, host.wave_sizes, host.cum_wave_sizes, causal=causal,
+                                   num_programs=programs, **limits)
+
+    def planned(plan, causal, signal=ones, src=qkv, sm_scale=scale):
+        return attention_forward(src[0], src[1], src[2], sm_scale, out=out, signal_ptr=signal, causal=causal,
+                                 pair_q_blocks=True, xcd_remap=True, work_plan=plan, **tables)
+
+    causal_plan = plan_for(True, 256, max_blocks="fair")
+    plain_plan = plan_for(False, 256)
+    gated_plan = plan_for(True, 224, max_visits=1)
+    # (planning is host work of a few tens of milliseconds during which the device idles and its clock drops:
+    # every timed region here follows some 15 ms of the same kernel)
+    warm = 40
+    ms = _timed(lambda i: planned(causal_plan, True), launches, warm)
     check_status()
-    noncausal_ms = _timed(lambda i: attention_forward(qkv[0], qkv[1], qkv[2], scale, out=out, signal_ptr=ones,
-                                                      **tables), launches, 2)
-    attention_forward(qkv[0], qkv[1], qkv[2], scale, out=out, signal_ptr=ones, causal=True, **tables)
+    noncausal_ms = _timed(lambda i: planned(plain_plan, False), launches, warm // 2)
+    # the reference's launch shape: one program per tile, the hardware's scheduler deals them
+    one_tile_ms = _timed(lambda i: attention_forward(qkv[0], qkv[1], qkv[2], scale, out=out, signal_ptr=ones, causal=True,
+                                                     **tables), launches, warm // 2)
     rows = torch.arange(3, S, 61, device=device)
-    s = (qkv[0, 0, 1][rows].float() @ qkv[1, 0, 1].float().t()) * scale
-    s = s.masked_fill(torch.arange(S, device=device)[None, :] > rows[:, None], float("-inf"))
-    ref = torch.softmax(s, dim=-1) @ qkv[2, 0, 1].float()
-    err = ((out[0, 1][rows].float() - ref).abs().max() / ref.abs().max()).item()
+
+    def error(sm_scale, head=1):
+        s = (qkv[0, 0, head][rows].float() @ qkv[1, 0, head].float().t()) * sm_scale
+        s = s.masked_fill(torch.arange(S, device=device)[None, :] > rows[:, None], float("-inf"))
+        ref = torch.softmax(s, dim=-1) @ qkv[2, 0, head].float()
+        return ((out[0, head][rows].float() - ref).abs().max() / ref.abs().max()).item()
+
+    planned(causal_plan, True)
+    err = error(scale)
+    # the reference's tests run this flow with sm_scale = 1.0 (tests/test_all2all_attn_transform.py:297)
+    unit_ms = _timed(lambda i: planned(causal_plan, True, sm_scale=1.0), launches, warm // 2)
+    err_unit = error(1.0)
 
     result = {"launches": launches, "waves": len(host.signal_offsets), "ms_causal": ms, "ms_non_causal": noncausal_ms,
+              "form": "planned: 256 programs, head groups, segments cut to a fair share, xcd_remap",
+              "plan_causal": {"segments": causal_plan.segments, "merged_segments": causal_plan.merged_segments,
+                              "kv_blocks_per_program_max": max(causal_plan.program_cost),
+                              "kv_blocks_per_program_fair": sum(causal_plan.program_cost) / 256},
               "flop_causal": 2.0 * B * H_local * S * S * D, "flop_non_causal": 4.0 * B * H_local * S * S * D,
-              "max_rel_err_vs_fp32": err}
+              "max_rel_err_vs_fp32": err, "ms_causal_sm_scale_1": unit_ms, "max_rel_err_vs_fp32_sm_scale_1": err_unit,
+              "ms_causal_one_program_per_tile": one_tile_ms}
     result["causal_tflops"] = result["flop_causal"] / (ms * 1e-3) / 1e12
     result["non_causal_tflops"] = result["flop_non_causal"] / (noncausal_ms * 1e-3) / 1e12
     if not gated:
         return result
 
-    # gated: Q, K and V of sequence chunk w land together (one box copy of the stacked buffer, then flag w)
-    from syncopate_amd import _lib
-    from syncopate_amd.communication.comm_runtime.persistent_copy import persistent_copy_last_contig
-    from syncopate_amd.communication.comm_runtime.streams import pick_side_streams
-
+    # gated: Q, K and V of sequence chunk w land together, then flag w.  224 programs, so that the stand-in
+    # producer's copy kernels find compute units, and a plan of single visits: a chunk's work is then spread over
+    # as many programs as it has visits, and what is left to do when the last chunk lands is one visit per program.
     lib = _lib.load()
     main = torch.cuda.current_stream()
     side = pick_side_streams(1, main, device)[0]
-    flags = torch.zeros(num_flags, dtype=torch.int64, device=device)
     buf = torch.zeros_like(qkv)
     # arrival order of the sequence chunks and each arrival's flag: the (Q_w x KV_w) waves of the table
     diag = [i for i in range(len(host.signal_offsets))
             if host.wave_offsets[i][2] == host.wave_offsets[i][3] and host.wave_sizes[i][2] == host.wave_sizes[i][3]]
     arrivals = [(host.wave_offsets[i][2] // S_local, host.signal_offsets[i]) for i in diag]
-    persistent_ms = _timed(lambda i: attention_forward(qkv[0], qkv[1], qkv[2], scale, out=out, signal_ptr=ones, causal=True,
-                                                       num_programs=448, **tables), launches, 2)
 
-    def step(i):
-        flags.zero_()
-        side.wait_stream(main)
-        with torch.cuda.stream(side):
-            for c, sig in arrivals:
-                persistent_copy_last_contig(qkv[:, :, :, c * S_local:(c + 1) * S_local],
-                                            buf[:, :, :, c * S_local:(c + 1) * S_local], num_sms=32)
-                if sig >= 0:
-                    _lib.check("syn_flag_set", lib.syn_flag_set(flags.data_ptr() + 8 * sig, 1, _lib.stream_handle(side)))
-        attention_forward(buf[0], buf[1], buf[2], scale, out=out, signal_ptr=flags, causal=True, num_programs=448,
-                          **tables)
-        main.wait_stream(side)
+    # producer (a): one box copy of the stacked buffer per chunk, then the flag kernel - two kernels per chunk
+    def copy_then_flag():
+        for c, sig in arrivals:
+            persistent_copy_last_contig(qkv[:, :, :, c * S_local:(c + 1) * S_local],
+                                        buf[:, :, :, c * S_local:(c + 1) * S_local], num_sms=32)
+            if sig >= 0:
+                _lib.check("syn_flag_set", lib.syn_flag_set(flags.data_ptr() + 8 * sig, 1, _lib.stream_handle(side)))
 
-    gated_ms = _timed(step, launches, 2)
-    check_status()
-    gated_err = ((out[0, 1][rows].float() - ref).abs().max() / ref.abs().max()).item()
-    # timed again behind the gated launches: the overhead is quoted against the mean of the two (the device warms up)
-    persistent_after_ms = _timed(lambda i: attention_forward(qkv[0], qkv[1], qkv[2], scale, out=out, signal_ptr=ones,
-                                                             causal=True, num_programs=448, **tables), launches, 2)
-    baseline_ms = 0.5 * (persistent_ms + persistent_after_ms)
-    result.update({"ms_causal_448_programs_resident": persistent_ms, "ms_causal_gated": gated_ms,
-                   "ms_causal_448_programs_resident_after_gated": persistent_after_ms,
-                   "gated_max_rel_err_vs_fp32": gated_err, "gathered_qkv_matches": bool(torch.equal(buf, qkv)),
-                   "flag_wait_overhead_pct": 100.0 * (gated_ms - baseline_ms) / baseline_ms,
-                   "gated_causal_tflops": result["flop_causal"] / (gated_ms * 1e-3) / 1e12})
+    # producer (b): ONE kernel of 32 workgroups that walks the list of every chunk's twelve rows-of-a-head and
+    # raises a chunk's flag behind its last piece - no kernel boundary, with its cache write-back and
+    # invalidate, while the attention kernel runs
+    records = []
+    for c, sig in arrivals:
+        pieces = [(t, h) for t in range(3) for h in range(H_local)]
+        for n, (t, h) in enumerate(pieces):
+            src_rows = qkv[t, 0, h, c * S_local:(c + 1) * S_local]
+            dst_rows = buf[t, 0, h, c * S_local:(c + 1) * S_local]
+            flag = flags.data_ptr() + 8 * sig if (n + 1 == len(pieces) and sig >= 0) else 0
+            records.append([dst_rows.data_ptr(), src_rows.data_ptr(), src_rows.numel() * 2 // 16, flag, 1, 0])
+    records = torch.tensor(records, dtype=torch.int64, device=device)
+    tickets = torch.zeros(records.shape[0], dtype=torch.int32, device=device)
+
+    def one_list_kernel():
+        _lib.check("syn_copy_flag_list_async",
+                   lib.syn_copy_flag_list_async(records.data_ptr(), records.shape[0], tickets.data_ptr(), 32,
+                                                _lib.stream_handle(side)))
+
+    def gated_ms(producer):
+        def step(i):
+            flags.zero_()
+            side.wait_stream(main)
+            # the kernel first: its persistent programs then hold 224 compute units and the copies get the rest
+            planned(gated_plan, True, signal=flags, src=buf)
+            with torch.cuda.stream(side):
+                producer()
+            main.wait_stream(side)
+        buf.zero_()
+        t = _timed(step, launches, 5)
+        check_status()
+        return t, bool(torch.equal(buf, qkv)), error(scale)
+
+    resident_before = _timed(lambda i: planned(gated_plan, True), launches, warm)
+    list_ms, list_ok, list_err = gated_ms(one_list_kernel)
+    resident_between = _timed(lambda i: planned(gated_plan, True), launches, 5)
+    pair_ms, pair_ok, pair_err = gated_ms(copy_then_flag)
+    resident_after = _timed(lambda i: planned(gated_plan, True), launches, 5)
+    # the device's clock moves over these launches: each gated form is quoted against the resident runs around it
+    result.update({"gated_form": "224 programs, single visits; producer: one list kernel of 32 workgroups",
+                   "ms_causal_224_programs_resident": [resident_before, resident_between, resident_after],
+                   "ms_causal_gated": list_ms, "gated_max_rel_err_vs_fp32": max(list_err, pair_err),
+                   "gathered_qkv_matches": list_ok and pair_ok,
+                   "flag_wait_overhead_pct": 100.0 * (list_ms / (0.5 * (resident_before + resident_between)) - 1.0),
+                   "gated_causal_tflops": result["flop_causal"] / (list_ms * 1e-3) / 1e12,
+                   "ms_causal_gated_copy_kernel_and_flag_kernel_per_chunk": pair_ms,
+                   "flag_wait_overhead_pct_copy_kernel_and_flag_kernel_per_chunk":
+                       100.0 * (pair_ms / (0.5 * (resident_between + resident_after)) - 1.0)})
     return result
 
 

@@ -264,7 +264,7 @@ typedef struct syn_attn_desc {
     const void* v;                  /* (z, h, kv row, d)                                  */
     void* o;                        /* (z, h, q row, d)                                   */
     float* lse;                     /* [Z, H, Sq]                                         */
-    int32_t* lock;                  /* [Z, H, Sq/block_m], zeroed                         */
+    int32_t* lock;                  /* [Z, H, Sq/block_m], zeroed; left in an unspecified state      */
     int32_t* first;                 /* [Z, H, Sq/block_m], zeroed                         */
     uint64_t* flags;
     const int32_t* wave_offsets;    /* device, [num_waves, 4]                             */
@@ -401,7 +401,9 @@ int syn_copy_flag_async(void* dst, const void* src, int64_t nbytes, uint64_t* fl
  * record while others still finish the last one).  `ops` is a DEVICE array of `count` records
  * (every dst / src 16-byte aligned, `bytes16` = length in 16-byte units), `tickets` `count` zeroed
  * 32-bit words of device memory, left zero again.  `delay_ticks` > 0 lets that many ticks of the
- * device's wall clock (100 MHz) pass in front of a record: a slow link.  The data is stored through the L2, so no
+ * device's wall clock (100 MHz) pass in front of a record: a slow link.  A record whose `flag` is NULL is a piece
+ * of a transfer in several pieces (the rows of a strided box): it is copied, and the flag of the next record that
+ * has one covers it.  The data is stored through the L2, so no
  * kernel boundary - with its cache write-back and invalidate - falls into a consumer kernel that
  * runs beside the list.  Replaces a whole stream of cudaMemcpyAsync + cuStreamWriteValue pairs of the
  * reference's executor (communication_context.py:129-150). */

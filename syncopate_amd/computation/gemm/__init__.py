@@ -5,3 +5,4 @@ from .template_remote import (  # noqa: F401
     gemm_rs_producer_persistent,
     gemm_splitk,
 )
+from .tile_policy import choose_tile  # noqa: F401

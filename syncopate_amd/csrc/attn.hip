@@ -645,6 +645,7 @@ __device__ __forceinline__ void dma_kv_block8(unsigned char* lds, const unsigned
 // block, the lower q block sits the last block out, and each masks its own diagonal block.
 constexpr int kPairTiles = 0, kPairChainWaves = 1, kPairWorkList = 2;
 constexpr int32_t kWorkPairMask = SYN_ATTN_WORK_PAIR_MASK;
+constexpr int kPairLdsWaves = 256, kPairLdsEntries = 512;
 
 template <typename T, int MODE, bool CAUSAL>
 __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnParams p) {
@@ -656,6 +657,12 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
     __shared__ __attribute__((aligned(1024))) unsigned char v_lds[2 * kBlockBytes];
     __shared__ int s_abort;
     __shared__ int s_spun;
+    // the head of the wave table and of this program's list, read once: what a visit is (a search over the prefix
+    // sums, then a row of the table) is looked up at every change of visit, where all eight wavefronts wait for it -
+    // from LDS that takes a tenth of a trip to memory
+    __shared__ int s_cum[kPairLdsWaves];             // tiles up to and including the wave (0: padding)
+    __shared__ int s_row[kPairLdsWaves][8];          // size_h, q blocks, first z, first h, first q block, kv_lo, kv blocks, signal
+    __shared__ int s_entries[kPairLdsEntries];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -666,7 +673,17 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
     const int half = lane >> 5;
 
     if (tid == 0) s_abort = 0;
-    __syncthreads();
+    for (int w = tid; w < min(p.num_waves, kPairLdsWaves); w += kPairThreads) {
+        s_cum[w] = p.cum_wave_sizes[w] / kBlockM;
+        s_row[w][0] = p.wave_sizes[w * 4 + 1];
+        s_row[w][1] = p.wave_sizes[w * 4 + 2] / kBlockM;
+        s_row[w][2] = p.wave_offsets[w * 4 + 0];
+        s_row[w][3] = p.wave_offsets[w * 4 + 1];
+        s_row[w][4] = p.wave_offsets[w * 4 + 2] / kBlockM;
+        s_row[w][5] = p.wave_offsets[w * 4 + 3] / kBlockN;
+        s_row[w][6] = p.wave_sizes[w * 4 + 3] / kBlockN;
+        s_row[w][7] = p.signal_offsets[w];
+    }
 
     // per-lane offsets exactly as in attn_fwd_kernel (the fill swizzle depends on wave8 % 4 only)
     const int f_row = lane >> 4, f_c = lane & 15;
@@ -701,13 +718,62 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
 
     // where the program stands: the next pair of the table (kPairTiles, kPairChainWaves) or the entry of its list
     int pair = program;
-    int e = 0, e_end = 0;
+    int e = 0, e_end = 0, e_begin = 0;
     const int32_t* entries = nullptr;
     if constexpr (MODE == kPairWorkList) {
-        e = __builtin_amdgcn_readfirstlane(p.work_list[program]);
+        e = e_begin = __builtin_amdgcn_readfirstlane(p.work_list[program]);
         e_end = __builtin_amdgcn_readfirstlane(p.work_list[program + 1]);
         entries = p.work_list + gridDim.x + 1;
+        for (int i = tid; i < min(e_end - e_begin, kPairLdsEntries); i += kPairThreads) s_entries[i] = entries[e_begin + i];
     }
+    __syncthreads();
+    auto entry_at = [&](const int i) __attribute__((always_inline)) {
+        return __builtin_amdgcn_readfirstlane(i - e_begin < kPairLdsEntries ? s_entries[i - e_begin] : entries[i]);
+    };
+    // what a tile id is: wave, (z, h, q block), kv range in blocks, flag (the lookup of find_wave, on the copy in LDS)
+    struct Where {
+        int w, z, h, qb, kv_lo, kv_len, sig;
+        bool paired;        // an even number of q blocks in the wave, an even number of tiles in front of it
+    };
+    auto locate = [&](const int tile, Where& at) __attribute__((always_inline)) -> bool {
+        int w = 0;
+        for (int base = 0; base < p.num_waves; base += 64) {
+            const int idx = base + lane;
+            const int cum = idx >= p.num_waves ? 0 : (idx < kPairLdsWaves ? s_cum[idx] : p.cum_wave_sizes[idx] / kBlockM);
+            const unsigned long long below = __builtin_amdgcn_ballot_w64(cum != 0 && cum <= tile);
+            w += __builtin_popcountll(below);
+            if (below != ~0ull) break;
+        }
+        if (w >= p.num_waves) return false;
+        int row[8], prev;
+        if (w < kPairLdsWaves) {
+#pragma unroll
+            for (int f = 0; f < 8; ++f) row[f] = __builtin_amdgcn_readfirstlane(s_row[w][f]);
+            prev = w == 0 ? 0 : __builtin_amdgcn_readfirstlane(s_cum[w - 1]);
+            if (__builtin_amdgcn_readfirstlane(s_cum[w]) == 0) return false;          // only padding is left
+        } else {
+            row[0] = p.wave_sizes[w * 4 + 1];
+            row[1] = p.wave_sizes[w * 4 + 2] / kBlockM;
+            row[2] = p.wave_offsets[w * 4 + 0];
+            row[3] = p.wave_offsets[w * 4 + 1];
+            row[4] = p.wave_offsets[w * 4 + 2] / kBlockM;
+            row[5] = p.wave_offsets[w * 4 + 3] / kBlockN;
+            row[6] = p.wave_sizes[w * 4 + 3] / kBlockN;
+            row[7] = p.signal_offsets[w];
+            prev = p.cum_wave_sizes[w - 1] / kBlockM;
+            if (p.cum_wave_sizes[w] == 0) return false;
+        }
+        const int t = tile - prev;
+        at.w = w;
+        at.z = t / (row[1] * row[0]) + row[2];
+        at.h = (t / row[1]) % row[0] + row[3];
+        at.qb = t % row[1] + row[4];
+        at.kv_lo = row[5];
+        at.kv_len = row[6];
+        at.sig = row[7];
+        at.paired = !(row[1] & 1) && !(prev & 1);
+        return true;
+    };
     auto advance = [&]() __attribute__((always_inline)) {
         if constexpr (MODE == kPairWorkList) ++e;
         else pair += gridDim.x;
@@ -715,9 +781,19 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
     auto pending = [&]() __attribute__((always_inline)) { return MODE == kPairWorkList ? e < e_end : pair < num_pairs; };
 
     // wait for flag `sg` of the wave `wv` that is being entered; false when the wait gave up
+    // A look ahead at the flag of the visit after the one being entered (thread 0): asked for here, read at the next
+    // change of visit, a kv range later.  A flag goes up once per launch, so a 1 seen early still holds then; a 0
+    // means nothing and the flag is read again.
+    int peeked_sig = -1;
+    unsigned long long peeked = 0;
+    auto peek_flag = [&](const int sg) __attribute__((always_inline)) {
+        peeked_sig = sg;
+        if (tid == 0 && sg >= 0) peeked = __hip_atomic_load(p.flags + sg, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    };
     auto wait_for_flag = [&](const int sg, const int wv) __attribute__((always_inline)) -> bool {
         if (tid == 0) {
-            s_spun = __hip_atomic_load(p.flags + sg, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 1ull;
+            const bool seen_up = peeked_sig == sg && peeked == 1ull;
+            s_spun = !seen_up && __hip_atomic_load(p.flags + sg, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 1ull;
             if (s_spun && !spin_until_equal(p.flags + sg, 1ull, p.timeout_ticks)) {
                 report_status(p.status, SYN_STATUS_SPIN_TIMEOUT, wv, (int)blockIdx.x, sg);
                 s_abort = 1;
@@ -736,27 +812,19 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
         // ---- the segment's first visit: tile id -> wave -> (z, h, q block, kv range); the two tiles of a pair
         //      differ in the q block only ----
         int entry = 0;
-        if constexpr (MODE == kPairWorkList) entry = __builtin_amdgcn_readfirstlane(entries[e]);
+        if constexpr (MODE == kPairWorkList) entry = entry_at(e);
         const int pair_id = MODE == kPairWorkList ? (entry & kWorkPairMask) : pair;
         const bool sole_writer = MODE == kPairChainWaves || (MODE == kPairWorkList && (entry & SYN_ATTN_WORK_SOLE_WRITER));
         const int tile_id = 2 * pair_id + grp;
-        const int w = find_wave(p.cum_wave_sizes, p.num_waves, kBlockM, tile_id, lane);
-        if (w >= p.num_waves) return;
-        const int prev = w == 0 ? 0 : p.cum_wave_sizes[w - 1] / kBlockM;
-        const int t = tile_id - prev;
-        const int size_h = p.wave_sizes[w * 4 + 1];
-        const int nq = p.wave_sizes[w * 4 + 2] / kBlockM;
-        const int z = t / (nq * size_h) + p.wave_offsets[w * 4 + 0];
-        const int h = (t / nq) % size_h + p.wave_offsets[w * 4 + 1];
-        const int qb = t % nq + p.wave_offsets[w * 4 + 2] / kBlockM;
-        const int kv_lo = p.wave_offsets[w * 4 + 3] / kBlockN;
-        const int kv_len = p.wave_sizes[w * 4 + 3] / kBlockN;
-        const int sig = p.signal_offsets[w];
+        Where first;
+        if (!locate(tile_id, first)) return;
+        const int w = first.w, z = first.z, h = first.h, qb = first.qb;
+        const int kv_lo = first.kv_lo, kv_len = first.kv_len, sig = first.sig;
         // the caller promised an even number of q blocks per wave (and, under a causal mask, q ranges and kv
         // ranges that begin at even blocks: the lower q block of a pair then never finds its whole visit masked
         // while the higher one has work); leave a note instead of wrong results
-        if ((nq & 1) || (prev & 1) || (CAUSAL && ((kv_lo | (qb - grp)) & 1))) {
-            if (lane == 0 && wave8 == 0) report_status(p.status, SYN_STATUS_BAD_PAIRING, w, (int)blockIdx.x, nq);
+        if (!first.paired || (CAUSAL && ((kv_lo | (qb - grp)) & 1))) {
+            if (lane == 0 && wave8 == 0) report_status(p.status, SYN_STATUS_BAD_PAIRING, w, (int)blockIdx.x, kv_lo);
             return;
         }
 
@@ -811,69 +879,62 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
             m2 = m0;
         }
 
+        // the flag of the visit that follows the one the K walk has just entered, if the segment goes on
+        auto look_ahead = [&]() __attribute__((always_inline)) {
+            int next_tile;
+            if constexpr (MODE == kPairTiles) {
+                return;
+            } else if constexpr (MODE == kPairChainWaves) {
+                if (k_wave + 1 >= p.num_waves) return;
+                next_tile = tile_id + 2 * (k_wave + 1) * pairs_per_wave;
+            } else {
+                if (!(entry & SYN_ATTN_WORK_CONTINUES) || e + 1 >= e_end) return;
+                next_tile = 2 * (entry_at(e + 1) & kWorkPairMask) + grp;
+            }
+            Where at;
+            if (locate(next_tile, at)) peek_flag(at.sig);
+        };
+
         // the K walk enters the segment's next visit: 1 entered, 0 the segment ends here, -1 give up
         auto enter_next_visit = [&]() __attribute__((always_inline)) -> int {
-            int wv;
             int next_tile;
             if constexpr (MODE == kPairTiles) {
                 return 0;
             } else if constexpr (MODE == kPairChainWaves) {
                 if (k_wave + 1 >= p.num_waves || p.cum_wave_sizes[k_wave + 1] == 0) return 0;
-                wv = ++k_wave;
-                bool same = true;
-#pragma unroll
-                for (int a = 0; a < 3; ++a)
-                    same = same && p.wave_offsets[wv * 4 + a] == p.wave_offsets[a] && p.wave_sizes[wv * 4 + a] == p.wave_sizes[a];
-                if (!same) {
-                    if (tid == 0) report_status(p.status, SYN_STATUS_BAD_CHAIN, wv, (int)blockIdx.x, -1);
-                    return -1;
-                }
-                next_tile = tile_id + 2 * wv * pairs_per_wave;
+                ++k_wave;
+                next_tile = tile_id + 2 * k_wave * pairs_per_wave;
             } else {
                 if (!(entry & SYN_ATTN_WORK_CONTINUES) || e + 1 >= e_end) return 0;
                 ++e;
-                entry = __builtin_amdgcn_readfirstlane(entries[e]);
+                entry = entry_at(e);
                 next_tile = 2 * (entry & kWorkPairMask) + grp;
-                wv = find_wave(p.cum_wave_sizes, p.num_waves, kBlockM, next_tile, lane);
-                bool same = wv < p.num_waves;
-                if (same) {
-                    const int pv = wv == 0 ? 0 : p.cum_wave_sizes[wv - 1] / kBlockM;
-                    const int tt = next_tile - pv;
-                    const int sh = p.wave_sizes[wv * 4 + 1];
-                    const int nn = p.wave_sizes[wv * 4 + 2] / kBlockM;
-                    same = !(nn & 1) && !(pv & 1) && tt / (nn * sh) + p.wave_offsets[wv * 4 + 0] == z &&
-                           (tt / nn) % sh + p.wave_offsets[wv * 4 + 1] == h &&
-                           tt % nn + p.wave_offsets[wv * 4 + 2] / kBlockM == qb;
-                }
-                if (!same) {
-                    // the entry does not continue on this segment's q blocks
-                    if (tid == 0) report_status(p.status, SYN_STATUS_BAD_CHAIN, wv, (int)blockIdx.x, next_tile);
-                    return -1;
-                }
             }
-            const int lo = p.wave_offsets[wv * 4 + 3] / kBlockN;
-            const int len = p.wave_sizes[wv * 4 + 3] / kBlockN;
-            const int sg = p.signal_offsets[wv];
-            const int walked = CAUSAL ? min(len, diag_hi + 1 - lo) : len;
-            if (CAUSAL && (walked <= 0 || (lo & 1))) {
-                // a visit with nothing below the diagonal cannot continue a segment
-                if (tid == 0) report_status(p.status, SYN_STATUS_BAD_CHAIN, wv, (int)blockIdx.x, next_tile);
+            Where at;
+            const bool found = locate(next_tile, at);
+            const int walked = CAUSAL ? min(at.kv_len, diag_hi + 1 - at.kv_lo) : at.kv_len;
+            // the visit has to be to this segment's q blocks (for kPairChainWaves: every wave lists the ranges of
+            // wave 0), and under a causal mask a visit with nothing below the diagonal cannot continue a segment
+            if (!found || !at.paired || at.z != z || at.h != h || at.qb != qb || (MODE == kPairChainWaves && at.w != k_wave) ||
+                (CAUSAL && (walked <= 0 || (at.kv_lo & 1)))) {
+                if (tid == 0) report_status(p.status, SYN_STATUS_BAD_CHAIN, found ? at.w : -1, (int)blockIdx.x, next_tile);
                 return -1;
             }
             if (p.visit_log != nullptr && lane == 0 && wave == 0) {
                 int4* rec = reinterpret_cast<int4*>(p.visit_log) + 2 * (size_t)next_tile;
-                rec[0] = make_int4(wv, z, h, qb);
-                rec[1] = make_int4(lo, lo + len, sg, (int)blockIdx.x);
+                rec[0] = make_int4(at.w, z, h, qb);
+                rec[1] = make_int4(at.kv_lo, at.kv_lo + at.kv_len, at.sig, (int)blockIdx.x);
             }
-            if (sg >= 0 && !wait_for_flag(sg, wv)) return -1;
-            k_lo = lo;
+            if (at.sig >= 0 && !wait_for_flag(at.sig, at.w)) return -1;
+            look_ahead();
+            k_lo = at.kv_lo;
             k_nkv = walked;
-            k_rot = rotation(lo, len, walked);
+            k_rot = rotation(at.kv_lo, at.kv_len, walked);
             k_next = 0;
-            k_walk = k_head + (size_t)lo * kBlockN * k_pitch;
+            k_walk = k_head + (size_t)at.kv_lo * kBlockN * k_pitch;
             return 1;
         };
-
+        look_ahead();
         // every wavefront has passed the barrier that ended the previous segment: all four buffers are free
         dma_kv_block8(k_lds, k_walk + (size_t)k_rot * kBlockN * k_pitch, k_pitch, k_fill_off, wave8);
 
@@ -1130,28 +1191,29 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
             }
             continue;
         }
+        // One lock word per PAIR of q blocks (the lower block's; every program of a launch of this kernel pairs the same
+        // blocks), and it carries whether the pair has been written: bit 0 held, bit 1 written.  Taking it is one
+        // atomic OR whose result says both whether it was free and whether somebody was first - one trip to memory
+        // where a compare-and-swap per block followed by a load of `first` were three - and the hand-over is one store.
         if (tid == 0) {
-            // one thread takes both locks, lower q block first: every workgroup that wants this
-            // pair of q blocks takes them in the same order
             const uint64_t t0 = wall_clock64();
-            bool ok = true;
-            for (int which = 0; which < 2 && ok; ++which) {
-                while (atomicCAS(p.lock + lock_idx + which, 0, 1) != 0) {
-                    __builtin_amdgcn_s_sleep(4);
-                    if ((int64_t)(wall_clock64() - t0) > p.timeout_ticks) { ok = false; break; }
+            int seen;
+            for (;;) {
+                seen = __hip_atomic_fetch_or(p.lock + lock_idx, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (!(seen & 1)) break;
+                __builtin_amdgcn_s_sleep(4);
+                if ((int64_t)(wall_clock64() - t0) > p.timeout_ticks) {
+                    report_status(p.status, SYN_STATUS_SPIN_TIMEOUT, w, (int)blockIdx.x, -2);
+                    s_abort = 1;
+                    break;
                 }
-                if (!ok && which == 1) __hip_atomic_store(p.lock + lock_idx, 0, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
             }
-            if (!ok) {
-                report_status(p.status, SYN_STATUS_SPIN_TIMEOUT, w, (int)blockIdx.x, -2);
-                s_abort = 1;
-            }
+            s_spun = (seen & 2) == 0;            // (the word is free between flag waits) nobody has written the pair yet
             lock_taken_fence();
         }
         __syncthreads();
-        if (s_abort) return;
-
-        const bool is_first = __hip_atomic_load(p.first + lock_idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0;
+        if (__builtin_amdgcn_readfirstlane(s_abort)) return;
+        const bool is_first = __builtin_amdgcn_readfirstlane(s_spun) != 0;
         // (the K and V blocks are free: every wavefront has passed the last slot's barrier)
         merge_rows_through_lds<T>(wave8 < 4 ? k_lds + wave8 * kStageBytes : v_lds + (wave8 - 4) * kStageBytes,
                                   O + z * p.o_st[0] + h * p.o_st[1] + (int64_t)(qb * kBlockM + wave * 32) * p.o_st[2], p.o_st[2],
@@ -1163,12 +1225,9 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
         if (tid == 0) {
             // tid 0 is in group 0: its lock_idx is the lower q block of the pair
             lock_release_fence();
+            __hip_atomic_store(p.lock + lock_idx, 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __hip_atomic_store(p.first + lock_idx, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __hip_atomic_store(p.first + lock_idx + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __builtin_amdgcn_s_waitcnt(attn_vmcnt(0));
-            lock_release_fence();
-            __hip_atomic_store(p.lock + lock_idx + 1, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(p.lock + lock_idx, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
 }

@@ -104,8 +104,10 @@ __device__ __forceinline__ void store16_through(u32x4_t* dst, u32x4_t v) {
 __global__ void __launch_bounds__(kCopyFlagThreads)
 copy_flag_list_kernel(const CopyFlagOp* __restrict__ ops, int count, uint32_t* tickets) {
     const int64_t stride = (int64_t)gridDim.x * kCopyFlagThreads;
+    CopyFlagOp next = ops[0];
     for (int k = 0; k < count; ++k) {
-        const CopyFlagOp op = ops[k];
+        const CopyFlagOp op = next;
+        if (k + 1 < count) next = ops[k + 1];       // asked for now, needed a record later: short records are not a trip to memory each
         if (op.delay_ticks > 0) {
             const uint64_t t0 = wall_clock64();
             while ((int64_t)(wall_clock64() - t0) < op.delay_ticks) __builtin_amdgcn_s_sleep(32);
@@ -119,6 +121,9 @@ copy_flag_list_kernel(const CopyFlagOp* __restrict__ ops, int count, uint32_t* t
             for (int u = 0; u < 4; ++u)
                 if (i + u * stride < op.vecs) store16_through(op.dst + i + u * stride, v[u]);
         }
+        // a record without a flag is a piece of a transfer whose last record carries it: a workgroup's stores
+        // go out in record order, so the wait in front of that record's ticket covers them
+        if (op.flag == nullptr) continue;
         __builtin_amdgcn_s_waitcnt(0x0070);          // vmcnt(0): this lane's stores have reached memory
         __syncthreads();
         if (threadIdx.x == 0) {

@@ -65,3 +65,24 @@ def test_padded_receive_buffer_layout():
     assert buf[4].data_ptr() - buf[3].data_ptr() == (rows * n + pad) * 2
     one = padded_receive_buffer(1, rows, n, torch.float16, "cpu")
     assert one.shape == (1, rows, n)
+
+
+def test_tile_policy_picks_a_shape_whose_last_chunk_fills_the_machine():
+    """The producer-bound regime of the all-gather GEMM: what is left to compute when the last chunk lands is
+    `rounds x tile time` of that chunk's tiles (reference: the tile shape is a call-site kwarg,
+    syncopate/computation/gemm/template.py:193-220, swept by hand in tests/test_ag_gemm_tile_size_sensitivity.py)."""
+    import pytest
+
+    from syncopate_amd.computation.gemm.tile_policy import choose_tile, rounds
+
+    # headline shape: chunks of 1024 rows x 3584 columns on 224 programs
+    assert rounds(1024, 3584, 256, 256, 224) == 1 and rounds(1024, 3584, 128, 128, 224) == 1
+    assert choose_tile(1024, 3584, 224, producer_bound=False) == (256, 256)
+    assert choose_tile(1024, 3584, 224, producer_bound=True) == (256, 128)
+    # a chunk that is many rounds of any shape: the cheapest per element wins either way
+    assert choose_tile(8192, 8192, 224, producer_bound=True) == (256, 256)
+    # only shapes that divide the chunk are offered
+    assert choose_tile(128, 256, 224, producer_bound=True) in ((128, 256), (128, 128))
+    assert choose_tile(1024, 3584, 224, producer_bound=True, shapes=[(256, 256), (128, 128)]) == (128, 128)
+    with pytest.raises(ValueError):
+        choose_tile(100, 3584, 224, producer_bound=True)
