@@ -225,7 +225,11 @@ def run_ag_gemm(state, steps, warmup, resident_only=False, use_graph=True, lead_
     ctx.check_status()
 
     # ---- same kernel, every chunk resident and every flag already set ----
+    # (a flag array of the benchmark's own: declared trusted, as the executor's are - nothing here reads a chunk
+    # before its flag - so that resident and gated launches run the same code path)
+    from syncopate_amd.computation._launch import trust_flags
     resident_flags = torch.ones_like(ctx.recv_signal_bufs[RANK])
+    trust_flags(resident_flags)
 
     def resident_ms(a_operand=symm, b_operand=b):
         for _ in range(warmup):
@@ -572,7 +576,7 @@ def _gated_attention(q, staged_kv, buf, arrival, chunk, tables, launches, device
     from syncopate_amd import _lib
     from syncopate_amd.communication.comm_runtime.persistent_copy import persistent_copy_last_contig
     from syncopate_amd.communication.comm_runtime.streams import pick_side_streams
-    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation._launch import check_status, trust_flags
     from syncopate_amd.computation.attn import attention_forward
 
     lib = _lib.load()
@@ -580,6 +584,7 @@ def _gated_attention(q, staged_kv, buf, arrival, chunk, tables, launches, device
     main = torch.cuda.current_stream()
     side = pick_side_streams(1, main, device)[0]
     flags = torch.zeros(len(arrival), dtype=torch.int64, device=device)
+    trust_flags(flags)
     out = torch.empty_like(q)
     signals = tables["signal_offsets"].tolist()
     own = arrival[0]
@@ -614,7 +619,7 @@ def run_attention_ag(device, launches=5, gated=True):
     blocks per workgroup in opposite phases (pair_q_blocks).  Resident (every flag set) in the chained form
     and in the forms that merge after every tile, and gated (224 persistent programs that merge: the
     stand-in producer's copy kernels need the other 32 compute units)."""
-    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation._launch import check_status, trust_flags
     from syncopate_amd.computation.attn import attention_forward
 
     B, H, Sq, Skv, D, chunks = 1, 32, 4096, 32768, 128, 8
@@ -628,6 +633,7 @@ def run_attention_ag(device, launches=5, gated=True):
                   wave_sizes=_table([[B, H, Sq, chunk]] * chunks, device), cum_wave_sizes=_table(cums, device),
                   signal_offsets=_table([-1, 0, 4, 1, 5, 2, 6, 3], device), cum_tiles=cums[-1])
     ones = torch.ones(chunks, dtype=torch.int64, device=device)
+    trust_flags(ones)
     out = torch.empty_like(q)
     def resident(**kw):
         return _timed(lambda i: attention_forward(q, kv[0], kv[1], D ** -0.5, out=out, pair_q_blocks=True,
@@ -824,12 +830,31 @@ def run_attention_a2a(device, launches=10, gated=True):
 
 # -------------------------------------------------------------------------------- CPU baselines
 
+def _host_cpu():
+    """What the CPU baselines ran on: the model string, the cores the host shows and the threads used.  A one-GPU box
+    of the pool gives a job 16 cores whatever the host shows (OMP_NUM_THREADS is 16 there), so the baselines use
+    at most that many threads."""
+    model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    threads = min(16, os.cpu_count() or 1)
+    return {"cpu_model": model, "host_cores": os.cpu_count(), "threads": threads,
+            "threads_note": "capped at the 16 cores a one-GPU job of this pool is given"}
+
+
 def cpu_baseline(state):
     """torch CPU matmul over the gathered operands (fp32 values of the same bf16 inputs):
     a bounded sample of the same GEMM — a band of rows of A against all of B."""
     from oracle import numerics
 
-    threads = min(16, os.cpu_count() or 1)
+    host = _host_cpu()
+    threads = host["threads"]
     torch.set_num_threads(threads)
     sample_rows = M
     a = state["a"][:sample_rows].cpu()
@@ -846,6 +871,10 @@ def cpu_baseline(state):
         "value": flop / spent / 1e12,
         "unit": "TFLOP/s",
         "cores": threads,
+        "torch_num_threads": torch.get_num_threads(),
+        "cpu_model": host["cpu_model"],
+        "host_cores": host["host_cores"],
+        "threads_note": host["threads_note"],
         "kind": "port",
         "sample": f"{reps} x torch CPU fp32 matmul of A[:{sample_rows}] (bf16 values) with all of B, "
                   f"{spent:.1f} s",
@@ -864,9 +893,10 @@ def cpu_baselines_other():
     from syncopate_amd.communication.common_descriptors import build_all_gather_plan_1d_swizzle
     from syncopate_amd.interface import lower_comm_plan_to_raw_schedules
 
-    threads = min(16, os.cpu_count() or 1)
+    host = _host_cpu()
+    threads = host["threads"]
     torch.set_num_threads(threads)
-    result = {"cores": threads}
+    result = {"cores": threads, "cpu_model": host["cpu_model"], "host_cores": host["host_cores"]}
 
     def compile_c1():
         plans = {r: build_all_gather_plan_1d_swizzle((4096, 512), torch.float16, 0, 4, r, "a", "pull") for r in range(4)}
@@ -958,6 +988,10 @@ def main():
     ap.add_argument("--list-blocks", type=int, default=LIST_BLOCKS,
                     help="N > 0: the producer is ONE kernel of N workgroups that walks the list of chunk copies and raises "
                          "each chunk's flag (two kernels with --lead-ops: the leading chunks, then the rest)")
+    ap.add_argument("--wave0-flag", type=int, default=-1,
+                    help="N >= 0 (with --lead-ops 0): the consumer is launched together with the first copy and its "
+                         "wave 0 - the rank's own, resident chunk - waits for flag N, so that the kernel's launch "
+                         "and the cross-queue event leave the path while it spins until chunk N + 1 has landed")
     ap.add_argument("--flag-write-values", action="store_true",
                     help="with --no-graph: flag writes are stream memory operations instead of one-wavefront kernels")
     ap.add_argument("--lead-on-compute-stream", action="store_true",
@@ -994,6 +1028,8 @@ def main():
     state = build_ag_gemm(device, args.copy_blocks, args.split_device, args.fuse_flags,
                           lead_copy_blocks=args.lead_copy_blocks, flag_write_values=args.flag_write_values,
                           list_blocks=args.list_blocks)
+    if args.wave0_flag >= 0:
+        state["tables"]["signal_offsets"][0] = args.wave0_flag
     with torch.cuda.stream(state["ctx"].compute_stream):
         wall_ms, gated_ms, no_lead_ms, resident_ms = run_ag_gemm(state, args.steps, args.warmup, args.resident_only,
                                                                  not args.no_graph)

@@ -54,11 +54,18 @@ def test_static_counter_producer_matches_the_allocating_one(hip):
         d = _desc(_lib, a, b, c, flags, sizes, offsets, signals, None, status, BM, BN, num_sms)
         torch.cuda.synchronize()
         before = torch.cuda.memory_stats()["allocation.all.allocated"]
+        free_before = torch.cuda.mem_get_info()[0]        # the driver's view: a hipMalloc inside the library would show here
         _lib.check("syn_gemm_producer_static", hip.syn_gemm_producer_static(ctypes.byref(d), stream))
         torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free_before
         assert torch.cuda.memory_stats()["allocation.all.allocated"] == before
         assert status.tolist()[0] == 0
-        assert counters.tolist() == [(M // world // BM) * (N // BN)] * world
+        tiles_per_wave = (M // world // BM) * (N // BN)
+        assert counters.tolist() == [tiles_per_wave] * world
+        # the library's own array holds this launch's counts (and nothing of the larger launch before it)
+        peek = (ctypes.c_int32 * world)()
+        _lib.check("syn_gemm_static_counters_peek", hip.syn_gemm_static_counters_peek(peek, world))
+        assert list(peek) == [tiles_per_wave] * world
         assert flags.tolist() == [1] * world and flags_ref.tolist() == [1] * world
         assert torch.equal(c, c_ref)                      # same kernel, same tile shape: bit for bit
         ref = a.float() @ b.float().t()
@@ -83,3 +90,29 @@ def test_static_counter_producer_rejects_what_it_cannot_hold(hip):
         _lib.check("syn_gemm_producer_static", _lib.SYN_E2BIG)
     torch.cuda.synchronize()
     assert flags.tolist() == [0, 0]
+
+
+def test_a_rejected_call_leaves_the_static_counters_alone(hip):
+    """The counters are cleared behind the checks of the descriptor: a call that is turned away must not zero words
+    that an earlier launch on the device may still be counting in."""
+    from syncopate_amd import _lib
+
+    stream = _lib.stream_handle(torch.cuda.current_stream())
+    status = torch.zeros(_lib.SYN_STATUS_WORDS, dtype=torch.int32, device="cuda")
+    a, b, sizes, offsets, signals = _case(512, 256, 128, 2, 0, seed=2)
+    flags = torch.zeros(2, dtype=torch.int64, device="cuda")
+    c = torch.zeros(512, 256, dtype=torch.bfloat16, device="cuda")
+    d = _desc(_lib, a, b, c, flags, sizes, offsets, signals, None, status, 128, 128, 8)
+    _lib.check("syn_gemm_producer_static", hip.syn_gemm_producer_static(ctypes.byref(d), stream))
+    torch.cuda.synchronize()
+    peek = (ctypes.c_int32 * 2)()
+    _lib.check("syn_gemm_static_counters_peek", hip.syn_gemm_static_counters_peek(peek, 2))
+    assert list(peek) == [4, 4]
+    bad = _desc(_lib, a, b, c, flags, sizes, offsets, signals, None, status, 128, 64, 8)      # divides N, but no kernel has this tile shape
+    assert hip.syn_gemm_producer_static(ctypes.byref(bad), stream) == _lib.SYN_EINVAL
+    bad = _desc(_lib, a, b, c, flags, sizes, offsets, signals, None, status, 128, 128, 8)
+    bad.a = a.data_ptr() + 2                                                                   # misaligned operand
+    assert hip.syn_gemm_producer_static(ctypes.byref(bad), stream) == _lib.SYN_EALIGN
+    torch.cuda.synchronize()
+    _lib.check("syn_gemm_static_counters_peek", hip.syn_gemm_static_counters_peek(peek, 2))
+    assert list(peek) == [4, 4]
