@@ -47,8 +47,6 @@ from .work_plan import WorkPlan, plan_attention_work
 BLOCK_M = 128
 BLOCK_N = 128
 DEFAULT_SPIN_TIMEOUT_US = 2_000_000
-# longest segment of an automatic plan, in visits (see work_plan.plan_attention_work)
-DEFAULT_PLAN_MAX_VISITS = 2
 
 
 @launches_on_stream
@@ -119,7 +117,10 @@ def attention_forward(
     `form="auto"` (what `attention()` passes): where none of the three options above, `causal`, `counter_ptr` or
     `visit_log` is given, the launcher reads the tables and takes the fastest form they allow - two q blocks per
     workgroup with the XCD remap where every wave holds an even number of q blocks, chained where the waves
-    also share their (z, h, q) ranges and `num_programs` is 0 or the pairs of a wave.  Results are the same
+    also share their (z, h, q) ranges and `num_programs` is 0 or the pairs of a wave.  With `causal` (and none of
+    the other options) it plans the visits itself where the tables pair up: `plan_attention_work` for one program
+    per compute unit (or `num_programs`), segments cut to a program's fair share of the kv blocks; the plan is
+    remembered with the caller's device tables.  Results are the same
     to rounding; what differs is which program a tile runs on, which only `visit_log` shows.
     """
     dev = require_cuda(q, k, v, signal_ptr)
@@ -186,7 +187,7 @@ def attention_forward(
             try:
                 plan = plan_attention_work(host_tables[0][:num_waves].tolist(), host_tables[1][:num_waves].tolist(),
                                            host_tables[2][:num_waves].tolist(), causal=True, num_programs=units,
-                                           max_visits=DEFAULT_PLAN_MAX_VISITS)
+                                           max_blocks="fair")
             except ValueError:
                 plan = False
             if caller_owned:

@@ -86,3 +86,29 @@ def test_tile_policy_picks_a_shape_whose_last_chunk_fills_the_machine():
     assert choose_tile(1024, 3584, 224, producer_bound=True, shapes=[(256, 256), (128, 128)]) == (128, 128)
     with pytest.raises(ValueError):
         choose_tile(100, 3584, 224, producer_bound=True)
+
+
+def test_trusted_flag_arrays_are_remembered_per_tensor_object():
+    """Launchers fence behind every flag wait unless the flag array has been declared trusted
+    (include/syncopate_hip.h, SYN_GEMM_ACQUIRE_ALWAYS); the declaration is for the tensor object, not for its
+    address or for views of it, and goes away with the tensor."""
+    import gc
+
+    import torch
+
+    from syncopate_amd.computation._launch import acquire_always, trust_flags
+
+    flags = torch.zeros(8, dtype=torch.int64)
+    other = torch.zeros(8, dtype=torch.int64)
+    assert acquire_always(flags) and acquire_always(other)
+    trust_flags(flags)
+    assert not acquire_always(flags)
+    assert acquire_always(other)
+    assert acquire_always(flags[2:])            # a view is another object: the conservative answer
+    key = id(flags)
+    del flags
+    gc.collect()
+    later = torch.zeros(8, dtype=torch.int64)
+    assert acquire_always(later)                 # whatever object now lives at that id is not trusted
+    from syncopate_amd.computation import _launch
+    assert key not in _launch._trusted_flags or _launch._trusted_flags.get(key) is None
