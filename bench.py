@@ -58,7 +58,7 @@ LEAD_ON_COMPUTE_STREAM = False       # see --lead-on-compute-stream
 LINK_CHUNK_US = 110                  # one 16.8 MB chunk over one xGMI link (~153 GB/s)
 
 SECTIONS = ("ag_gemm", "throttled", "mfma_ceiling", "library", "reduce", "box_copies", "gemm_rs", "attn_ag", "attn_a2a",
-            "cpu")
+            "attn_slot", "cpu")
 
 
 def _events(n):
@@ -830,6 +830,50 @@ def run_attention_a2a(device, launches=10, gated=True):
 
 # -------------------------------------------------------------------------------- CPU baselines
 
+def run_attention_slot(device, launches=10):
+    """What the pieces of the paired attention kernel's slot cost beside each other (`syn_probe_attn_slot`): the 64
+    MFMAs of a slot on register operands, fed from LDS through the kernel's reads, beside the other group's softmax,
+    with the fills, with the first fragments of a phase asked for early, on constant and on random operands.  Per
+    configuration: time and shader-clock cycles per slot, the clock the device held (cycles / time), and the rate
+    the slot's products run at, as a fraction of the matrix pipes' peak.  2048 matrix-pipe cycles per slot."""
+    from syncopate_amd import _lib
+
+    lib = _lib.load()
+    workgroups, iters = 256, 2000
+    pool = torch.randn((workgroups * 65536 + (32 << 20)) // 2, device=device).bfloat16()
+    sink = torch.empty(workgroups * 512, dtype=torch.float32, device=device)
+    cycles = torch.zeros(2, dtype=torch.int64, device=device)
+    stream = _lib.stream_handle(torch.cuda.current_stream())
+    PRODUCTS, SOFTMAX, LDS, FILLS, PREFETCH, RANDOM, PRIVATE = 1, 2, 4, 8, 16, 32, 64
+    configs = (("products_register_operands", PRODUCTS),
+               ("products_from_lds", PRODUCTS | LDS),
+               ("softmax_alone", SOFTMAX),
+               ("products_from_lds_beside_softmax", PRODUCTS | LDS | SOFTMAX),
+               ("products_from_lds_beside_softmax_with_fills", PRODUCTS | LDS | SOFTMAX | FILLS),
+               ("same_fragments_asked_for_a_phase_early", PRODUCTS | LDS | SOFTMAX | FILLS | PREFETCH),
+               ("same_fills_that_miss_the_l2", PRODUCTS | LDS | SOFTMAX | FILLS | PRIVATE),
+               ("products_register_operands_random", PRODUCTS | RANDOM),
+               ("products_from_lds_beside_softmax_with_fills_random", PRODUCTS | LDS | SOFTMAX | FILLS | RANDOM),
+               ("same_fragments_asked_for_a_phase_early_random", PRODUCTS | LDS | SOFTMAX | FILLS | PREFETCH | RANDOM))
+    out = {"workgroups": workgroups, "slots_per_launch": iters, "launches": launches, "matrix_pipe_cycles_per_slot": 2048}
+    flop_per_slot = workgroups * 4 * 64 * 32768.0
+    for name, what in (("warm-up", configs[-2][1]),) + configs:
+        def probe(i):
+            _lib.check("syn_probe_attn_slot", lib.syn_probe_attn_slot(pool.data_ptr(), pool.numel() * 2, workgroups, iters, what,
+                                                                     sink.data_ptr(), cycles.data_ptr(), stream))
+        ms = _timed(probe, launches, 2)
+        if name == "warm-up":           # the clock the device holds depends on what it has just been doing
+            continue
+        cyc = cycles.tolist()
+        per_slot = max(cyc) / iters
+        entry = {"ns_per_slot": ms * 1e6 / iters, "cycles_per_slot": per_slot, "clock_GHz": per_slot / (ms * 1e6 / iters)}
+        if what & PRODUCTS:
+            entry["products_tflops"] = flop_per_slot / (ms * 1e-3 / iters) / 1e12
+            entry["products_pct_bf16_mfma_peak"] = 100.0 * entry["products_tflops"] / MFMA_BF16_PEAK_TFLOPS
+        out[name] = entry
+    return out
+
+
 def _host_cpu():
     """What the CPU baselines ran on: the model string, the cores the host shows and the threads used.  A one-GPU box
     of the pool gives a job 16 cores whatever the host shows (OMP_NUM_THREADS is 16 there), so the baselines use
@@ -1158,6 +1202,8 @@ def main():
                                       pct_bf16_mfma_peak=100.0 * ag["flop"] / (ag["ms"] * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS)
     if "attn_a2a" in only:
         line["attn_all2all"] = run_attention_a2a(device, gated=gated)
+    if "attn_slot" in only:
+        line["attn_slot_probe"] = run_attention_slot(device)
     if "cpu" in only:
         line["cpu_baseline"] = cpu_baseline(state)
         line["cpu_baselines_other"] = cpu_baselines_other()

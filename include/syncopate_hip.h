@@ -481,6 +481,21 @@ int syn_probe_mfma_rate(float* sink, int32_t workgroups, int32_t iters, int32_t 
 int syn_probe_read_streams(const void* base, int64_t stream_bytes, int64_t stride_bytes, int32_t streams,
                            int32_t workgroups, void* sink, syn_stream_t stream);
 
+/* Measurement aid, no counterpart in the reference: the slot of the paired attention kernel, piece by piece.
+ * `workgroups` workgroups of eight wavefronts (two per SIMD) run `iters` slots; in a slot wavefronts 0-3 run that
+ * kernel's 64 MFMAs 32x32x16 and wavefronts 4-7 one softmax pass over 64 scores per lane, then all meet at a
+ * barrier.  `what` is a sum of: 1 the products run, 2 the softmax runs (a half that does not run only joins the
+ * barriers), 4 the products' K and V fragments come from LDS through the kernel's reads (else register
+ * operands), 8 every wavefront issues four 1 KB LDS-DMA fills per slot from `pool`, 16 (with 4) the first
+ * fragments of a phase are asked for in the tail of the previous one, 32 pseudo-random operands instead of a
+ * constant, 64 a workgroup's fills read a region of its own (L2 misses; else all workgroups read the same 32 KB
+ * piece per slot: L2 hits but for the first reader of an XCD).  pool: device memory of at least 65536 * workgroups + 32 MiB bytes, 16-byte aligned.  sink: device
+ * float[512 * workgroups].  cycles: device int64[2], the shader-clock cycles workgroup 0 spent in the loop
+ * (wavefront 0, wavefront 4); with the launch's duration they give the clock the device held.
+ * matrix-pipe cycles per slot: 2048. */
+int syn_probe_attn_slot(const void* pool, int64_t pool_bytes, int32_t workgroups, int32_t iters, int32_t what,
+                        float* sink, int64_t* cycles, syn_stream_t stream);
+
 /* Library/ABI version: major*10000 + minor*100 + patch. */
 int syn_version(void);
 

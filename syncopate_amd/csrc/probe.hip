@@ -143,6 +143,251 @@ read_streams_kernel(const u32x4_probe_t* __restrict__ base, int64_t stride_vecs,
     if ((mix.x ^ mix.y ^ mix.z ^ mix.w) == 0x9e3779b9u) sink[blockIdx.x] = mix;
 }
 
+
+// ---- the paired attention kernel's slot, piece by piece -------------------------------------------------------
+// A workgroup of eight wavefronts, two per SIMD, like attn_pair_kernel.  Per iteration ("slot") wavefronts 0-3
+// run that kernel's matrix products - 32 MFMAs 32x32x16 fed by transposing 8-byte LDS reads (P.V) and 32 fed by
+// 16-byte LDS reads (Q.K), the reads two steps ahead of their MFMA, same addresses and swizzles - and wavefronts
+// 4-7 one softmax pass over 64 scores per lane (maximum, exponentials, sum, conversion to 16-bit pairs).  Every
+// piece can be switched off, so that what each costs beside the others is measured and not inferred:
+//   kSlotProducts / kSlotSoftmax   which half of the workgroup works (the other only joins the barriers)
+//   kSlotLds        the products' K and V fragments come from LDS (else the loop runs on register operands)
+//   kSlotFills      every wavefront issues four 1 KB LDS-DMA fills per slot (the kernel's 64 KB per two slots)
+//   kSlotPrefetch   the first fragments of the next phase are asked for in the tail of the previous one
+//   kSlotRandom     LDS and the register operands hold pseudo-random values instead of one constant
+//   kSlotPrivate    a workgroup's fills read a region of its own (misses in the L2); else every workgroup reads the
+//                   same 32 KB piece per slot - one miss per XCD, then L2 hits, like programs that walk one head's K, V
+// A slot ends like the kernel's: wait for the wavefront's own LDS reads (and fills), then the barrier.
+constexpr int kSlotProducts = 1, kSlotSoftmax = 2, kSlotLds = 4, kSlotFills = 8, kSlotPrefetch = 16, kSlotRandom = 32,
+              kSlotPrivate = 64;
+constexpr int kSlotRowBytes = 256, kSlotBlockBytes = 32768;
+typedef short slot_s16x4_t __attribute__((ext_vector_type(4)));
+typedef short slot_s16x8_t __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) slot_s16x4_t* slot_lds_s16x4_ptr;
+typedef __attribute__((address_space(3))) void* slot_lds_ptr;
+typedef const __attribute__((address_space(1))) void* slot_global_ptr;
+
+__device__ __forceinline__ f32x16_t slot_mfma(bf16x8_t a, bf16x8_t b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ void slot_fills(unsigned char* lds, const unsigned char* src, int wave8, int lane) {
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int blk = i * 8 + wave8;
+        __builtin_amdgcn_global_load_lds((slot_global_ptr)(src + (size_t)blk * 1024 + lane * 16), (slot_lds_ptr)(lds + blk * 1024),
+                                         16, 0, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+__device__ __forceinline__ void slot_end(bool fills) {
+    __builtin_amdgcn_sched_barrier(0);
+    if (fills) __builtin_amdgcn_s_waitcnt(0x0070);      // vmcnt(0) lgkmcnt(0)
+    else __builtin_amdgcn_s_waitcnt(0xc07f);            // lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+template <bool LDS, bool PREFETCH>
+__device__ __forceinline__ void slot_products(int what, int iters, unsigned char* k_lds, unsigned char* v_lds,
+                                              const unsigned char* pool, float* sink) {
+    const int lane = threadIdx.x & 63, wave8 = threadIdx.x >> 6, r = lane & 31, half = lane >> 5;
+    const bool fills = (what & kSlotFills) != 0;
+    const int k_rd = r * kSlotRowBytes;
+    const int i16 = lane & 15;
+    const int v_row = 4 * half + (i16 >> 2);
+    const int v_col_bytes = (16 * ((lane >> 4) & 1) + 4 * (i16 & 3)) * 2;
+    const int v_swz = (i16 >> 2) << 2;
+    int v_rd[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        v_rd[i] = v_row * kSlotRowBytes + ((((4 * i + (v_col_bytes >> 4)) ^ v_swz) << 4) | (v_col_bytes & 15));
+    const int k_swz = (half ^ (r & 15)) << 4;
+    const int pattern = (what & kSlotRandom) ? 2 : 1;
+    f32x16_t o_acc[4], s[4];
+    bf16x8_t qf[8], pf[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) { o_acc[i][e] = 0.f; s[i][e] = 0.f; }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        qf[i] = probe_fragment(pattern, threadIdx.x * 16 + i);
+        pf[i] = probe_fragment(pattern, threadIdx.x * 16 + 8 + i);
+    }
+    slot_s16x4_t vlo[2][4], vhi[2][4];
+    bf16x8_t kf[2][4];
+    auto v_first = [&](const unsigned char* v_blk, int b, int i) __attribute__((always_inline)) {
+        const unsigned char* src = v_blk + 16 * b * kSlotRowBytes + v_rd[i];
+        vlo[b][i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((slot_lds_s16x4_ptr)src);
+        vhi[b][i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((slot_lds_s16x4_ptr)(src + 8 * kSlotRowBytes));
+    };
+    if (LDS && PREFETCH) {
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v_first(v_lds, b, i);
+    }
+    for (int it = 0; it < iters; ++it) {
+        if (fills)
+            slot_fills((it & 1) ? k_lds + ((it + 1) & 1) * kSlotBlockBytes : v_lds + (it & 1) * kSlotBlockBytes,
+                       pool + (size_t)(it & 1023) * kSlotBlockBytes, wave8, lane);
+        if (!LDS) {
+#pragma unroll
+            for (int t2 = 0; t2 < 8; ++t2)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) o_acc[i] = slot_mfma(qf[t2], pf[t2], o_acc[i]);
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) s[j] = slot_mfma(pf[ks], qf[ks], s[j]);
+        } else {
+            const unsigned char* v_blk = v_lds + (it & 1) * kSlotBlockBytes;
+            const unsigned char* v_nxt = v_lds + ((it + 1) & 1) * kSlotBlockBytes;
+            const unsigned char* k_row = k_lds + (it & 1) * kSlotBlockBytes + k_rd;
+            int swz = k_swz;
+            asm volatile("" : "+v"(swz));
+            auto k_read = [&](int b, int j, int ks) __attribute__((always_inline)) {
+                kf[b][j] = *reinterpret_cast<const bf16x8_t*>(k_row + 32 * j * kSlotRowBytes + (swz ^ (32 * ks)));
+            };
+            // O^T += V^T . P^T
+            if (!PREFETCH) {
+#pragma unroll
+                for (int b = 0; b < 2; ++b)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) v_first(v_blk, b, i);
+                __builtin_amdgcn_sched_group_barrier(0x100, 16, 0);
+            }
+#pragma unroll
+            for (int t2 = 0; t2 < 8; ++t2) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const slot_s16x4_t lo = vlo[t2 & 1][i], hi = vhi[t2 & 1][i];
+                    const slot_s16x8_t both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    o_acc[i] = slot_mfma(__builtin_bit_cast(bf16x8_t, both), pf[t2], o_acc[i]);
+                    if (t2 + 2 < 8) {
+                        const unsigned char* src = v_blk + 16 * (t2 + 2) * kSlotRowBytes + v_rd[i];
+                        vlo[t2 & 1][i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((slot_lds_s16x4_ptr)src);
+                        vhi[t2 & 1][i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((slot_lds_s16x4_ptr)(src + 8 * kSlotRowBytes));
+                    } else if (PREFETCH) {
+                        k_read(t2 & 1, i, t2 & 1);           // the first two steps of Q.K, asked for in the tail of P.V
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    if (t2 + 2 < 8) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                    else if (PREFETCH) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                }
+            }
+            // S^T = K . Q^T
+            if (!PREFETCH) {
+#pragma unroll
+                for (int b = 0; b < 2; ++b)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) k_read(b, j, b);
+                __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+            }
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    s[j] = slot_mfma(kf[ks & 1][j], qf[ks], s[j]);
+                    if (ks + 2 < 8) k_read(ks & 1, j, ks + 2);
+                    else if (PREFETCH) v_first(v_nxt, ks & 1, j);   // the next slot's first two steps of P.V
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    if (ks + 2 < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    else if (PREFETCH) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                }
+            }
+        }
+        slot_end(fills);
+    }
+    float t = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) t += o_acc[i][e] + s[i][e];
+    if (LDS && PREFETCH) t += (float)vlo[0][0][0] + (float)vhi[1][3][1];
+    sink[blockIdx.x * 512 + threadIdx.x] = t;
+}
+
+__device__ __forceinline__ void slot_softmax(int what, int iters, unsigned char* k_lds, unsigned char* v_lds,
+                                             const unsigned char* pool, float* sink) {
+    const int lane = threadIdx.x & 63, wave8 = threadIdx.x >> 6;
+    const bool fills = (what & kSlotFills) != 0;
+    float s[64];
+#pragma unroll
+    for (int e = 0; e < 64; ++e) s[e] = (float)(probe_hash(threadIdx.x * 64 + e) & 0xffff) * (1.0f / 4096.f);
+    float m_i = -1e30f, l_i = 0.f;
+    unsigned packed = 0;
+    for (int it = 0; it < iters; ++it) {
+        if (fills)
+            slot_fills((it & 1) ? k_lds + ((it + 1) & 1) * kSlotBlockBytes : v_lds + (it & 1) * kSlotBlockBytes,
+                       pool + (size_t)(it & 1023) * kSlotBlockBytes, wave8, lane);
+#pragma unroll
+        for (int e = 0; e < 64; ++e) asm volatile("" : "+v"(s[e]));      // new scores every slot, as far as the compiler knows
+        float mx = -1e30f;
+#pragma unroll
+        for (int e = 0; e < 64; ++e) mx = fmaxf(mx, s[e]);
+        const float m_new = fmaxf(m_i, mx * 0.088f);
+        const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
+        float row = 0.f;
+#pragma unroll
+        for (int e = 0; e < 64; e += 2) {
+            const float p0 = __builtin_amdgcn_exp2f(s[e] * 0.088f - m_new);
+            const float p1 = __builtin_amdgcn_exp2f(s[e + 1] * 0.088f - m_new);
+            row += p0;
+            row += p1;
+            typedef __bf16 bf16x2_slot_t __attribute__((ext_vector_type(2)));
+            const bf16x2_slot_t pk = {(__bf16)p0, (__bf16)p1};
+            unsigned u = __builtin_bit_cast(unsigned, pk);
+            asm volatile("" : "+v"(u));
+            packed ^= u;
+        }
+        l_i = l_i * alpha + row;
+        m_i = m_new;
+        slot_end(fills);
+    }
+    sink[blockIdx.x * 512 + threadIdx.x] = l_i + m_i + (float)packed;
+}
+
+template <bool LDS, bool PREFETCH>
+__global__ void __launch_bounds__(512, 1) attn_slot_kernel(int what, int iters, const unsigned char* pool, float* sink,
+                                                           long long* cycles) {
+    __shared__ __attribute__((aligned(1024))) unsigned char k_lds[2 * kSlotBlockBytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char v_lds[2 * kSlotBlockBytes];
+    for (int i = threadIdx.x; i < 2 * kSlotBlockBytes / 4; i += 512) {
+        unsigned a = 0x3c003c00u, b = 0x3c003c00u;
+        if (what & kSlotRandom) {
+            const bf16x8_t f = probe_fragment(2, blockIdx.x * 65536 + i);
+            const u32x4_probe_t w = __builtin_bit_cast(u32x4_probe_t, f);
+            a = w[0];
+            b = w[1];
+        }
+        reinterpret_cast<unsigned*>(k_lds)[i] = a;
+        reinterpret_cast<unsigned*>(v_lds)[i] = b;
+    }
+    __syncthreads();
+    const int wave8 = threadIdx.x >> 6;
+    const unsigned char* mine = (what & kSlotPrivate) ? pool + (size_t)blockIdx.x * 65536 : pool;
+    const long long t0 = clock64();
+    if (wave8 < 4) {
+        if (what & kSlotProducts) slot_products<LDS, PREFETCH>(what, iters, k_lds, v_lds, mine, sink);
+        else for (int it = 0; it < iters; ++it) __builtin_amdgcn_s_barrier();
+    } else {
+        if (what & kSlotSoftmax) slot_softmax(what, iters, k_lds, v_lds, mine, sink);
+        else for (int it = 0; it < iters; ++it) __builtin_amdgcn_s_barrier();
+    }
+    const long long t1 = clock64();
+    if (blockIdx.x == 0 && (threadIdx.x & 255) == 0) cycles[wave8 >> 2] = t1 - t0;
+}
+
 }  // namespace syn
 
 extern "C" int syn_probe_read_streams(const void* base, int64_t stream_bytes, int64_t stride_bytes, int32_t streams,
@@ -174,5 +419,24 @@ extern "C" int syn_probe_mfma_rate(float* sink, int32_t workgroups, int32_t iter
     else
         hipLaunchKernelGGL(mfma_rate_kernel, dim3(workgroups), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), sink,
                            iters, pattern);
+    return (int)hipGetLastError();
+}
+
+extern "C" int syn_probe_attn_slot(const void* pool, int64_t pool_bytes, int32_t workgroups, int32_t iters, int32_t what,
+                                   float* sink, int64_t* cycles, syn_stream_t stream) {
+    using namespace syn;
+    if (pool == nullptr || sink == nullptr || cycles == nullptr || workgroups <= 0 || iters <= 0) return SYN_EINVAL;
+    if (what <= 0 || what >= 128 || !(what & (kSlotProducts | kSlotSoftmax))) return SYN_EINVAL;
+    if ((what & kSlotPrefetch) && !(what & kSlotLds)) return SYN_EINVAL;
+    // a workgroup's fills read 32 KB pieces at pool (+ 64 KB * workgroup with kSlotPrivate) + 32 KB * (slot % 1024)
+    if (pool_bytes < (int64_t)workgroups * 65536 + 1024 * (int64_t)kSlotBlockBytes) return SYN_EINVAL;
+    if (!aligned16(pool)) return SYN_EALIGN;
+    const unsigned char* g = reinterpret_cast<const unsigned char*>(pool);
+    long long* c = reinterpret_cast<long long*>(cycles);
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const dim3 grid(workgroups), block(512);
+    if (!(what & kSlotLds)) hipLaunchKernelGGL((attn_slot_kernel<false, false>), grid, block, 0, s, what, iters, g, sink, c);
+    else if (what & kSlotPrefetch) hipLaunchKernelGGL((attn_slot_kernel<true, true>), grid, block, 0, s, what, iters, g, sink, c);
+    else hipLaunchKernelGGL((attn_slot_kernel<true, false>), grid, block, 0, s, what, iters, g, sink, c);
     return (int)hipGetLastError();
 }

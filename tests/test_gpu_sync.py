@@ -125,3 +125,35 @@ def test_flag_write_as_a_stream_memory_operation(hip):
     side.synchronize()
     assert flags.tolist() == [0, 0, 1, 0]
     assert hip.syn_flag_write_value(None, 1, _lib.stream_handle(side)) == _lib.SYN_EINVAL
+
+
+def test_attention_slot_probe_runs_every_piece_and_rejects_bad_arguments(hip):
+    """syn_probe_attn_slot: every combination of pieces runs to completion on a few workgroups and reports the
+    cycles of both halves; the argument checks of the entry point."""
+    from syncopate_amd import _lib
+
+    stream = _lib.stream_handle(torch.cuda.current_stream())
+    workgroups, iters = 4, 3
+    needed = workgroups * 65536 + (32 << 20)
+    pool = torch.zeros(needed + 64, dtype=torch.uint8, device="cuda")
+    sink = torch.zeros(workgroups * 512, dtype=torch.float32, device="cuda")
+    cycles = torch.zeros(2, dtype=torch.int64, device="cuda")
+
+    def run(what, nbytes=needed, wg=workgroups):
+        return hip.syn_probe_attn_slot(pool.data_ptr(), nbytes, wg, iters, what, sink.data_ptr(), cycles.data_ptr(), stream)
+
+    for what in (1, 2, 3, 1 | 4, 3 | 4, 3 | 4 | 8, 3 | 4 | 8 | 16, 3 | 4 | 8 | 32, 1 | 4 | 16, 2 | 8, 3 | 4 | 8 | 64):
+        cycles.zero_()
+        _lib.check("syn_probe_attn_slot", run(what))
+        torch.cuda.synchronize()
+        assert min(cycles.tolist()) > 0, what
+        assert torch.isfinite(sink).all()
+    assert run(0) == _lib.SYN_EINVAL
+    assert run(128) == _lib.SYN_EINVAL
+    assert run(4) == _lib.SYN_EINVAL                 # operands from LDS, but neither half runs
+    assert run(1 | 16) == _lib.SYN_EINVAL            # early fragments without LDS reads
+    assert run(3, nbytes=needed - 1) == _lib.SYN_EINVAL
+    assert run(3, wg=0) == _lib.SYN_EINVAL
+    assert hip.syn_probe_attn_slot(None, needed, workgroups, iters, 3, sink.data_ptr(), cycles.data_ptr(), stream) == _lib.SYN_EINVAL
+    assert hip.syn_probe_attn_slot(pool.data_ptr() + 8, needed, workgroups, iters, 3, sink.data_ptr(),
+                                   cycles.data_ptr(), stream) == _lib.SYN_EALIGN
