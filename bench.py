@@ -853,6 +853,8 @@ def run_attention_slot(device, launches=10):
                ("same_fragments_asked_for_a_phase_early", PRODUCTS | LDS | SOFTMAX | FILLS | PREFETCH),
                ("same_fills_that_miss_the_l2", PRODUCTS | LDS | SOFTMAX | FILLS | PRIVATE),
                ("products_register_operands_random", PRODUCTS | RANDOM),
+               ("products_from_lds_random", PRODUCTS | LDS | RANDOM),
+               ("products_from_lds_beside_softmax_random", PRODUCTS | LDS | SOFTMAX | RANDOM),
                ("products_from_lds_beside_softmax_with_fills_random", PRODUCTS | LDS | SOFTMAX | FILLS | RANDOM),
                ("same_fragments_asked_for_a_phase_early_random", PRODUCTS | LDS | SOFTMAX | FILLS | PREFETCH | RANDOM))
     out = {"workgroups": workgroups, "slots_per_launch": iters, "launches": launches, "matrix_pipe_cycles_per_slot": 2048}
