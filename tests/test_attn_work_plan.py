@@ -327,3 +327,39 @@ def test_kernel_reports_a_list_that_breaks_a_segment(hip):
         template._lib.load().syn_attn_check_work_list = real
     with pytest.raises(RuntimeError, match="kernel status"):
         _launch.check_status()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("form", ["auto", "planned", "pairs", "tiles"])
+def test_causal_attention_of_a_q_shard_that_does_not_start_at_zero(hip, form):
+    """A rank's q rows [512, 1024) against kv gathered in four chunks (arrival order 1, 0, 3, 2) under a causal
+    mask: q positions are the table's q offsets (syncopate/computation/attn/template.py:80-121 takes `offs_m` from
+    the wave's q start, for the addresses and for the mask alike).  The chunk wholly above the shard's first q
+    blocks is a visit that costs nothing; rows outside the shard are not written.  Every launch form gives the
+    masked softmax of torch."""
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.attn import attention_forward
+
+    H, S, lo, chunk, order = 2, 1024, 512, 256, [1, 0, 3, 2]
+    q, k, v = _qkv(1, H, S, torch.bfloat16, seed=21)
+    offsets = [[0, 0, lo, c * chunk] for c in order]
+    sizes = [[1, H, S - lo, chunk]] * len(order)
+    cums = [(i + 1) * H * (S - lo) for i in range(len(order))]
+    signals = [-1, 0, 1, 2]
+    flags = torch.ones(3, dtype=torch.int64, device="cuda")
+    kw = dict(wave_offsets=offsets, wave_sizes=sizes, cum_wave_sizes=cums, signal_ptr=flags, signal_offsets=signals,
+              cum_tiles=cums[-1], causal=True)
+    if form == "planned":
+        plan = plan_attention_work(offsets, sizes, cums, causal=True, num_programs=3, max_visits=2)
+        assert any(vis.kv_blocks == 0 for vis in table_visits(offsets, sizes, cums, causal=True))
+        kw.update(pair_q_blocks=True, work_plan=plan)
+    elif form == "pairs":
+        kw.update(pair_q_blocks=True, num_programs=5)
+    elif form == "auto":
+        kw.update(form="auto")
+    out = torch.full((1, H, S, 128), 7.0, dtype=torch.bfloat16, device="cuda")
+    o = attention_forward(q.cuda(), k.cuda(), v.cuda(), 128 ** -0.5, out=out, **kw)
+    check_status()
+    ref = numerics.sdpa_fp32(q, k, v, 128 ** -0.5, causal=True)
+    assert _rel(o[:, :, lo:], ref[:, :, lo:]) <= REL_TOL
+    assert (o[:, :, :lo] == 7.0).all()
