@@ -99,7 +99,7 @@ def attention_forward(
     `pair_q_blocks` (an extension): one workgroup of eight wavefronts takes two consecutive q
     blocks and runs them half a kv block apart, the softmax of one beside the matrix products of
     the other, both reading K and V from the same LDS blocks.  Every wave must hold an even
-    number of q blocks; not with `causal` or `counter_ptr`.
+    number of q blocks (with `causal`: q and kv ranges that begin at even blocks); not with `counter_ptr`.
     `xcd_remap` (an extension): the workgroups of one XCD take consecutive tiles (the q blocks of
     one head), so that a head's K and V are fetched into one L2 instead of eight.
     `chain_q_blocks` (an extension, with `pair_q_blocks`): for tables whose waves all list the same
@@ -117,10 +117,11 @@ def attention_forward(
     `form="auto"` (what `attention()` passes): where none of the three options above, `causal`, `counter_ptr` or
     `visit_log` is given, the launcher reads the tables and takes the fastest form they allow - two q blocks per
     workgroup with the XCD remap where every wave holds an even number of q blocks, chained where the waves
-    also share their (z, h, q) ranges and `num_programs` is 0 or the pairs of a wave.  With `causal` (and none of
-    the other options) it plans the visits itself where the tables pair up: `plan_attention_work` for one program
-    per compute unit (or `num_programs`), segments cut to a program's fair share of the kv blocks; the plan is
-    remembered with the caller's device tables.  Results are the same
+    also share their (z, h, q) ranges and `num_programs` is 0 or the pairs of a wave.  Where the waves cover
+    different q ranges (the all-to-all table), and with `causal` (and none of the other options), it plans the
+    visits itself where the tables pair up: `plan_attention_work` for one program per compute unit (or
+    `num_programs`), segments cut to a program's fair share of the kv blocks; the plan is remembered with the
+    caller's device tables.  Results are the same
     to rounding; what differs is which program a tile runs on, which only `visit_log` shows.
     """
     dev = require_cuda(q, k, v, signal_ptr)
@@ -175,23 +176,31 @@ def attention_forward(
     host_tables = None
     if form not in ("explicit", "auto"):
         raise ValueError("form must be 'explicit' or 'auto'")
-    if form == "auto" and causal and not (pair_q_blocks or chain_q_blocks or xcd_remap or counter_ptr is not None
-                                          or consumer_signal_ptr is not None or visit_log is not None
-                                          or work_plan is not None):
-        # under a causal mask the visits differ in cost and many cost nothing: a planned launch of one program per
-        # compute unit where the tables pair up, the one-tile-per-program kernel where they do not
+    def planned_by_the_launcher(with_mask: bool):
+        """A work plan for these tables (one program per compute unit, or `num_programs`; segments cut to a program's
+        fair share of the kv blocks), remembered with the caller's device tables; False where the tables do not pair up."""
+        nonlocal host_tables
         units = num_programs or torch.cuda.get_device_properties(dev).multi_processor_count
-        plan = recall_note(tables, f"causal work plan {units}") if caller_owned else None
+        note = f"work plan, causal {int(with_mask)}, {units} programs"
+        plan = recall_note(tables, note) if caller_owned else None
         if plan is None:
-            host_tables = (host_copy(offs), host_copy(sizes), host_copy(cums), host_copy(sigs))
+            host_tables = host_tables or (host_copy(offs), host_copy(sizes), host_copy(cums), host_copy(sigs))
             try:
                 plan = plan_attention_work(host_tables[0][:num_waves].tolist(), host_tables[1][:num_waves].tolist(),
-                                           host_tables[2][:num_waves].tolist(), causal=True, num_programs=units,
+                                           host_tables[2][:num_waves].tolist(), causal=with_mask, num_programs=units,
                                            max_blocks="fair")
             except ValueError:
                 plan = False
             if caller_owned:
-                remember_note(tables, f"causal work plan {units}", plan)
+                remember_note(tables, note, plan)
+        return plan
+
+    if form == "auto" and causal and not (pair_q_blocks or chain_q_blocks or xcd_remap or counter_ptr is not None
+                                          or consumer_signal_ptr is not None or visit_log is not None
+                                          or work_plan is not None):
+        # under a causal mask the visits differ in cost and many cost nothing: a planned launch where the tables pair
+        # up, the one-tile-per-program kernel where they do not
+        plan = planned_by_the_launcher(True)
         if plan:
             pair_q_blocks = xcd_remap = True
             work_plan, num_programs = plan, plan.num_programs
@@ -199,7 +208,7 @@ def attention_forward(
                                or consumer_signal_ptr is not None or visit_log is not None):
         choice = recall_note(tables, "attention form") if caller_owned else None
         if choice is None:
-            host_tables = (host_copy(offs), host_copy(sizes), host_copy(cums), host_copy(sigs))
+            host_tables = host_tables or (host_copy(offs), host_copy(sizes), host_copy(cums), host_copy(sigs))
             ho, hs, hc, _ = host_tables
             real = [i for i in range(num_waves) if int(hc[i]) > 0]
             even = bool(real) and all(int(hs[i, 2]) % (2 * BLOCK_M) == 0 for i in real)
@@ -214,6 +223,12 @@ def attention_forward(
             pair_q_blocks = xcd_remap = True
             if pairs and num_programs in (0, pairs):
                 chain_q_blocks, num_programs = True, pairs
+            elif not pairs:
+                # waves over different q ranges (the all-to-all table): the visits to a pair of q blocks are planned as
+                # segments that keep their sums in registers, instead of one merge into the output per visit
+                plan = planned_by_the_launcher(False)
+                if plan:
+                    work_plan, num_programs = plan, plan.num_programs
     given_programs = num_programs
     if chain_q_blocks and num_programs <= 0 and caller_owned:
         # filled in by an earlier call on these tables; `already_checked` below vouches for it
