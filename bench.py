@@ -1207,6 +1207,13 @@ def main():
         line["attn_all2all"] = run_attention_a2a(device, gated=gated)
     if "attn_slot" in only:
         line["attn_slot_probe"] = run_attention_slot(device)
+        slot = line["attn_slot_probe"]["products_from_lds_beside_softmax_with_fills_random"]["products_tflops"]
+        # the kernels' rates against the bare slot loop's (same MFMAs, LDS reads, softmax and fills on random operands,
+        # nothing else): what is left is the kernels' own doing, the rest is the board's power limit
+        if "attn_allgather" in line:
+            line["attn_allgather"]["frac_of_slot_loop_on_random_operands"] = line["attn_allgather"]["tflops"] / slot
+        if "attn_all2all" in line:
+            line["attn_all2all"]["non_causal_frac_of_slot_loop_on_random_operands"] = line["attn_all2all"]["non_causal_tflops"] / slot
     if "cpu" in only:
         line["cpu_baseline"] = cpu_baseline(state)
         line["cpu_baselines_other"] = cpu_baselines_other()
