@@ -548,8 +548,9 @@ def run_gemm_rs(device, steps, warmup, gated=True):
     from syncopate_amd.computation.gemm import gemm_rs_producer_persistent
     owners = [torch.zeros(rows, n, dtype=torch.bfloat16, device=device) for _ in range(world)]
     targets = [row // rows for row, _ in tables.block_offsets]
+    owner_table = _table(targets, device)
     def direct():
-        gemm_rs_producer_persistent(a, b, owners, sizes, offsets, targets, world, world, 256, 256, 256, BK, GROUP_M)
+        gemm_rs_producer_persistent(a, b, owners, sizes, offsets, owner_table, world, world, 256, 256, 256, BK, GROUP_M)
     direct()
     torch.cuda.synchronize()
     direct_matches = True
@@ -558,11 +559,41 @@ def run_gemm_rs(device, steps, warmup, gated=True):
         direct_matches = direct_matches and bool(((owners[p][5:6].float() - ref).abs().max() / ref.abs().max()) < 1e-2)
     direct_ms = _timed(lambda i: direct(), steps, max(3, warmup // 4))
     check_status()
+    # A third form, from the same per-wave peer bindings with a plain store (RemoteBinding without a reduction,
+    # transform/transformer.py:1158-1178): the epilogue writes every tile straight into this rank's slot of its
+    # owner's receive buffer - no pushes, so nothing beside the GEMM needs compute units and all 256 programs run -
+    # and the chunked reduce follows.  The same bytes land in the same places as in the fused step.
+    from syncopate_amd.computation.gemm import gemm_remote
+    peers = ctx.comm_buffers["dst"]
+    slots = [src[RANK * rows:(RANK + 1) * rows] if p == RANK else peers[p][RANK] for p in range(world)]
+    slot_offsets = torch.tensor(tables.block_offsets, dtype=torch.int32)
+    slot_offsets[:, 0] = 0                       # rows are wave-local in the owner's slot, columns keep their place
+    slot_offsets, owner_of_wave = slot_offsets.to(device), _table(targets, device)
+    for p in (1, 4, 7):
+        peers[p][RANK].zero_()
+
+    def stored(reduce=True):
+        gemm_remote(a, b, slots, 256, 256, 256, BK, GROUP_M, cur_wave_sizes=sizes, wave_offsets=offsets, M=m,
+                    target_rank=owner_of_wave, dst_offsets=slot_offsets, cum_tiles=tables.cum_tiles)
+        if reduce:
+            ring_reduce(dst, out, src, RANK)
+    stored()
+    torch.cuda.synchronize()
+    stored_matches = all(torch.equal(peers[p][RANK], src[p * rows:(p + 1) * rows]) for p in (1, 4, 7))
+    acc = src[RANK * rows:(RANK + 1) * rows][sample].clone()
+    for i in range(1, world):
+        acc = acc + dst[(RANK + i) % world][sample]
+    stored_matches = stored_matches and torch.equal(out[sample], acc)
+    stored_ms = _timed(lambda i: stored(), steps, max(3, warmup // 4))
+    stored_gemm_ms = _timed(lambda i: stored(reduce=False), steps, max(3, warmup // 4))
+    check_status()
     return {"launches": steps, "producer_ms": producer_ms, "producer_ms_without_xcd_remap": no_remap_ms,
             "flop": 2.0 * m * n * k, "fused_step_ms": fused_ms,
             "fused_step_ms_by_programs": {str(k_): v for k_, v in fused_by_programs.items()},
             "reduce_matches": bool(reduce_matches), "pushed_chunks_match": bool(pushed),
-            "direct_reduce_form_ms": direct_ms, "direct_reduce_form_matches": direct_matches}
+            "direct_reduce_form_ms": direct_ms, "direct_reduce_form_matches": direct_matches,
+            "remote_store_form_ms": stored_ms, "remote_store_form_gemm_ms": stored_gemm_ms,
+            "remote_store_form_matches": bool(stored_matches)}
 
 
 # ------------------------------------------------------------------------------------ attention
@@ -1196,6 +1227,11 @@ def main():
                 "direct_reduce_form_ms": rs["direct_reduce_form_ms"],
                 "direct_reduce_form_tflops": rs["flop"] / (rs["direct_reduce_form_ms"] * 1e-3) / 1e12,
                 "direct_reduce_form_matches": rs["direct_reduce_form_matches"],
+                "remote_store_form_ms": rs["remote_store_form_ms"],
+                "remote_store_form_gemm_ms": rs["remote_store_form_gemm_ms"],
+                "remote_store_form_tflops": rs["flop"] / (rs["remote_store_form_ms"] * 1e-3) / 1e12,
+                "remote_store_form_over_producer_pct": 100.0 * (rs["remote_store_form_ms"] - rs["producer_ms"]) / rs["producer_ms"],
+                "remote_store_form_matches": rs["remote_store_form_matches"],
                 "reduce_matches": rs["reduce_matches"],
                 "pushed_chunks_match": rs["pushed_chunks_match"],
             })

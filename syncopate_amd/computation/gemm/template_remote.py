@@ -25,8 +25,8 @@ from typing import Optional, Sequence
 import torch
 
 from ... import _lib
-from .._launch import (TableLike, acquire_always, as_device_table, host_copy, host_ptr, launches_on_stream, require_cuda,
-                       status_words)
+from .._launch import (TableLike, acquire_always, as_device_table, host_copy, host_ptr, launches_on_stream, recall_note,
+                       remember_note, require_cuda, status_words)
 
 _pointer_tables: dict = {}
 
@@ -53,6 +53,66 @@ def _check_ranks(name: str, ranks: torch.Tensor, count: int, num_waves: int) -> 
 
 
 @launches_on_stream
+def _prepare_binding(lib, sizes, offsets, signals, flags, num_waves, M, N, K, block_m, block_n, block_k, cum_tiles,
+                     a_list, a_target_rank, c_list, target_rank, dst_offsets, atomic_add, k_ranges, dev):
+    """The host's share of a bound launch: table checks, and the device tables the kernel reads (pointer tables,
+    ranks, destination offsets, k ranges).  Returns the fields of the remote descriptor and the tensors they point into."""
+    hs, ho, hg = host_copy(sizes), host_copy(offsets), host_copy(signals)
+    _lib.check("syn_gemm_check_waves",
+               lib.syn_gemm_check_waves(host_ptr(hs), host_ptr(ho), host_ptr(hg), num_waves, M, N, K,
+                                        block_m, block_n, block_k, int(cum_tiles), flags.numel()))
+    fields, keep = {}, []
+    if a_list is not None:
+        if a_target_rank is None:
+            raise ValueError("a list of A shards needs a_target_rank")
+        a_ranks = as_device_table(a_target_rank, dev, None)
+        _check_ranks("a_target_rank", a_ranks, len(a_list), num_waves)
+        shard_rows = min(t.shape[0] for t in a_list)
+        if int(hs[:, 0].max()) > shard_rows:
+            raise ValueError("a wave has more rows than an A shard")
+        table = _pointer_table(a_list, dev)
+        keep += [a_ranks, table]
+        fields.update(a_peers=table.data_ptr(), a_target_rank=a_ranks.data_ptr())
+    if c_list is not None:
+        if target_rank is None or dst_offsets is None:
+            raise ValueError("a list of C buffers needs target_rank and dst_offsets")
+        c_ranks = as_device_table(target_rank, dev, None)
+        dst = as_device_table(dst_offsets, dev, 2)
+        _check_ranks("target_rank", c_ranks, len(c_list), num_waves)
+        ldc = c_list[0].shape[1]
+        rows = min(t.shape[0] for t in c_list)
+        if any(t.shape[1] != ldc for t in c_list) or ldc % 4:
+            raise ValueError("peer C buffers must share one row length, a multiple of 4")
+        hd = host_copy(dst)
+        if dst.shape[0] < num_waves or int(hd.min()) < 0:
+            raise ValueError("dst_offsets must hold one non-negative (row, col) pair per wave")
+        if int((hd[:num_waves, 0] + hs[:, 0]).max()) > rows or int((hd[:num_waves, 1] + hs[:, 1]).max()) > ldc:
+            raise ValueError("a wave's destination region does not fit the peer C buffer")
+        if int(hd[:num_waves, 1].max()) % 4:
+            raise ValueError("dst column offsets must be multiples of 4 elements")
+        table = _pointer_table(c_list, dev)
+        keep += [c_ranks, dst, table]
+        fields.update(c_peers=table.data_ptr(), c_target_rank=c_ranks.data_ptr(), c_dst_offsets=dst.data_ptr(), c_ld=ldc,
+                      c_atomic_add=1 if atomic_add else 0)
+    elif atomic_add:
+        raise ValueError("atomic_add needs c bound to peers")
+    if k_ranges is not None:
+        if c_list is None or not atomic_add:
+            raise ValueError("k_ranges produce partial products: c must be bound and added into (atomic_add)")
+        ranges = as_device_table(k_ranges, dev, 2)
+        hk = host_copy(ranges)
+        if ranges.shape[0] < num_waves:
+            raise ValueError("k_ranges is shorter than the wave tables")
+        k0, kn = hk[:num_waves, 0], hk[:num_waves, 1]
+        if int(k0.min()) < 0 or int(kn.min()) <= 0 or int((k0 % 64).max()) or int((kn % 64).max()):
+            raise ValueError("k ranges must start at and span positive multiples of 64")
+        if int((k0 + kn).max()) > K:
+            raise ValueError("a k range runs past K")
+        keep.append(ranges)
+        fields["k_ranges"] = ranges.data_ptr()
+    return fields, keep
+
+
 def gemm_remote(
     a,
     b: torch.Tensor,
@@ -126,62 +186,26 @@ def gemm_remote(
         flags = signal_ptr
 
     lib = _lib.load()
-    hs, ho, hg = host_copy(sizes), host_copy(offsets), host_copy(signals)
-    _lib.check("syn_gemm_check_waves",
-               lib.syn_gemm_check_waves(host_ptr(hs), host_ptr(ho), host_ptr(hg), num_waves, M, N, K,
-                                        BLOCK_SIZE_M, BLOCK_SIZE_N, BLOCK_SIZE_K, int(cum_tiles), flags.numel()))
-
+    # What the host works out from the tables - the checks, the pointer tables, the converted rank and offset
+    # tables - is kept with the caller's device tables (per tensor objects and versions), so that a launch repeated
+    # on the same operands costs no device-to-host copy.
+    given = [t for t in (cur_wave_sizes, wave_offsets, signal_offsets, a_target_rank, target_rank, dst_offsets, k_ranges)
+             if t is not None]
+    caller_owned = all(isinstance(t, torch.Tensor) and t.is_cuda for t in given)
+    params = (M, N, K, BLOCK_SIZE_M, BLOCK_SIZE_N, BLOCK_SIZE_K, int(cum_tiles), flags.numel(), bool(atomic_add),
+              None if a_list is None else tuple((t.data_ptr(), t.shape[0]) for t in a_list),
+              None if c_list is None else tuple((t.data_ptr(), tuple(t.shape)) for t in c_list))
+    prepared = recall_note(given, "remote binding") if caller_owned else None
+    if prepared is None or prepared[0] != params:
+        prepared = (params, _prepare_binding(lib, sizes, offsets, signals, flags, num_waves, M, N, K, BLOCK_SIZE_M, BLOCK_SIZE_N,
+                                             BLOCK_SIZE_K, cum_tiles, a_list, a_target_rank, c_list, target_rank, dst_offsets,
+                                             atomic_add, k_ranges, dev))
+        if caller_owned:
+            remember_note(given, "remote binding", prepared)
+    fields, keep = prepared[1]
     remote = _lib.GemmRemote()
-    keep = []
-    if a_list is not None:
-        if a_target_rank is None:
-            raise ValueError("a list of A shards needs a_target_rank")
-        a_ranks = as_device_table(a_target_rank, dev, None)
-        _check_ranks("a_target_rank", a_ranks, len(a_list), num_waves)
-        shard_rows = min(t.shape[0] for t in a_list)
-        if int(hs[:, 0].max()) > shard_rows:
-            raise ValueError("a wave has more rows than an A shard")
-        table = _pointer_table(a_list, dev)
-        keep += [a_ranks, table]
-        remote.a_peers, remote.a_target_rank = table.data_ptr(), a_ranks.data_ptr()
-    if c_list is not None:
-        if target_rank is None or dst_offsets is None:
-            raise ValueError("a list of C buffers needs target_rank and dst_offsets")
-        c_ranks = as_device_table(target_rank, dev, None)
-        dst = as_device_table(dst_offsets, dev, 2)
-        _check_ranks("target_rank", c_ranks, len(c_list), num_waves)
-        ldc = c_list[0].shape[1]
-        rows = min(t.shape[0] for t in c_list)
-        if any(t.shape[1] != ldc for t in c_list) or ldc % 4:
-            raise ValueError("peer C buffers must share one row length, a multiple of 4")
-        hd = host_copy(dst)
-        if dst.shape[0] < num_waves or int(hd.min()) < 0:
-            raise ValueError("dst_offsets must hold one non-negative (row, col) pair per wave")
-        if int((hd[:num_waves, 0] + hs[:, 0]).max()) > rows or int((hd[:num_waves, 1] + hs[:, 1]).max()) > ldc:
-            raise ValueError("a wave's destination region does not fit the peer C buffer")
-        if int(hd[:num_waves, 1].max()) % 4:
-            raise ValueError("dst column offsets must be multiples of 4 elements")
-        table = _pointer_table(c_list, dev)
-        keep += [c_ranks, dst, table]
-        remote.c_peers, remote.c_target_rank = table.data_ptr(), c_ranks.data_ptr()
-        remote.c_dst_offsets, remote.c_ld = dst.data_ptr(), ldc
-        remote.c_atomic_add = 1 if atomic_add else 0
-    elif atomic_add:
-        raise ValueError("atomic_add needs c bound to peers")
-    if k_ranges is not None:
-        if c_list is None or not atomic_add:
-            raise ValueError("k_ranges produce partial products: c must be bound and added into (atomic_add)")
-        ranges = as_device_table(k_ranges, dev, 2)
-        hk = host_copy(ranges)
-        if ranges.shape[0] < num_waves:
-            raise ValueError("k_ranges is shorter than the wave tables")
-        k0, kn = hk[:num_waves, 0], hk[:num_waves, 1]
-        if int(k0.min()) < 0 or int(kn.min()) <= 0 or int((k0 % 64).max()) or int((kn % 64).max()):
-            raise ValueError("k ranges must start at and span positive multiples of 64")
-        if int((k0 + kn).max()) > K:
-            raise ValueError("a k range runs past K")
-        keep.append(ranges)
-        remote.k_ranges = ranges.data_ptr()
+    for name, value in fields.items():
+        setattr(remote, name, value)
 
     if visit_log is not None:
         tiles = (int(cum_tiles) if cum_tiles else M * N) // (BLOCK_SIZE_M * BLOCK_SIZE_N)
@@ -201,7 +225,7 @@ def gemm_remote(
     with torch.cuda.device(dev):
         _lib.check("syn_gemm_remote_binding",
                    lib.syn_gemm_remote_binding(ctypes.byref(desc), ctypes.byref(remote), _lib.stream_handle(stream)))
-    del keep
+    del keep, prepared
 
 
 def gemm_ag_direct_read(
@@ -268,8 +292,13 @@ def gemm_rs_producer_persistent(
     assert m_per_rank % BLOCK_SIZE_M == 0
     # rows are wave-local in the owner's buffer, columns keep their global position
     # (template_rs.py:157-166: offs_cm from the wave-local pid_m, offs_bn from the global pid_n)
-    dst = host_copy(as_device_table(wave_offset, a.device, 2)).clone()
-    dst[:, 0] = 0
+    owned = isinstance(wave_offset, torch.Tensor) and wave_offset.is_cuda
+    dst = recall_note([wave_offset], "owner slot offsets") if owned else None
+    if dst is None:
+        dst = as_device_table(wave_offset, a.device, 2).clone()
+        dst[:, 0] = 0
+        if owned:
+            remember_note([wave_offset], "owner slot offsets", dst)      # the same tensor next time: gemm_remote's notes hold
     gemm_remote(a, b, bufs, num_gemm_sms, BLOCK_SIZE_M, BLOCK_SIZE_N, BLOCK_SIZE_K, GROUP_SIZE_M, STAGES,
                 cur_wave_sizes=cur_wave_size, wave_offsets=wave_offset, M=m, target_rank=target_rank,
                 dst_offsets=dst, atomic_add=True, cum_tiles=m * b.shape[0], **kwargs)

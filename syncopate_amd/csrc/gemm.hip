@@ -70,7 +70,7 @@ struct GemmParams {
 };
 
 // kernel modes
-constexpr int kConsumer = 0, kProducer = 1, kRemote = 2;
+constexpr int kConsumer = 0, kProducer = 1, kRemote = 2, kRemoteAtomic = 3;   // kRemoteAtomic: kRemote whose C tiles are added
 
 template <typename T>
 struct Mfma32;
@@ -1008,7 +1008,10 @@ __device__ __forceinline__ void store16_write_through(void* dst, uint4 v) {
 template <typename T, typename Pipe, int BM, int BN, int WGM, int WGN, int MODE>
 __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmParams p) {
     constexpr bool PRODUCER = MODE == kProducer;
-    constexpr bool REMOTE = MODE == kRemote;
+    constexpr bool REMOTE = MODE == kRemote || MODE == kRemoteAtomic;
+    // a kernel of its own for the adding form: with both epilogues in one kernel the compiler spills some 170 registers
+    // in the per-tile code, and the storing form runs 10 % slower than the producer it otherwise equals
+    constexpr bool ATOMIC = MODE == kRemoteAtomic;
     constexpr int WM = BM / WGM, WN = BN / WGN;   // wavefront tile
     constexpr int TM = WM / 32, TN = WN / 32;     // 32x32 MFMA tiles per wavefront
 
@@ -1140,6 +1143,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
         size_t ldc;
         int k_rot, wave, sig, wave_tiles;
         int k_len;                       // elements of K the tile contracts over (the panels start at its first k)
+        bool c_rows_16;                  // (peer C) every row of the tile starts on a 16-byte boundary
     };
     // get_pid_mn (template.py:10-18) on the wave-local tile id, and the tile's K phase
     auto locate = [&](int tile_id) -> Tile {
@@ -1168,6 +1172,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
                 t.c_tile = c_base + ((size_t)dst_m + (size_t)pid_m_local * BM) * t.ldc + dst_n + (size_t)pid_n_local * BN;
             }
         }
+        t.c_rows_16 = (reinterpret_cast<uintptr_t>(t.c_tile) % 16 == 0) && (t.ldc * sizeof(T)) % 16 == 0;
         // Tiles walk K cyclically, neighbouring tiles starting 128 elements apart.  With a
         // power-of-two row pitch, programs that all sweep K from 0 in lockstep keep hitting the
         // same few memory channels; four phases spread them while tiles that share a panel of A
@@ -1261,33 +1266,41 @@ __global__ void __launch_bounds__(64 * WGM * WGN) gemm_wave_kernel(const GemmPar
                                 pack4<T>(acc[i][js + jj][4 * g], acc[i][js + jj][4 * g + 1],
                                          acc[i][js + jj][4 * g + 2], acc[i][js + jj][4 * g + 3]);
                     }
-                    if constexpr (REMOTE) {
-                        if (p.c_atomic) {
-                            // one packed atomic per lane, the lanes of an instruction side by side in a row: every
-                            // instruction adds into whole cache lines.  (Issued as 8 or 16 bytes per lane - four
-                            // instructions that each touch a quarter of every line - the atomic form of the
-                            // 8192 x 8192 x 3584 GEMM took 0.82-0.86 ms against 0.33 for the stores.)
-                            constexpr int DPR = CS_COLS / 2;          // dwords of a staged row
-                            constexpr int RPA = 64 / DPR;             // rows per atomic instruction
+                    if constexpr (ATOMIC) {
+                        // one packed atomic per lane, the lanes of an instruction side by side in a row: every
+                        // instruction adds into whole cache lines.  (Issued as 8 or 16 bytes per lane - four
+                        // instructions that each touch a quarter of every line - the atomic form of the
+                        // 8192 x 8192 x 3584 GEMM took 0.82-0.86 ms against 0.33 for the stores.)
+                        constexpr int DPR = CS_COLS / 2;          // dwords of a staged row
+                        constexpr int RPA = 64 / DPR;             // rows per atomic instruction
+                        // (one carried address: written as a product per row, the unrolled loops keep dozens of 64-bit
+                        // row addresses alive and the kernel spills them)
+                        T* row_ptr = tile.c_tile + (size_t)(wm * WM + 32 * i + lane / DPR) * tile.ldc + wn * WN + 32 * js +
+                                     (lane % DPR) * 2;
 #pragma unroll
-                            for (int t = 0; t < 32 / RPA; ++t) {
-                                const int row = t * RPA + lane / DPR;
-                                const unsigned v = *reinterpret_cast<const unsigned*>(cs + row * CS_ROW + (lane % DPR) * 4);
-                                atomic_add2<T>(tile.c_tile + (size_t)(wm * WM + 32 * i + row) * tile.ldc + wn * WN + 32 * js +
-                                                   (lane % DPR) * 2, v);
-                            }
-                            continue;
+                        for (int t = 0; t < 32 / RPA; ++t) {
+                            const int row = t * RPA + lane / DPR;
+                            const unsigned v = *reinterpret_cast<const unsigned*>(cs + row * CS_ROW + (lane % DPR) * 4);
+                            atomic_add2<T>(row_ptr, v);
+                            row_ptr += (size_t)RPA * tile.ldc;
+                            asm volatile("" : "+v"(row_ptr));
                         }
+                        continue;
                     }
 #pragma unroll
                     for (int t = 0; t < 32 / RPI; ++t) {
                         const uint4 v = *reinterpret_cast<const uint4*>(cs_rd + t * RPI * CS_ROW);
                         T* dst = c_out + (size_t)(32 * i + t * RPI) * tile.ldc + 32 * js;
                         if constexpr (REMOTE) {
-                            // peer buffers are only 8-byte aligned: two 8-byte stores per lane
-                            const uint2 lo = {v.x, v.y}, hi = {v.z, v.w};
-                            *reinterpret_cast<uint2*>(dst) = lo;
-                            *reinterpret_cast<uint2*>(dst + 4) = hi;
+                            // peer buffers need only be 8-byte aligned (two 8-byte stores per lane); where the
+                            // tile's rows sit on 16-byte boundaries, one store
+                            if (tile.c_rows_16) {
+                                *reinterpret_cast<uint4*>(dst) = v;
+                            } else {
+                                const uint2 lo = {v.x, v.y}, hi = {v.z, v.w};
+                                *reinterpret_cast<uint2*>(dst) = lo;
+                                *reinterpret_cast<uint2*>(dst + 4) = hi;
+                            }
                         } else if (PRODUCER) {
                             // written through the XCD's L2: the release below then has nothing
                             // of this tile left to write back
@@ -1367,9 +1380,9 @@ template <typename T, int MODE>
 static int dispatch_pipe(const GemmParams& p, int bm, int bn, bool eight, bool ring, bool two_stage, bool mfma32,
                          int grid, hipStream_t stream) {
     // the remote-binding form exists for the default pipeline only
-    if (MODE != kRemote) {
-        if (ring) return dispatch_tile<T, RingPipe, MODE == kRemote ? kConsumer : MODE>(p, bm, bn, eight, grid, stream);
-        if (two_stage) return dispatch_tile<T, PairPipe, MODE == kRemote ? kConsumer : MODE>(p, bm, bn, eight, grid, stream);
+    if (MODE < kRemote) {
+        if (ring) return dispatch_tile<T, RingPipe, MODE >= kRemote ? kConsumer : MODE>(p, bm, bn, eight, grid, stream);
+        if (two_stage) return dispatch_tile<T, PairPipe, MODE >= kRemote ? kConsumer : MODE>(p, bm, bn, eight, grid, stream);
     }
     // tiles of which three stages do not fit have two forms of the early-read pipeline
     if (mfma32) return dispatch_tile<T, DeepPipe32, MODE>(p, bm, bn, eight, grid, stream);
@@ -1469,11 +1482,15 @@ static int gemm_entry(const syn_gemm_desc* d, hipStream_t stream, int mode,
         if (err != hipSuccess) return (int)err;
     }
     if (d->dtype == SYN_DTYPE_BF16) {
-        if (mode == kRemote) return dispatch_pipe<__bf16, kRemote>(p, bm, bn, eight, false, false, m32, grid, stream);
+        if (mode == kRemote)
+            return p.c_atomic ? dispatch_pipe<__bf16, kRemoteAtomic>(p, bm, bn, eight, false, false, m32, grid, stream)
+                              : dispatch_pipe<__bf16, kRemote>(p, bm, bn, eight, false, false, m32, grid, stream);
         return producer ? dispatch_pipe<__bf16, kProducer>(p, bm, bn, eight, ring, two, m32, grid, stream)
                         : dispatch_pipe<__bf16, kConsumer>(p, bm, bn, eight, ring, two, m32, grid, stream);
     }
-    if (mode == kRemote) return dispatch_pipe<_Float16, kRemote>(p, bm, bn, eight, false, false, m32, grid, stream);
+    if (mode == kRemote)
+        return p.c_atomic ? dispatch_pipe<_Float16, kRemoteAtomic>(p, bm, bn, eight, false, false, m32, grid, stream)
+                          : dispatch_pipe<_Float16, kRemote>(p, bm, bn, eight, false, false, m32, grid, stream);
     return producer ? dispatch_pipe<_Float16, kProducer>(p, bm, bn, eight, ring, two, m32, grid, stream)
                     : dispatch_pipe<_Float16, kConsumer>(p, bm, bn, eight, ring, two, m32, grid, stream);
 }
