@@ -15,30 +15,44 @@ constexpr int kMaxWorld = 16;
 template <typename T>
 __device__ __forceinline__ float to_f32(T x) { return (float)x; }
 
-template <typename T, bool ROUND_EACH>
-__device__ __forceinline__ u32x4_t add8(const u32x4_t* parts, int count) {
+// the running sum of one 16-byte group: eight fp32 values, added to in ring order
+template <typename T>
+__device__ __forceinline__ void sum_begin(float (&acc)[8], const u32x4_t first) {
     typedef T vec8 __attribute__((ext_vector_type(8)));
-    float acc[8];
-    {
-        const vec8 v = __builtin_bit_cast(vec8, parts[0]);
+    const vec8 v = __builtin_bit_cast(vec8, first);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) acc[e] = (float)v[e];
-    }
-    for (int i = 1; i < count; ++i) {
-        const vec8 v = __builtin_bit_cast(vec8, parts[i]);
+    for (int e = 0; e < 8; ++e) acc[e] = (float)v[e];
+}
+
+template <typename T, bool ROUND_EACH>
+__device__ __forceinline__ void sum_add(float (&acc)[8], const u32x4_t part) {
+    typedef T vec8 __attribute__((ext_vector_type(8)));
+    const vec8 v = __builtin_bit_cast(vec8, part);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            float s = acc[e] + (float)v[e];
-            // fp32 add followed by round-to-nearest-even equals a correctly
-            // rounded add in the 16-bit type (both operands have <= 11 bits)
-            if (ROUND_EACH) s = (float)(T)s;
-            acc[e] = s;
-        }
+    for (int e = 0; e < 8; ++e) {
+        float s = acc[e] + (float)v[e];
+        // fp32 add followed by round-to-nearest-even equals a correctly
+        // rounded add in the 16-bit type (both operands have <= 11 bits)
+        if (ROUND_EACH) s = (float)(T)s;
+        acc[e] = s;
     }
+}
+
+template <typename T>
+__device__ __forceinline__ u32x4_t sum_end(const float (&acc)[8]) {
+    typedef T vec8 __attribute__((ext_vector_type(8)));
     vec8 r;
 #pragma unroll
     for (int e = 0; e < 8; ++e) r[e] = (T)acc[e];
     return __builtin_bit_cast(u32x4_t, r);
+}
+
+template <typename T, bool ROUND_EACH>
+__device__ __forceinline__ u32x4_t add8(const u32x4_t* parts, int count) {
+    float acc[8];
+    sum_begin<T>(acc, parts[0]);
+    for (int i = 1; i < count; ++i) sum_add<T, ROUND_EACH>(acc, parts[i]);
+    return sum_end<T>(acc);
 }
 
 constexpr int kVecsPerThread = 4;      // 16-byte groups per lane and pass: 4 x W loads in flight
@@ -73,19 +87,39 @@ ring_reduce_kernel(const u32x4_t* __restrict__ recv, const u32x4_t* __restrict__
 #pragma unroll
             for (int u = 0; u < kVecsPerThread; ++u)
                 __builtin_nontemporal_store(add8<T, ROUND_EACH>(parts[u], w), out + v0 + u * kReduceThreads);
-        } else {
+        } else if (W > 0) {
             for (int64_t v = v0; v < chunk_vecs; v += kReduceThreads) {
                 u32x4_t parts[kParts];
                 parts[0] = __builtin_nontemporal_load(own + v);
 #pragma unroll
                 for (int i = 1; i < kParts; ++i) {
-                    if (i < w) {
-                        int src = rank + i;
-                        if (src >= w) src -= w;
-                        parts[i] = __builtin_nontemporal_load(recv + (int64_t)src * recv_stride_vecs + v);
-                    }
+                    int src = rank + i;
+                    if (src >= w) src -= w;
+                    parts[i] = __builtin_nontemporal_load(recv + (int64_t)src * recv_stride_vecs + v);
                 }
                 __builtin_nontemporal_store(add8<T, ROUND_EACH>(parts, w), out + v);
+            }
+        } else {
+            // any world size: the received blocks four at a time (registers the compiler can name: an array of
+            // `world` parts indexed by a run-time count would live in scratch memory), added in ring order
+            for (int64_t v = v0; v < chunk_vecs && v < g0 + kGroup; v += kReduceThreads) {
+                float acc[8];
+                sum_begin<T>(acc, __builtin_nontemporal_load(own + v));
+                for (int i = 1; i < w; i += 4) {
+                    u32x4_t parts[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        if (i + j < w) {
+                            int src = rank + i + j;
+                            if (src >= w) src -= w;
+                            parts[j] = __builtin_nontemporal_load(recv + (int64_t)src * recv_stride_vecs + v);
+                        }
+                    }
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        if (i + j < w) sum_add<T, ROUND_EACH>(acc, parts[j]);
+                }
+                __builtin_nontemporal_store(sum_end<T>(acc), out + v);
             }
         }
     }

@@ -95,3 +95,35 @@ def test_ring_reduce_rejects_bad_arguments(hip):
     out = torch.zeros(8, 8, dtype=torch.bfloat16, device="cuda")
     with pytest.raises(_lib.SyncopateHipError):
         ring_reduce(recv, out, local, 4)                                  # rank out of range
+
+
+def test_every_world_size_makes_one_pass_over_its_chunk(hip):
+    """World sizes without a kernel of their own (3, 5, 6, 7, 9 ... 16) share a general kernel; like the others it
+    reads every received block once.  A launch that walked its chunk once per workgroup gave the same bits a
+    thousand times slower - so the bound here is generous: within 20 x of the time of world 8 on the same chunk."""
+    from syncopate_amd.computation.reduce import ring_reduce
+
+    rows, n = 512, 8192
+
+    def launch_ms(world):
+        g = torch.Generator(device="cuda").manual_seed(world)
+        recv = torch.randn(world, rows, n, device="cuda", generator=g).bfloat16()
+        local = torch.randn(world * rows, n, device="cuda", generator=g).bfloat16()
+        out = torch.empty(rows, n, dtype=torch.bfloat16, device="cuda")
+        for _ in range(3):
+            ring_reduce(recv, out, local, 1)
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(10):
+            ring_reduce(recv, out, local, 1)
+        stop.record()
+        torch.cuda.synchronize()
+        acc = local[rows:2 * rows].clone()
+        for i in range(1, world):
+            acc = acc + recv[(1 + i) % world]
+        assert torch.equal(out, acc)
+        return start.elapsed_time(stop) / 10
+
+    eight = launch_ms(8)
+    for world in (3, 7, 13):
+        assert launch_ms(world) < 20 * eight * max(1.0, world / 8), world
