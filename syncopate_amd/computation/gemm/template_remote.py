@@ -335,9 +335,17 @@ def gemm_splitk(
     num_waves = sizes3.shape[0]
     if offsets3.shape[0] != num_waves:
         raise ValueError("wave size and offset tables disagree on the number of waves")
+    # the two-column tables gemm_remote takes, kept with the caller's three-column ones (so that its notes hold too)
+    owned = all(isinstance(t, torch.Tensor) and t.is_cuda for t in (cur_wave_sizes, wave_offsets))
+    split = recall_note([cur_wave_sizes, wave_offsets], "split-k tables") if owned else None
+    if split is None:
+        split = (sizes3[:, :2].contiguous(), offsets3[:, :2].contiguous(),
+                 torch.zeros(num_waves, dtype=torch.int32, device=dev),
+                 torch.stack([offsets3[:, 2], sizes3[:, 2]], dim=1).contiguous())
+        if owned:
+            remember_note([cur_wave_sizes, wave_offsets], "split-k tables", split)
+    sizes2, offsets2, ranks, k_ranges = split
     gemm_remote(a, b, [c], num_gemm_sms, BLOCK_SIZE_M, BLOCK_SIZE_N, BLOCK_SIZE_K, GROUP_SIZE_M, STAGES,
-                cur_wave_sizes=sizes3[:, :2].contiguous(), wave_offsets=offsets3[:, :2].contiguous(), M=a.shape[0],
-                target_rank=torch.zeros(num_waves, dtype=torch.int32, device=dev),
-                dst_offsets=offsets3[:, :2].contiguous(), atomic_add=True,
-                k_ranges=torch.stack([offsets3[:, 2], sizes3[:, 2]], dim=1).contiguous(),
-                signal_ptr=signal_ptr, signal_offsets=signal_offsets, cum_tiles=cum_tiles, **kwargs)
+                cur_wave_sizes=sizes2, wave_offsets=offsets2, M=a.shape[0], target_rank=ranks, dst_offsets=offsets2,
+                atomic_add=True, k_ranges=k_ranges, signal_ptr=signal_ptr, signal_offsets=signal_offsets,
+                cum_tiles=cum_tiles, **kwargs)
