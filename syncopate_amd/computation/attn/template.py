@@ -290,10 +290,16 @@ def attention_forward(
             raise ValueError("without counter_ptr, signal_ptr itself is what the kernel waits for")
         wait_flags = flag_buffer(consumer_signal_ptr)
         wait_sigs = as_device_table(consumer_signal_offsets, dev, None)
-        hw = host_copy(wait_sigs)
-        if wait_sigs.numel() < num_waves or int(hw[:num_waves].min()) < -1 or \
-                int(hw[:num_waves].max()) >= wait_flags.numel():
-            raise ValueError("consumer_signal_offsets must hold one index into consumer_signal_ptr (or -1) per wave")
+        # read back once per table object: a device-to-host copy per launch would wait for the stream to drain
+        owned = isinstance(consumer_signal_offsets, torch.Tensor) and consumer_signal_offsets.is_cuda
+        note = f"indices to wait for, {num_waves} waves, {wait_flags.numel()} flags"
+        if not (owned and recall_note([consumer_signal_offsets], note)):
+            hw = host_copy(wait_sigs)
+            if wait_sigs.numel() < num_waves or int(hw[:num_waves].min()) < -1 or \
+                    int(hw[:num_waves].max()) >= wait_flags.numel():
+                raise ValueError("consumer_signal_offsets must hold one index into consumer_signal_ptr (or -1) per wave")
+            if owned:
+                remember_note([consumer_signal_offsets], note, True)
     o = torch.empty(q.shape, dtype=q.dtype, device=dev) if out is None else out
     if o.shape != q.shape or o.dtype != q.dtype:
         raise ValueError("out must match q")

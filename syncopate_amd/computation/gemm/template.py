@@ -28,7 +28,9 @@ from .._launch import (
     host_ptr,
     launches_on_stream,
     acquire_always,
+    recall_note,
     remember_checked,
+    remember_note,
     require_cuda,
     status_words,
 )
@@ -112,9 +114,15 @@ def _launch(
         wait_sigs = as_device_table(wait_signal_offsets, dev, None)
         if wait_sigs.numel() != num_waves:
             raise ValueError("one index to wait for per wave (-1: none)")
-        hw = host_copy(wait_sigs)
-        if int(hw.min()) < -1 or int(hw.max()) >= wait_flags.numel():
-            raise ValueError("an index to wait for is outside its flag array")
+        # read back once per table object: a device-to-host copy per launch would wait for the stream to drain
+        owned = isinstance(wait_signal_offsets, torch.Tensor) and wait_signal_offsets.is_cuda
+        note = f"indices to wait for, {wait_flags.numel()} flags"
+        if not (owned and recall_note([wait_signal_offsets], note)):
+            hw = host_copy(wait_sigs)
+            if int(hw.min()) < -1 or int(hw.max()) >= wait_flags.numel():
+                raise ValueError("an index to wait for is outside its flag array")
+            if owned:
+                remember_note([wait_signal_offsets], note, True)
 
     if producer:
         if counter_buffer is None:
