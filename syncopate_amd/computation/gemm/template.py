@@ -35,6 +35,8 @@ from .._launch import (
     status_words,
 )
 
+from .tile_policy import choose_xcd_remap
+
 DEFAULT_SPIN_TIMEOUT_US = 2_000_000
 
 
@@ -56,7 +58,7 @@ def _launch(
     cum_tiles: int,
     counter_buffer: Optional[torch.Tensor],
     visit_log: Optional[torch.Tensor],
-    xcd_remap: bool,
+    xcd_remap: Optional[bool],
     eight_waves: bool,
     ring_pipe: bool,
     k_stagger: bool,
@@ -139,6 +141,8 @@ def _launch(
         if visit_log.dtype != torch.int32 or visit_log.numel() < 4 * tiles or not visit_log.is_contiguous():
             raise ValueError(f"visit_log must be a contiguous int32 tensor of at least {4 * tiles} words")
 
+    if xcd_remap is None:
+        xcd_remap = choose_xcd_remap(BLOCK_SIZE_M, BLOCK_SIZE_N)
     desc = _lib.GemmDesc(
         a=a.data_ptr(),
         b=b.data_ptr(),
@@ -197,7 +201,7 @@ def gemm_consumer(
     *,
     cum_tiles=0,
     visit_log=None,
-    xcd_remap=True,
+    xcd_remap=None,
     eight_waves=False,
     ring_pipe=False,
     k_stagger=True,
@@ -239,7 +243,7 @@ def gemm_producer(
     cum_tiles=0,
     counter_buffer=None,
     visit_log=None,
-    xcd_remap=True,
+    xcd_remap=None,
     eight_waves=False,
     ring_pipe=False,
     k_stagger=True,
@@ -279,7 +283,7 @@ def gemm(
     consumer_signal_offsets=None,
     cum_tiles=0,
     visit_log=None,
-    xcd_remap=True,
+    xcd_remap=None,
     eight_waves=False,
     ring_pipe=False,
     k_stagger=True,

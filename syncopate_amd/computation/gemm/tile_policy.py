@@ -56,3 +56,12 @@ def choose_tile(chunk_rows: int, n: int, programs: int, *, producer_bound: bool,
         return (r - 1) * RESIDENT_COST[s] + LAST_ROUND_COST[s]
 
     return min(candidates, key=lambda s: (left_over(s), -s[0] * s[1]))
+
+
+def choose_xcd_remap(bm: int, bn: int) -> bool:
+    """Whether the programs of one XCD should take consecutive tiles (SYN_GEMM_XCD_REMAP), for a launcher that was not
+    told.  Measured on the resident 8192 x 8192 x 3584 consumer: 128x256, 256x128 and 128x128 tiles gain 4-10 % from
+    the remap (224 programs: 373 / 369 / 502 us against 409 / 385 / 559); 256x256 tiles gain nothing on 224 programs
+    (340 either way) and LOSE 9 % on 256 (365 against 336 us); the 8192 x 8192 x 3584 producer on 256x256 tiles is
+    the same either way (335 us)."""
+    return (bm, bn) != (256, 256)

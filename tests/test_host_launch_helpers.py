@@ -112,3 +112,12 @@ def test_trusted_flag_arrays_are_remembered_per_tensor_object():
     assert acquire_always(later)                 # whatever object now lives at that id is not trusted
     from syncopate_amd.computation import _launch
     assert key not in _launch._trusted_flags or _launch._trusted_flags.get(key) is None
+
+
+def test_xcd_remap_policy_follows_the_measurements():
+    """Smaller tiles gain from the remap, the 256 x 256 tile does not (and loses with 256 programs): a launcher that was
+    not told takes it for the former only."""
+    from syncopate_amd.computation.gemm.tile_policy import choose_xcd_remap
+
+    assert not choose_xcd_remap(256, 256)
+    assert all(choose_xcd_remap(bm, bn) for bm, bn in ((128, 256), (256, 128), (128, 128), (256, 224)))
