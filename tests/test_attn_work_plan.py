@@ -363,3 +363,45 @@ def test_causal_attention_of_a_q_shard_that_does_not_start_at_zero(hip, form):
     ref = numerics.sdpa_fp32(q, k, v, 128 ** -0.5, causal=True)
     assert _rel(o[:, :, lo:], ref[:, :, lo:]) <= REL_TOL
     assert (o[:, :, :lo] == 7.0).all()
+
+
+@pytest.mark.gpu
+def test_tables_and_lists_longer_than_the_kernels_lds_copies(hip):
+    """The paired kernel keeps the first 256 waves of the tables and the first 512 entries of a program's list in
+    LDS and reads the rest from memory: 600 waves of one kv block over one pair of q blocks, as one program's list of
+    600 single-visit segments, as one chained walk, and as tiles dealt to three programs."""
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.attn import attention_forward
+
+    H, Sq, chunk, waves = 1, 256, 128, 600
+    order = [(7 * i) % waves for i in range(waves)]            # 7 and 600 are coprime: every chunk once
+    offsets, sizes, cums, signals, total = allgather_tables(H, Sq, chunk, order)
+    g = torch.Generator(device="cpu").manual_seed(31)
+    q = torch.randn(1, H, Sq, 128, generator=g).bfloat16()
+    k = torch.randn(1, H, waves * chunk, 128, generator=g).bfloat16()
+    v = torch.randn(1, H, waves * chunk, 128, generator=g).bfloat16()
+    flags = torch.ones(waves - 1, dtype=torch.int64, device="cuda")
+    kw = dict(wave_offsets=offsets, wave_sizes=sizes, cum_wave_sizes=cums, signal_ptr=flags, signal_offsets=signals,
+              cum_tiles=total, pair_q_blocks=True)
+    ref = numerics.sdpa_fp32(q, k, v, 128 ** -0.5)
+    # Every merge rounds the stored partial output to bf16, as in the reference (attn/template.py:307-361): 600
+    # merges are a random walk of 600 steps of half a unit in the last place (2^-9 each), some 5 % - a property of
+    # the merged form, not of how long its tables are.  The forms that keep their sums in registers stay within REL_TOL.
+    merged_tol = 1e-1
+    log = torch.full((total // 128, 8), -1, dtype=torch.int32, device="cuda")
+    for max_visits, tol in ((None, REL_TOL), (1, merged_tol)):
+        plan = plan_attention_work(offsets, sizes, cums, causal=False, num_programs=1, max_visits=max_visits)
+        assert len(plan.program_entries[0]) == waves and plan.segments == (1 if max_visits is None else waves)
+        log.fill_(-1)
+        o = attention_forward(q.cuda(), k.cuda(), v.cuda(), 128 ** -0.5, work_plan=plan, visit_log=log, **kw)
+        check_status()
+        assert _rel(o, ref) <= tol, max_visits
+        _assert_visit_log(log, offsets, sizes, cums, signals)
+    o = attention_forward(q.cuda(), k.cuda(), v.cuda(), 128 ** -0.5, chain_q_blocks=True, **kw)
+    check_status()
+    assert _rel(o, ref) <= REL_TOL
+    log.fill_(-1)
+    o = attention_forward(q.cuda(), k.cuda(), v.cuda(), 128 ** -0.5, num_programs=3, visit_log=log, **kw)
+    check_status()
+    assert _rel(o, ref) <= merged_tol
+    _assert_visit_log(log, offsets, sizes, cums, signals)
