@@ -383,3 +383,44 @@ def test_launch_on_a_stream_that_is_not_current(hip):
         assert flags.tolist() == [1] * world
         assert _max_rel_err(c, ref) <= REL_TOL
         assert torch.equal(c, c2)
+
+
+@pytest.mark.parametrize("producer", [False, True])
+def test_more_waves_than_the_kernel_keeps_in_lds(hip, producer):
+    """The walk keeps the first 128 rows of the wave tables in LDS and reads the rest from memory: 200 waves of one
+    tile row each, in a shuffled order, every wave behind its own flag; visit log against the oracle's walk, product
+    against fp32, and (producer) every wave's counter and flag."""
+    import numpy as np
+
+    from syncopate_amd.computation._launch import check_status
+    from syncopate_amd.computation.gemm import gemm, gemm_producer
+
+    waves, BM, BN, K, N = 200, 128, 256, 128, 512
+    M = waves * BM
+    order = np.random.default_rng(5).permutation(waves).tolist()
+    sizes = [[BM, N]] * waves
+    offsets = [[o * BM, 0] for o in order]
+    signals = list(range(waves))
+    a, b = _inputs(M, N, K, torch.bfloat16, seed=9)
+    ref = numerics.gemm_fp32(a, b)
+    c = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    tiles = (M // BM) * (N // BN)
+    log = torch.full((tiles, 4), -1, dtype=torch.int32, device="cuda")
+    if producer:
+        flags = torch.zeros(waves, dtype=torch.int64, device="cuda")
+        counters = torch.zeros(waves, dtype=torch.int32, device="cuda")
+        gemm_producer(a.cuda(), b.cuda(), c, flags, sizes, offsets, signals, 7, BM, BN, 64, 8, cum_tiles=M * N,
+                      counter_buffer=counters, visit_log=log, xcd_remap=False)
+        check_status()
+        assert flags.tolist() == [1] * waves and counters.tolist() == [N // BN] * waves
+    else:
+        flags = torch.ones(waves, dtype=torch.int64, device="cuda")
+        gemm(a.cuda(), b.cuda(), c, 1, 7, BM, BN, 64, 8, cur_wave_sizes=sizes, wave_offsets=offsets, signal_ptr=flags,
+             signal_offsets=signals, cum_tiles=M * N, visit_log=log, xcd_remap=False)
+        check_status()
+    assert _max_rel_err(c, ref) <= REL_TOL
+    want = visit_order.gemm_tile_visits(sizes, offsets, signals, M=M, N=N, BM=BM, BN=BN, group_m=8, num_sms=7,
+                                        cum_tiles=M * N)
+    got = log.cpu().tolist()
+    for v in want:
+        assert tuple(got[v["tile_id"]][1:]) == (v["wave"], v["pid_m"], v["pid_n"]), v
