@@ -73,6 +73,11 @@ def test_consumer_resident_matches_fp32_and_visit_order(hip, dtype, BM, BN):
     # every variant sums each dot product over k in the same order: results are bitwise equal
     for other in outputs[1:]:
         assert torch.equal(outputs[0], other)
+    # without the tile-dependent starting slab every tile sums k from 0: another order, the same product to rounding
+    c.zero_()
+    gemm_consumer(ad, bd, c, flags, sizes, offsets, signals, world, 24, BM, BN, 64, 8, cum_tiles=M * N, k_stagger=False)
+    check_status()
+    assert _max_rel_err(c, ref) <= REL_TOL
 
 
 def test_consumer_k_not_multiple_of_128(hip):
