@@ -438,6 +438,14 @@ def run_hbm_read_ceiling(device, launches=30):
     for name, (nbytes, stride, streams) in forms.items():
         ms = _timed(lambda i: probe(i % sets, nbytes, stride, streams), launches, sets)
         result[name + "_GBps"] = 8 * stream_bytes / (ms * 1e-3) / 1e9
+
+    # the eight streams 16 MiB apart again, read the way the reduce walks them: skewed by one 4 KB block per stream
+    def skewed(region):
+        _lib.check("syn_probe_read_streams_skewed",
+                   lib.syn_probe_read_streams_skewed(pool.data_ptr() + region * span, stream_bytes, stream_bytes, blocks,
+                                                     sink.data_ptr(), _lib.stream_handle(None)))
+    ms = _timed(lambda i: skewed(i % sets), launches, sets)
+    result["eight_streams_16MiB_apart_skewed_walk_GBps"] = 8 * stream_bytes / (ms * 1e-3) / 1e9
     return result
 
 
@@ -1202,7 +1210,7 @@ def main():
         line["hbm_read_ceiling"] = ceiling_reads
         # the reduce moves its bytes (8/9 of them reads at that placement, 1/9 writes) at this fraction of the
         # rate at which the same reads alone can be had
-        line["rs_reduce_over_eight_stream_read_ceiling"] = line["rs_reduce_GBps"] / ceiling_reads["eight_streams_16MiB_apart_GBps"]
+        line["rs_reduce_over_eight_stream_read_ceiling"] = line["rs_reduce_GBps"] / ceiling_reads["eight_streams_16MiB_apart_skewed_walk_GBps"]
     if "box_copies" in only:
         boxes = run_box_copies(device, steps_small, args.warmup)
         line["box_copy_launches"] = steps_small

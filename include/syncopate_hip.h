@@ -480,6 +480,12 @@ int syn_probe_mfma_rate(float* sink, int32_t workgroups, int32_t iters, int32_t 
  * what the memory system gives the reduce's reads at that placement of its operands. */
 int syn_probe_read_streams(const void* base, int64_t stream_bytes, int64_t stride_bytes, int32_t streams,
                            int32_t workgroups, void* sink, syn_stream_t stream);
+/* The same eight streams (`stream_bytes` a multiple of 32768) read the way the chunked reduce walks a chunk of at
+ * least 16 MiB per stream: a workgroup takes eight consecutive 4 KB blocks of every stream and reads, in step t,
+ * block t - i of stream i - streams that lie a multiple of the DRAM interleave apart are then never asked for the
+ * same bank at the same time. */
+int syn_probe_read_streams_skewed(const void* base, int64_t stream_bytes, int64_t stride_bytes, int32_t workgroups,
+                                  void* sink, syn_stream_t stream);
 
 /* Measurement aid, no counterpart in the reference: the slot of the paired attention kernel, piece by piece.
  * `workgroups` workgroups of eight wavefronts (two per SIMD) run `iters` slots; in a slot wavefronts 0-3 run that

@@ -195,6 +195,7 @@ _SIGNATURES = {
     "syn_where_async": (c_int32, [c_void_p, c_int32, c_int32, c_void_p]),
     "syn_probe_mfma_rate": (c_int32, [c_void_p, c_int32, c_int32, c_int32, c_void_p]),
     "syn_probe_read_streams": (c_int32, [c_void_p, ctypes.c_int64, ctypes.c_int64, c_int32, c_int32, c_void_p, c_void_p]),
+    "syn_probe_read_streams_skewed": (c_int32, [c_void_p, ctypes.c_int64, ctypes.c_int64, c_int32, c_void_p, c_void_p]),
     "syn_probe_attn_slot": (c_int32, [c_void_p, ctypes.c_int64, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_void_p]),
     "syn_version": (c_int32, []),
 }

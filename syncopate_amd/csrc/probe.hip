@@ -388,6 +388,47 @@ __global__ void __launch_bounds__(512, 1) attn_slot_kernel(int what, int iters, 
     if (blockIdx.x == 0 && (threadIdx.x & 255) == 0) cycles[wave8 >> 2] = t1 - t0;
 }
 
+// The same streams read the way the reduce's skewed walk reads them: a workgroup takes eight consecutive blocks of
+// 4 KB per stream and in step t reads block t - i of stream i, the next step's loads issued before this step's are used.
+template <int STREAMS>
+__global__ void __launch_bounds__(kStreamThreads)
+read_streams_skewed_kernel(const u32x4_probe_t* __restrict__ base, int64_t stride_vecs, int64_t stream_vecs,
+                           u32x4_probe_t* __restrict__ sink) {
+    constexpr int kBlocks = 8;
+    constexpr int64_t kSuper = (int64_t)kStreamThreads * kBlocks;
+    constexpr int kSteps = kBlocks + STREAMS - 1;
+    u32x4_probe_t mix = {0u, 0u, 0u, 0u};
+    for (int64_t g0 = (int64_t)blockIdx.x * kSuper; g0 + kSuper <= stream_vecs; g0 += (int64_t)gridDim.x * kSuper) {
+        u32x4_probe_t even[STREAMS], odd[STREAMS];
+        auto issue = [&](const int t, u32x4_probe_t (&dst)[STREAMS]) __attribute__((always_inline)) {
+#pragma unroll
+            for (int i = 0; i < STREAMS; ++i) {
+                const int b = t - i;
+                if (b >= 0 && b < kBlocks)
+                    dst[i] = __builtin_nontemporal_load(base + (int64_t)i * stride_vecs + g0 + b * kStreamThreads + threadIdx.x);
+            }
+        };
+        auto take = [&](const int t, const u32x4_probe_t (&src)[STREAMS]) __attribute__((always_inline)) {
+#pragma unroll
+            for (int i = 0; i < STREAMS; ++i) {
+                const int b = t - i;
+                if (b >= 0 && b < kBlocks) mix ^= src[i];
+            }
+        };
+        issue(0, even);
+#pragma unroll
+        for (int t = 0; t < kSteps; ++t) {
+            if (t + 1 < kSteps) {
+                if (t & 1) issue(t + 1, even);
+                else issue(t + 1, odd);
+            }
+            if (t & 1) take(t, odd);
+            else take(t, even);
+        }
+    }
+    if ((mix.x ^ mix.y ^ mix.z ^ mix.w) == 0x9e3779b9u) sink[blockIdx.x] = mix;
+}
+
 }  // namespace syn
 
 extern "C" int syn_probe_read_streams(const void* base, int64_t stream_bytes, int64_t stride_bytes, int32_t streams,
@@ -406,6 +447,18 @@ extern "C" int syn_probe_read_streams(const void* base, int64_t stream_bytes, in
     else
         hipLaunchKernelGGL(read_streams_kernel<8>, dim3(workgroups), dim3(kStreamThreads), 0, s, b, stride_bytes / 16,
                            stream_bytes / 16, k);
+    return (int)hipGetLastError();
+}
+
+extern "C" int syn_probe_read_streams_skewed(const void* base, int64_t stream_bytes, int64_t stride_bytes, int32_t workgroups,
+                                             void* sink, syn_stream_t stream) {
+    using namespace syn;
+    if (base == nullptr || sink == nullptr || workgroups <= 0) return SYN_EINVAL;
+    if (stream_bytes <= 0 || stream_bytes % (16 * kStreamThreads * 8)) return SYN_EINVAL;
+    if (stride_bytes < 0 || stride_bytes % 16 || !aligned16(base) || !aligned16(sink)) return SYN_EALIGN;
+    hipLaunchKernelGGL(read_streams_skewed_kernel<8>, dim3(workgroups), dim3(kStreamThreads), 0,
+                       reinterpret_cast<hipStream_t>(stream), reinterpret_cast<const u32x4_probe_t*>(base), stride_bytes / 16,
+                       stream_bytes / 16, reinterpret_cast<u32x4_probe_t*>(sink));
     return (int)hipGetLastError();
 }
 

@@ -1,8 +1,7 @@
 // Chunked ring reduce of GEMM+RS for gfx950 (tests/test_gemm_rs.py:22-72 of the reference):
 //   out[e] = local[rank*chunk + e] + sum_{i=1..W-1} recv[((rank+i) % W)*chunk + e]
-// A pure HBM stream: W reads and one write of 16 bytes per lane and element group,
-// four groups per lane and pass, all 4 W loads issued before the first add so that
-// each lane keeps 4 W 128-bit requests in flight.
+// A pure HBM stream: W reads and one write of 16 bytes per lane and element group; the streams are walked
+// skewed against each other (see skewed_walk), what is left over in passes of four groups per lane.
 #include "common.h"
 
 namespace syn {
@@ -55,18 +54,76 @@ __device__ __forceinline__ u32x4_t add8(const u32x4_t* parts, int count) {
     return sum_end<T>(acc);
 }
 
-constexpr int kVecsPerThread = 4;      // 16-byte groups per lane and pass: 4 x W loads in flight
+constexpr int kVecsPerThread = 4;      // 16-byte groups per lane and pass of the plain walk: 4 x W loads in flight
+constexpr int kSkewBlocks = 8;         // blocks of 256 16-byte groups (4 KB per stream) a workgroup takes in one skewed walk
+
+// The received blocks lie a whole number of MiB apart (the reference's [W, rows, N] layout), so element e of
+// every stream sits in the same DRAM bank and channel, in another row: W reads of one element at one time are W
+// row conflicts in one bank.  A workgroup therefore walks its 32 KB of every stream SKEWED: in step t it reads
+// block t - i of stream i (4 KB further on for each earlier stream), adds it to that block's running sum -
+// still own block first, then the received ones in ring order - and stores a block once its last stream is in.
+// Read alone, the eight streams come at 6.6-6.7 TB/s this way against 6.1-6.2 at equal offsets: what the layout
+// with 4 KiB between the blocks gives (syn_ring_reduce_strided), without asking the caller for it.
+template <typename T, bool ROUND_EACH, int W>
+__device__ __forceinline__ void skewed_walk(const u32x4_t* __restrict__ recv, const u32x4_t* __restrict__ own,
+                                            u32x4_t* __restrict__ out, int rank, int64_t recv_stride_vecs, int64_t v0) {
+    float acc[kSkewBlocks][8];
+    u32x4_t even[W], odd[W];
+    auto stream = [&](int i) __attribute__((always_inline)) -> const u32x4_t* {
+        if (i == 0) return own;
+        int src = rank + i;
+        if (src >= W) src -= W;
+        return recv + (int64_t)src * recv_stride_vecs;
+    };
+    auto issue = [&](const int t, u32x4_t (&dst)[W]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < W; ++i) {
+            const int b = t - i;
+            if (b >= 0 && b < kSkewBlocks) dst[i] = __builtin_nontemporal_load(stream(i) + v0 + b * kReduceThreads);
+        }
+    };
+    auto take = [&](const int t, const u32x4_t (&src)[W]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < W; ++i) {
+            const int b = t - i;
+            if (b >= 0 && b < kSkewBlocks) {
+                if (i == 0) sum_begin<T>(acc[b], src[0]);
+                else sum_add<T, ROUND_EACH>(acc[b], src[i]);
+                if (i == W - 1) __builtin_nontemporal_store(sum_end<T>(acc[b]), out + v0 + b * kReduceThreads);
+            }
+        }
+    };
+    constexpr int kSteps = kSkewBlocks + W - 1;
+    issue(0, even);
+#pragma unroll
+    for (int t = 0; t < kSteps; ++t) {
+        // the next step's loads go out before this step's are used
+        if (t + 1 < kSteps) {
+            if (t & 1) issue(t + 1, even);
+            else issue(t + 1, odd);
+        }
+        if (t & 1) take(t, odd);
+        else take(t, even);
+    }
+}
 
 template <typename T, bool ROUND_EACH, int W>
 __global__ void __launch_bounds__(kReduceThreads)
 ring_reduce_kernel(const u32x4_t* __restrict__ recv, const u32x4_t* __restrict__ local,
-                   u32x4_t* __restrict__ out, int world, int rank, int64_t chunk_vecs, int64_t recv_stride_vecs) {
+                   u32x4_t* __restrict__ out, int world, int rank, int64_t chunk_vecs, int64_t recv_stride_vecs, int skew) {
     // W > 0: world known at compile time (fully unrolled loads); W == 0: generic
     constexpr int kParts = W > 0 ? W : kMaxWorld;
     constexpr int64_t kGroup = (int64_t)kReduceThreads * kVecsPerThread;
+    constexpr int64_t kSuper = (int64_t)kReduceThreads * kSkewBlocks;
     const int w = W > 0 ? W : world;
     const u32x4_t* own = local + (int64_t)rank * chunk_vecs;
-    for (int64_t g0 = (int64_t)blockIdx.x * kGroup; g0 < chunk_vecs; g0 += (int64_t)gridDim.x * kGroup) {
+    int64_t done = 0;                      // 16-byte groups covered by skewed walks
+    if (W > 0 && skew) {
+        done = chunk_vecs / kSuper * kSuper;
+        for (int64_t s0 = (int64_t)blockIdx.x * kSuper; s0 < done; s0 += (int64_t)gridDim.x * kSuper)
+            skewed_walk<T, ROUND_EACH, W == 0 ? 2 : W>(recv, own, out, rank, recv_stride_vecs, s0 + threadIdx.x);
+    }
+    for (int64_t g0 = done + (int64_t)blockIdx.x * kGroup; g0 < chunk_vecs; g0 += (int64_t)gridDim.x * kGroup) {
         const int64_t v0 = g0 + threadIdx.x;
         if (W > 0 && g0 + kGroup <= chunk_vecs) {
             // a full group (world known at compile time): every load of the pass is issued before the first add
@@ -128,21 +185,27 @@ ring_reduce_kernel(const u32x4_t* __restrict__ recv, const u32x4_t* __restrict__
 template <typename T, bool ROUND_EACH>
 static int launch_reduce(const void* recv, const void* local, void* out, int world, int rank,
                          int64_t chunk_vecs, int64_t recv_stride_vecs, hipStream_t stream) {
-    // a workgroup takes 1024 16-byte groups per pass; two workgroups per CU, beyond that they loop
+    // a workgroup takes 2048 16-byte groups per skewed walk (1024 per pass of the plain walk); two workgroups per
+    // CU, beyond that they loop
     const int64_t group = (int64_t)kReduceThreads * kVecsPerThread;
     int64_t blocks = (chunk_vecs + group - 1) / group;
     const int64_t cap = 256 * 2;
     if (blocks > cap) blocks = cap;
     if (blocks < 1) blocks = 1;
+    // skewed walks where they fill the grid (a chunk of at least 16 MiB per stream) and the received blocks lie a
+    // multiple of 64 KiB apart; smaller chunks keep the plain walk, whose workgroups are twice as many, and so do
+    // blocks that the caller has already moved out of each other's banks (the 4 KiB of padded_receive_buffer would
+    // be undone by a skew of 4 KiB blocks)
+    const int skew = (chunk_vecs / ((int64_t)kReduceThreads * kSkewBlocks) >= cap && recv_stride_vecs % 4096 == 0) ? 1 : 0;
     const dim3 grid((unsigned)blocks), block(kReduceThreads);
     const u32x4_t* r = reinterpret_cast<const u32x4_t*>(recv);
     const u32x4_t* l = reinterpret_cast<const u32x4_t*>(local);
     u32x4_t* o = reinterpret_cast<u32x4_t*>(out);
     switch (world) {
-        case 2: hipLaunchKernelGGL((ring_reduce_kernel<T, ROUND_EACH, 2>), grid, block, 0, stream, r, l, o, world, rank, chunk_vecs, recv_stride_vecs); break;
-        case 4: hipLaunchKernelGGL((ring_reduce_kernel<T, ROUND_EACH, 4>), grid, block, 0, stream, r, l, o, world, rank, chunk_vecs, recv_stride_vecs); break;
-        case 8: hipLaunchKernelGGL((ring_reduce_kernel<T, ROUND_EACH, 8>), grid, block, 0, stream, r, l, o, world, rank, chunk_vecs, recv_stride_vecs); break;
-        default: hipLaunchKernelGGL((ring_reduce_kernel<T, ROUND_EACH, 0>), grid, block, 0, stream, r, l, o, world, rank, chunk_vecs, recv_stride_vecs); break;
+        case 2: hipLaunchKernelGGL((ring_reduce_kernel<T, ROUND_EACH, 2>), grid, block, 0, stream, r, l, o, world, rank, chunk_vecs, recv_stride_vecs, skew); break;
+        case 4: hipLaunchKernelGGL((ring_reduce_kernel<T, ROUND_EACH, 4>), grid, block, 0, stream, r, l, o, world, rank, chunk_vecs, recv_stride_vecs, skew); break;
+        case 8: hipLaunchKernelGGL((ring_reduce_kernel<T, ROUND_EACH, 8>), grid, block, 0, stream, r, l, o, world, rank, chunk_vecs, recv_stride_vecs, skew); break;
+        default: hipLaunchKernelGGL((ring_reduce_kernel<T, ROUND_EACH, 0>), grid, block, 0, stream, r, l, o, world, rank, chunk_vecs, recv_stride_vecs, 0); break;
     }
     return (int)hipGetLastError();
 }

@@ -127,3 +127,31 @@ def test_every_world_size_makes_one_pass_over_its_chunk(hip):
     eight = launch_ms(8)
     for world in (3, 7, 13):
         assert launch_ms(world) < 20 * eight * max(1.0, world / 8), world
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("world", [2, 4, 8])
+def test_skewed_walk_of_large_chunks_is_bit_exact(hip, world, dtype):
+    """Chunks of at least 16 MiB per block are walked skewed (stream i one 4 KB block behind stream i - 1), plus a
+    ragged tail in the plain walk: the sums are those of the ring order, bit for bit, in both accumulation modes'
+    default; blocks a multiple of 64 KiB apart but not adjacent take the same path."""
+    from syncopate_amd.computation.reduce import ring_reduce
+
+    rows, n, rank = 1024 + 3, 8192, world - 1               # 16 MiB + three rows per block
+    g = torch.Generator(device="cuda").manual_seed(7 * world)
+    recv = torch.randn(world, rows, n, device="cuda", generator=g).to(dtype)
+    local = torch.randn(world * rows, n, device="cuda", generator=g).to(dtype)
+    out = torch.full((rows, n), float("nan"), dtype=dtype, device="cuda")
+    ring_reduce(recv, out, local, rank)
+    acc = local[rank * rows:(rank + 1) * rows].clone()
+    for i in range(1, world):
+        acc = acc + recv[(rank + i) % world]
+    assert torch.equal(out, acc)
+    # the same blocks inside a buffer whose blocks are 64 KiB further apart
+    apart = rows * n + 32768
+    wide = torch.zeros(world * apart, dtype=dtype, device="cuda")
+    view = torch.as_strided(wide, (world, rows, n), (apart, n, 1))
+    view.copy_(recv)
+    out.fill_(float("nan"))
+    ring_reduce(view, out, local, rank)
+    assert torch.equal(out, acc)

@@ -157,3 +157,26 @@ def test_attention_slot_probe_runs_every_piece_and_rejects_bad_arguments(hip):
     assert hip.syn_probe_attn_slot(None, needed, workgroups, iters, 3, sink.data_ptr(), cycles.data_ptr(), stream) == _lib.SYN_EINVAL
     assert hip.syn_probe_attn_slot(pool.data_ptr() + 8, needed, workgroups, iters, 3, sink.data_ptr(),
                                    cycles.data_ptr(), stream) == _lib.SYN_EALIGN
+
+
+def test_skewed_read_stream_probe_reads_what_it_says(hip):
+    """The skewed form of the read probe (eight blocks of 4 KB per stream and workgroup, stream i one block behind
+    stream i - 1): the marker in the first block of the last stream reaches every lane once; past the stream's
+    end it is never read."""
+    from syncopate_amd import _lib
+
+    magic, stream_bytes, stride = 0x9E3779B9, 32768, 32768 + 4096
+    stream = _lib.stream_handle(torch.cuda.current_stream())
+    for beyond in (False, True):
+        words = torch.zeros((8 * stride + 32768) // 4, dtype=torch.int32, device="cuda")
+        first = (7 * stride + (stream_bytes if beyond else 0)) // 4
+        words[first:first + 4 * 256:4] = magic - (1 << 32)
+        sink = torch.zeros(4, dtype=torch.int32, device="cuda")
+        _lib.check("syn_probe_read_streams_skewed",
+                   hip.syn_probe_read_streams_skewed(words.data_ptr(), stream_bytes, stride, 1, sink.data_ptr(), stream))
+        torch.cuda.synchronize()
+        got = [w & 0xFFFFFFFF for w in sink.tolist()]
+        assert got == ([0, 0, 0, 0] if beyond else [magic, 0, 0, 0])
+    assert hip.syn_probe_read_streams_skewed(words.data_ptr(), 16384, stride, 1, sink.data_ptr(), stream) == _lib.SYN_EINVAL
+    assert hip.syn_probe_read_streams_skewed(words.data_ptr(), stream_bytes, stride + 8, 1, sink.data_ptr(), stream) == _lib.SYN_EALIGN
+    assert hip.syn_probe_read_streams_skewed(None, stream_bytes, stride, 1, sink.data_ptr(), stream) == _lib.SYN_EINVAL
