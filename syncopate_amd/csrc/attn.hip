@@ -93,6 +93,21 @@ struct AttnMfma<_Float16> {
     }
 };
 
+// The paired kernel's products: v_mfma_f32_16x16x32 (A: 16 rows x 32 k, lane l holds row l % 16, k 8 (l / 16) .. + 8;
+// B: 32 k x 16 columns, lane l holds column l % 16, the same k; C: lane l holds column l % 16, rows 4 (l / 16) .. + 4).
+// Same flop per cycle as the 32x32x16 form, and on random operands 11 % less energy per flop for the bare
+// instruction (syn_probe_mfma_rate) - this kernel runs at the board's power limit, so that is speed.
+template <typename T>
+__device__ __forceinline__ f32x4_t mfma16(typename AttnMfma<T>::frag_t a, typename AttnMfma<T>::frag_t b, f32x4_t c);
+template <>
+__device__ __forceinline__ f32x4_t mfma16<__bf16>(bf16x8_t a, bf16x8_t b, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+template <>
+__device__ __forceinline__ f32x4_t mfma16<_Float16>(f16x8_t a, f16x8_t b, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+
 // The merged partial results (O, lse) of a q block pass from workgroup to workgroup, possibly on
 // different XCDs, whose L2s are not coherent with each other.  A release / acquire fence pair
 // would do it - but a release writes back every dirty line of the XCD's L2 and an acquire drops
@@ -202,6 +217,77 @@ __device__ __forceinline__ void merge_rows_through_lds(unsigned char* stage, T* 
 #pragma unroll
     for (int k = 0; k < 16; ++k) store8_through(mine + 2 * k * o_pitch, (vec4_t)tile[by_row_pair(k)]);
     if (half == 0) store_f32_through(lse_rows + r, lse_out);
+}
+
+// The same merge for the paired kernel, whose accumulators come from 16 x 16 products: a lane owns, of the q rows
+// 16 b + l % 16 (b = 0, 1), the columns 16 t + 4 (l / 16) .. + 4 (t = 0..7) - again 8-byte pieces, which pass through
+// the same tile in LDS to and from whole rows in memory.
+template <typename T>
+__device__ __forceinline__ void merge_rows16_through_lds(unsigned char* stage, T* o_rows, const int64_t o_pitch,
+                                                         float* lse_rows, const f32x4_t (&o_acc)[8][2],
+                                                         const float (&inv_l)[2], const float (&lse2)[2],
+                                                         const bool is_first, const int lane) {
+    typedef T vec4_t __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) vec4_t* lds_vec4_ptr;
+    const int r = lane & 31, half = lane >> 5, c16 = lane & 15, g = lane >> 4;
+    const lds_vec4_ptr tile = (lds_vec4_ptr)(__attribute__((address_space(3))) void*)stage;
+    // element offsets in units of 8 bytes
+    auto by_row_pair = [&](const int k) { return ((2 * k + half) * kStageRowBytes >> 3) + r; };
+    auto by_accumulator = [&](const int t, const int b) { return ((16 * b + c16) * kStageRowBytes >> 3) + 4 * t + g; };
+    T* const mine = o_rows + (int64_t)half * o_pitch + 4 * r;      // instruction k: + 2 * k * o_pitch
+
+    float w_old[2] = {0.f, 0.f}, w_new[2] = {1.f, 1.f}, lse_out[2] = {lse2[0], lse2[1]};
+    vec4_t old[8][2];
+    if (!is_first) {
+        vec4_t in[16];
+        float m_old[2];
+#pragma unroll
+        for (int b = 0; b < 2; ++b) m_old[b] = load_f32_coherent(lse_rows + 16 * b + c16);
+#pragma unroll
+        for (int k = 0; k < 16; ++k) in[k] = load8_coherent<vec4_t>(mine + 2 * k * o_pitch);
+#pragma unroll
+        for (int k = 0; k < 16; ++k) tile[by_row_pair(k)] = in[k];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int t = 0; t < 8; ++t)
+#pragma unroll
+            for (int b = 0; b < 2; ++b) old[t][b] = tile[by_accumulator(t, b)];
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            const float delta = m_old[b] - lse2[b];
+            const float mmax = fmaxf(m_old[b], lse2[b]);
+            lse_out[b] = mmax + fast_log2(1.0f + fast_exp2(-fabsf(delta)));
+            w_old[b] = fast_exp2(m_old[b] - lse_out[b]);
+            w_new[b] = fast_exp2(lse2[b] - lse_out[b]);
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < 8; ++t)
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            float x[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) x[c] = o_acc[t][b][c] * inv_l[b] * w_new[b];
+            if (!is_first) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) x[c] += (float)old[t][b][c] * w_old[b];
+            }
+            vec4_t out;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) out[c] = (T)x[c];
+            tile[by_accumulator(t, b)] = out;
+        }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int k = 0; k < 16; ++k) store8_through(mine + 2 * k * o_pitch, (vec4_t)tile[by_row_pair(k)]);
+    if (g == 0) {
+#pragma unroll
+        for (int b = 0; b < 2; ++b) store_f32_through(lse_rows + 16 * b + c16, lse_out[b]);
+    }
 }
 
 
@@ -604,8 +690,8 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
 // Two q blocks per workgroup, in opposite phases.
 //
 // A kv block costs a wavefront about as many cycles on the vector ALU (the softmax: 64 scores per
-// lane, one quarter-rate exponential each) as on the matrix pipe (64 MFMAs), and two independent
-// workgroups on a compute unit drift into step, so that both pipes idle half of the time.  Here
+// lane, one quarter-rate exponential each) as on the matrix pipe (128 MFMAs of 16 x 16 x 32), and two
+// independent workgroups on a compute unit drift into step, so that both pipes idle half of the time.  Here
 // one workgroup of eight wavefronts holds two q blocks that read the same kv range - group 0
 // (wavefronts 0-3) tile 2i, group 1 (wavefronts 4-7) tile 2i + 1 - and runs them one slot apart:
 //
@@ -618,6 +704,12 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
 // K(n+1) are fetched at slot 2n by all eight wavefronts, into the buffers whose last readers
 // (V(n-2), K(n-1)) finished in slot 2n-1, and have landed by the end of slot 2n+1.  One barrier
 // per slot, i.e. two per kv block and wavefront instead of four.
+//
+// The products are 16 x 16 x 32 MFMAs (a wavefront's 32 q rows as two halves of 16 that share every K and V
+// fragment).  With 32 x 32 x 16 products - the same flop, the same LDS reads, a third fewer vector instructions
+// around them - the board ran this kernel at its power limit, 1.75 to 2.2 GHz instead of 2.4; the narrower
+// form draws less per flop, the clock stays at 2.4 GHz, and the launch is 2 to 6 % shorter although it takes
+// more cycles.
 // ---------------------------------------------------------------------------------------------
 constexpr int kPairThreads = 512;
 constexpr int kPairFills = kBlockBytes / 1024 / 8;      // 4 fills of 1 KB per wavefront and block
@@ -629,6 +721,22 @@ __device__ __forceinline__ void dma_kv_block8(unsigned char* lds, const unsigned
         const int blk = i * 8 + wave8;                  // blk % 4 == wave8 % 4: the swizzle of the 4-wave form holds
         __builtin_amdgcn_global_load_lds((global_void_ptr)(src + (size_t)(blk * 4) * pitch + lane_off),
                                          (lds_void_ptr)(lds + blk * 1024), 16, 0, 0);
+    }
+}
+
+// A V block of the paired kernel in LDS: the fills (4 rows of 256 bytes each) with an even number lie one after the
+// other, those with an odd number likewise, 16 KB + 128 bytes further on - so rows 4..7 of every eight sit half a row
+// (32 banks) askew of rows 0..3, which an exclusive-or of the column could only do at the price of a per-lane address
+// for every 16 columns (see the kernel's note on its layouts).
+constexpr int kPairVOddFills = kBlockBytes / 2 + 128;
+constexpr int kPairVBlockBytes = kBlockBytes + 1024;
+__device__ __forceinline__ void dma_v_block8(unsigned char* lds, const unsigned char* src, size_t pitch,
+                                             unsigned lane_off, int wave8) {
+#pragma unroll
+    for (int i = 0; i < kPairFills; ++i) {
+        const int blk = i * 8 + wave8;
+        __builtin_amdgcn_global_load_lds((global_void_ptr)(src + (size_t)(blk * 4) * pitch + lane_off),
+                                         (lds_void_ptr)(lds + (blk >> 1) * 1024 + (wave8 & 1) * kPairVOddFills), 16, 0, 0);
     }
 }
 
@@ -654,7 +762,7 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
     static_assert(!(CAUSAL && MODE == kPairChainWaves), "the waves of a causal table do not share their kv extent");
 
     __shared__ __attribute__((aligned(1024))) unsigned char k_lds[2 * kBlockBytes];
-    __shared__ __attribute__((aligned(1024))) unsigned char v_lds[2 * kBlockBytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char v_lds[2 * kPairVBlockBytes];
     __shared__ int s_abort;
     __shared__ int s_spun;
     // the head of the wave table and of this program's list, read once: what a visit is (a search over the prefix
@@ -669,8 +777,8 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
     const int wave8 = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int grp = wave8 >> 2;          // which of the two q blocks
     const int wave = wave8 & 3;          // 32-row slice of the q block
-    const int r = lane & 31;
-    const int half = lane >> 5;
+    const int c16 = lane & 15;           // the lane's column of a 16 x 16 MFMA tile: q rows c16 and 16 + c16 of the slice
+    const int g = lane >> 4;             // the lane's group of four rows of a tile / its eight k of an operand
 
     if (tid == 0) s_abort = 0;
     for (int w = tid; w < min(p.num_waves, kPairLdsWaves); w += kPairThreads) {
@@ -685,23 +793,35 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
         s_row[w][7] = p.signal_offsets[w];
     }
 
-    // per-lane offsets exactly as in attn_fwd_kernel (the fill swizzle depends on wave8 % 4 only)
+    // LDS layouts of this kernel (row = kv position in the block, 16 chunks of 16 bytes per row):
+    //   K: logical chunk c of row r at physical chunk c ^ (r & 15): a 16-byte read per lane of the rows 16 a + l % 16
+    //      at the chunk 4 ks + l / 16 - an A operand of S^T = K . Q^T - finds 16 distinct chunks per 16 lanes.
+    //   V: logical chunk c of row r at physical chunk c ^ ((r & 3) << 1), and the fills with an odd number (rows 4..7
+    //      of every eight) half a row askew, see dma_v_block8.  A transposing read touches, per 32 lanes, 8 rows x 32
+    //      bytes (rows 4 g + i / 4 for two values of g): rows 0..3 land in the four 32-byte granules of one half of
+    //      the 64 banks, rows 4..7 in the other half.  The 16 columns a read is for enter the address as 32 t: the
+    //      exclusive-or moves bits 5 and 6 only, so t / 4 is an offset in the instruction and a lane carries four
+    //      addresses.  (With the exclusive-or over all three bits, c ^ ((r & 7) << 1), the layout needs no askew
+    //      half - and eight addresses per lane, or two instructions per read to make them: both were measured,
+    //      the one spills registers, the other costs 40 % more vector instructions than the whole softmax.)
+    // A fill of 1 KB is 4 rows; wavefront wave8 issues fills wave8, wave8 + 8, ...: row = 4 blk + l / 16 with
+    // blk % 4 == wave8 % 4, so both swizzles are per-wavefront constants on the fill side.
     const int f_row = lane >> 4, f_c = lane & 15;
     const size_t k_pitch = (size_t)p.k_st[2] * sizeof(T), v_pitch = (size_t)p.v_st[2] * sizeof(T);
     const unsigned k_fill_off = (unsigned)(f_row * k_pitch + ((f_c ^ (4 * wave + f_row)) << 4));
-    const unsigned v_fill_off = (unsigned)(f_row * v_pitch + ((f_c ^ (f_row << 2)) << 4));
-    const int k_rd = r * kRowBytes;
-    const int i16 = lane & 15;
-    const int v_row = 4 * half + (i16 >> 2);
-    const int v_col_bytes = (16 * ((lane >> 4) & 1) + 4 * (i16 & 3)) * 2;
-    const int v_swz = (i16 >> 2) << 2;
+    const unsigned v_fill_off = (unsigned)(f_row * v_pitch + ((f_c ^ (f_row << 1)) << 4));
+    // K fragment of kv tile a, k step ks: row 16 a + c16, logical chunk 4 ks + g = 4 ks ^ g, physical (4 ks) ^ (g ^ c16)
+    const int k_rd = c16 * kRowBytes;
+    const int k_swz = (g ^ c16) << 4;
+    // V^T fragment of d tile t, kv step u: lane i of its 16 points at V[32 u + 4 g + i / 4][16 t + 4 (i % 4) ..] and
+    // receives V[32 u + 4 g + 0..3][16 t + i]; a second read 16 rows further down gives the other four k of the
+    // operand.  Row 32 u + 4 g + i / 4 is row i / 4 of fill 8 u + g: at 4096 u + 1024 (g / 2), askew if g is odd.
+    // v_rd[t % 4] + 128 (t / 4) + 4096 u (+ 2048 for the second read) is the address in the block.
     int v_rd[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-        v_rd[i] = v_row * kRowBytes + ((((4 * i + (v_col_bytes >> 4)) ^ v_swz) << 4) | (v_col_bytes & 15));
-    // logical chunk 2 ks + half of row r sits at physical chunk (2 ks + half) ^ (r & 15) = 2 ks ^ (half ^ (r & 15)): one
-    // register, and an exclusive-or with a constant per step (see `scores`)
-    const int k_swz = (half ^ (r & 15)) << 4;
+    for (int t = 0; t < 4; ++t)
+        v_rd[t] = (g >> 1) * 1024 + (g & 1) * kPairVOddFills + (c16 >> 2) * kRowBytes +
+                  (((2 * t + ((c16 & 3) >> 1)) ^ ((c16 >> 2) << 1)) << 4) + 8 * (c16 & 1);
 
     const T* __restrict__ Q = reinterpret_cast<const T*>(p.q);
     const unsigned char* __restrict__ K = reinterpret_cast<const unsigned char*>(p.k);
@@ -842,8 +962,8 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
         if (sig >= 0 && !wait_for_flag(sig, w)) return;
 
         const size_t head = (size_t)z * p.H + h;
-        const int q_row = qb * kBlockM + wave * 32 + r;
-        const T* q_src = Q + z * p.q_st[0] + h * p.q_st[1] + q_row * p.q_st[2] + 8 * half;
+        const int q_row = qb * kBlockM + wave * 32 + c16;          // and q_row + 16
+        const T* q_src = Q + z * p.q_st[0] + h * p.q_st[1] + q_row * p.q_st[2] + 8 * g;
         const unsigned char* const k_head = K + (z * p.k_st[0] + h * p.k_st[1]) * (int64_t)sizeof(T);
         const unsigned char* const v_head = V + (z * p.v_st[0] + h * p.v_st[1]) * (int64_t)sizeof(T);
 
@@ -938,18 +1058,25 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
         // every wavefront has passed the barrier that ended the previous segment: all four buffers are free
         dma_kv_block8(k_lds, k_walk + (size_t)k_rot * kBlockN * k_pitch, k_pitch, k_fill_off, wave8);
 
-        frag_t qf[8];
+        // Q^T operands of the two 16-row halves of the slice: [b][ks] = Q[q_row + 16 b][32 ks + 8 g .. + 8]
+        frag_t qf[2][4];
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) qf[ks] = *reinterpret_cast<const frag_t*>(q_src + 16 * ks);
-        f32x16_t o_acc[4];
+        for (int b = 0; b < 2; ++b)
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+            for (int ks = 0; ks < 4; ++ks) qf[b][ks] = *reinterpret_cast<const frag_t*>(q_src + 16 * b * p.q_st[2] + 32 * ks);
+        // O^T: [t][b] = columns 16 t + 4 g + 0..3 of q row 16 b + c16
+        f32x4_t o_acc[8][2];
 #pragma unroll
-            for (int e2 = 0; e2 < 16; ++e2) o_acc[i][e2] = 0.f;
-        float m_i = -INFINITY;
-        float l_i = 0.f;
-        f32x16_t s[4];
-        frag_t pf[8];
+        for (int t = 0; t < 8; ++t)
+#pragma unroll
+            for (int b = 0; b < 2; ++b) o_acc[t][b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        float m_i[2] = {-INFINITY, -INFINITY};
+        float l_i[2] = {0.f, 0.f};
+        // S^T: [a][b] = kv positions 16 a + 4 g + 0..3 of the block against q row 16 b + c16
+        f32x4_t s[8][2];
+        // P^T operands: [b][u] holds, as k 8 g + x, the kv position 16 (2 u + x / 4) + 4 g + x % 4 - the lane's own
+        // probabilities of the tiles 2 u and 2 u + 1; the V^T operand reads its rows in the same order
+        frag_t pf[2][4];
 
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_waitcnt(attn_vmcnt(0));       // K block 0 (and Q) have landed
@@ -975,7 +1102,7 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
             }
             int b = v_next + v_rot;
             b = b >= v_nkv ? b - v_nkv : b;
-            dma_kv_block8(v_lds + (m & 1) * kBlockBytes, v_walk + (size_t)b * kBlockN * v_pitch, v_pitch, v_fill_off, wave8);
+            dma_v_block8(v_lds + (m & 1) * kPairVBlockBytes, v_walk + (size_t)b * kBlockN * v_pitch, v_pitch, v_fill_off, wave8);
             ++v_next;
             int more = 1;
             if (k_next == k_nkv) more = enter_next_visit();
@@ -991,41 +1118,46 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
             return __builtin_amdgcn_readfirstlane(more);       // the same in every lane: a scalar for the compiler too
         };
 
-        // S^T = K(n) . Q^T
+        constexpr int kG = 4, kPer = 8 / kG, kGroups = 4 * kPer;          // V^T fragments per group of products, groups per step
+        constexpr int kGS = 2, kPerS = 8 / kGS, kGroupsS = 4 * kPerS;     // the same for the K fragments of the scores
+        // S^T = K(n) . Q^T: 8 kv tiles x 4 k steps, each K fragment against the two halves of the q slice
         auto scores = [&](const int n) __attribute__((always_inline)) {
-            const f32x16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-            // fragments of steps ks and ks + 1 are in registers; the register a product has just
-            // consumed is refilled with the fragment of step ks + 2, so a read has almost two steps
-            // (256 MFMA cycles) to come back
-            frag_t kf[2][4];
+            const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
+            // group u = k step u / 2, kv tiles 4 (u % 2) .. + 4.  The fragments of groups u and u + 1 are in registers;
+            // the register a pair of products has just consumed is refilled with the fragment of group u + 2, so a
+            // read has almost two groups (256 MFMA cycles) to come back
+            frag_t kf[2][kGS];
             const unsigned char* k_row = k_lds + (n & 1) * kBlockBytes + k_rd;
-            // (opaque to the compiler, which would otherwise carry the eight chunk offsets in eight registers around
-            // the loop over kv blocks - registers this kernel does not have)
+            // (opaque to the compiler, which would otherwise carry the four chunk offsets in registers around the loop
+            // over kv blocks - registers this kernel does not have)
             int swz = k_swz;
             asm volatile("" : "+v"(swz));
-            auto k_chunk = [&](const int ks) __attribute__((always_inline)) { return swz ^ (32 * ks); };
+            auto k_at = [&](const int u, const int j) __attribute__((always_inline)) {
+                return k_row + 16 * (kGS * (u % kPerS) + j) * kRowBytes + (swz ^ (64 * (u / kPerS)));
+            };
 #pragma unroll
-            for (int b = 0; b < 2; ++b)
+            for (int u = 0; u < 2; ++u)
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    kf[b][j] = *reinterpret_cast<const frag_t*>(k_row + 32 * j * kRowBytes + k_chunk(b));
-            __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+                for (int j = 0; j < kGS; ++j) kf[u][j] = *reinterpret_cast<const frag_t*>(k_at(u, j));
+            __builtin_amdgcn_sched_group_barrier(0x100, 2 * kGS, 0);
 #pragma unroll
-            for (int ks = 0; ks < 8; ++ks) {
+            for (int u = 0; u < kGroupsS; ++u) {
+                const int ks = u / kPerS;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    s[j] = AttnMfma<T>::run(kf[ks & 1][j], qf[ks], ks == 0 ? zero : s[j]);
-                    if (ks + 2 < 8)
-                        kf[ks & 1][j] = *reinterpret_cast<const frag_t*>(k_row + 32 * j * kRowBytes + k_chunk(ks + 2));
+                for (int j = 0; j < kGS; ++j) {
+                    const int a = kGS * (u % kPerS) + j;
+#pragma unroll
+                    for (int b = 0; b < 2; ++b) s[a][b] = mfma16<T>(kf[u & 1][j], qf[b][ks], ks == 0 ? zero : s[a][b]);
+                    if (u + 2 < kGroupsS) kf[u & 1][j] = *reinterpret_cast<const frag_t*>(k_at(u + 2, j));
                 }
-                if (ks + 2 < 8) {
+                if (u + 2 < kGroupsS) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    for (int j = 0; j < kGS; ++j) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
                         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
                     }
                 } else {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 2 * kGS, 0);
                 }
             }
         };
@@ -1037,75 +1169,101 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
         // exact zeros.
         auto softmax = [&](const int past) __attribute__((always_inline)) {
             if ((CAUSAL || MODE != kPairTiles) && past > 0) {
-                const int lim = wave * 32 + r - 4 * half - (past - 1) * kBlockN;     // mask where 32j + 8(e/4) + e%4 > lim
+                // q row wave * 32 + 16 b + c16 against kv position 16 a + 4 g + i of the block
+                const int lim = wave * 32 + c16 - 4 * g - (past - 1) * kBlockN;     // mask where 16 a + i > lim + 16 b
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
+                for (int a = 0; a < 8; ++a)
 #pragma unroll
-                    for (int e2 = 0; e2 < 16; ++e2)
-                        if (32 * j + 8 * (e2 >> 2) + (e2 & 3) > lim) s[j][e2] = -INFINITY;
+                    for (int b = 0; b < 2; ++b)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            if (16 * a + i - 16 * b > lim) s[a][b][i] = -INFINITY;
             }
-            float mx = -INFINITY;
+            float mx[2] = {-INFINITY, -INFINITY};
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+            for (int a = 0; a < 8; ++a)
 #pragma unroll
-                for (int e2 = 0; e2 < 16; ++e2) mx = fmaxf(mx, s[j][e2]);
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
-            const float m_new = fmaxf(m_i, mx * p.qk_scale);
-            const float alpha = fast_exp2(m_i - m_new);
-            if (__builtin_amdgcn_ballot_w64(m_new != m_i) != 0) {
+                for (int b = 0; b < 2; ++b)
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
+                    for (int i = 0; i < 4; ++i) mx[b] = fmaxf(mx[b], s[a][b][i]);
+            float m_new[2], alpha[2];
 #pragma unroll
-                    for (int e2 = 0; e2 < 16; ++e2) o_acc[i][e2] *= alpha;
+            for (int b = 0; b < 2; ++b) {
+                mx[b] = fmaxf(mx[b], __shfl_xor(mx[b], 16));
+                mx[b] = fmaxf(mx[b], __shfl_xor(mx[b], 32));
+                m_new[b] = fmaxf(m_i[b], mx[b] * p.qk_scale);
+                alpha[b] = fast_exp2(m_i[b] - m_new[b]);
             }
-            float row_sum = 0.f;
+            if (__builtin_amdgcn_ballot_w64(m_new[0] != m_i[0] || m_new[1] != m_i[1]) != 0) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+                for (int t = 0; t < 8; ++t)
 #pragma unroll
-                for (int e2 = 0; e2 < 16; ++e2) {
-                    const float pe = fast_exp2(s[j][e2] * p.qk_scale - m_new);
-                    row_sum += pe;
-                    pf[2 * j + (e2 >> 3)][e2 & 7] = (T)pe;
-                }
-            l_i = l_i * alpha + row_sum;
-            m_i = m_new;
-        };
-
-        // O^T += V(n)^T . P^T
-        auto weighted_values = [&](const int n) __attribute__((always_inline)) {
-            typedef short s16x8_t __attribute__((ext_vector_type(8)));
-            const unsigned char* v_blk = v_lds + (n & 1) * kBlockBytes;
-            s16x4_t vlo[2][4], vhi[2][4];
+                    for (int b = 0; b < 2; ++b)
 #pragma unroll
-            for (int b = 0; b < 2; ++b)
+                        for (int i = 0; i < 4; ++i) o_acc[t][b][i] *= alpha[b];
+            }
+            float row_sum[2] = {0.f, 0.f};
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const unsigned char* src = v_blk + 16 * b * kRowBytes + v_rd[i];
-                    vlo[b][i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)src);
-                    vhi[b][i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(src + 8 * kRowBytes));
-                }
-            __builtin_amdgcn_sched_group_barrier(0x100, 16, 0);
+            for (int a = 0; a < 8; ++a)
 #pragma unroll
-            for (int t2 = 0; t2 < 8; ++t2) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const s16x4_t lo = vlo[t2 & 1][i], hi = vhi[t2 & 1][i];
-                    const s16x8_t both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                    o_acc[i] = AttnMfma<T>::run(__builtin_bit_cast(frag_t, both), pf[t2], o_acc[i]);
-                    if (t2 + 2 < 8) {
-                        const unsigned char* src = v_blk + 16 * (t2 + 2) * kRowBytes + v_rd[i];
-                        vlo[t2 & 1][i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)src);
-                        vhi[t2 & 1][i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(src + 8 * kRowBytes));
-                    }
-                }
-                if (t2 + 2 < 8) {
+                for (int b = 0; b < 2; ++b)
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
-                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        const float pe = fast_exp2(s[a][b][i] * p.qk_scale - m_new[b]);
+                        row_sum[b] += pe;
+                        pf[b][a >> 1][4 * (a & 1) + i] = (T)pe;
+                    }
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                l_i[b] = l_i[b] * alpha[b] + row_sum[b];
+                m_i[b] = m_new[b];
+            }
+        };
+
+        // O^T += V(n)^T . P^T: 8 d tiles x 4 kv steps of 32, each V^T fragment against the two halves of the q slice
+        auto weighted_values = [&](const int n) __attribute__((always_inline)) {
+            typedef short s16x8_t __attribute__((ext_vector_type(8)));
+            const unsigned char* v_blk = v_lds + (n & 1) * kPairVBlockBytes;
+            // group w = kv step w / kPer, d tiles kG (w % kPer) .. + kG
+            auto v_at = [&](const int w, const int j) __attribute__((always_inline)) {
+                const int t = kG * (w % kPer) + j;
+                return v_blk + 4096 * (w / kPer) + 128 * (t >> 2) + v_rd[t & 3];
+            };
+            s16x4_t vlo[2][kG], vhi[2][kG];
+#pragma unroll
+            for (int w = 0; w < 2; ++w)
+#pragma unroll
+                for (int j = 0; j < kG; ++j) {
+                    const unsigned char* src = v_at(w, j);
+                    vlo[w][j] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)src);
+                    vhi[w][j] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(src + 2048));
+                }
+            __builtin_amdgcn_sched_group_barrier(0x100, 4 * kG, 0);
+#pragma unroll
+            for (int w = 0; w < kGroups; ++w) {
+                const int u = w / kPer;
+#pragma unroll
+                for (int j = 0; j < kG; ++j) {
+                    const int t = kG * (w % kPer) + j;
+                    const s16x4_t lo = vlo[w & 1][j], hi = vhi[w & 1][j];
+                    const s16x8_t both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+#pragma unroll
+                    for (int b = 0; b < 2; ++b)
+                        o_acc[t][b] = mfma16<T>(__builtin_bit_cast(frag_t, both), pf[b][u], o_acc[t][b]);
+                    if (w + 2 < kGroups) {
+                        const unsigned char* src = v_at(w + 2, j);
+                        vlo[w & 1][j] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)src);
+                        vhi[w & 1][j] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(src + 2048));
+                    }
+                }
+                if (w + 2 < kGroups) {
+#pragma unroll
+                    for (int j = 0; j < kG; ++j) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
                         __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
                     }
                 } else {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 2 * kG, 0);
                 }
             }
         };
@@ -1175,13 +1333,18 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
         }
 
         // ---- epilogue: lse2 = m + log2(l), O = acc / l, merged into the output under the q blocks' locks ----
-        const float l_tot = l_i + __shfl_xor(l_i, 32);
-        const float lse2 = m_i + fast_log2(l_tot);
-        const float inv_l = 1.0f / l_tot;
+        float lse2[2], inv_l[2];
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            float l_tot = l_i[b] + __shfl_xor(l_i[b], 16);
+            l_tot += __shfl_xor(l_tot, 32);
+            lse2[b] = m_i[b] + fast_log2(l_tot);
+            inv_l[b] = 1.0f / l_tot;
+        }
         const int lock_idx = (int)(head * (p.Sq / kBlockM)) + qb;
         if (sole_writer) {
             // the only segment that writes these q blocks: nothing to merge with and nobody to exclude
-            merge_rows_through_lds<T>(wave8 < 4 ? k_lds + wave8 * kStageBytes : v_lds + (wave8 - 4) * kStageBytes,
+            merge_rows16_through_lds<T>(wave8 < 4 ? k_lds + wave8 * kStageBytes : v_lds + (wave8 - 4) * kStageBytes,
                                       O + z * p.o_st[0] + h * p.o_st[1] + (int64_t)(qb * kBlockM + wave * 32) * p.o_st[2], p.o_st[2],
                                       p.lse + head * p.Sq + qb * kBlockM + wave * 32, o_acc, inv_l, lse2, true, lane);
             __syncthreads();       // the tiles in LDS are free for the next segment's fills
@@ -1215,7 +1378,7 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
         if (__builtin_amdgcn_readfirstlane(s_abort)) return;
         const bool is_first = __builtin_amdgcn_readfirstlane(s_spun) != 0;
         // (the K and V blocks are free: every wavefront has passed the last slot's barrier)
-        merge_rows_through_lds<T>(wave8 < 4 ? k_lds + wave8 * kStageBytes : v_lds + (wave8 - 4) * kStageBytes,
+        merge_rows16_through_lds<T>(wave8 < 4 ? k_lds + wave8 * kStageBytes : v_lds + (wave8 - 4) * kStageBytes,
                                   O + z * p.o_st[0] + h * p.o_st[1] + (int64_t)(qb * kBlockM + wave * 32) * p.o_st[2], p.o_st[2],
                                   p.lse + head * p.Sq + qb * kBlockM + wave * 32, o_acc, inv_l, lse2, is_first, lane);
 

@@ -347,8 +347,9 @@ def test_more_waves_than_a_wavefront_has_lanes(hip, pair):
                           cum_wave_sizes=cums, signal_ptr=flags, signal_offsets=signals, NUM_WAVES=128, cum_tiles=total,
                           visit_log=log, pair_q_blocks=pair, num_programs=3)
     check_status()
-    # eighty partial results merged with a rounding each: twice the usual bound
-    assert _rel(o, numerics.sdpa_fp32(q, k, v, sm_scale)) <= 2 * REL_TOL
+    # eighty partial results merged with a rounding to bf16 each (a random walk of 80 steps of up to 2^-9, in the order in
+    # which the programs happen to take the locks: 0.016 to 0.021 from run to run): three times the usual bound
+    assert _rel(o, numerics.sdpa_fp32(q, k, v, sm_scale)) <= 3 * REL_TOL
     for tile_id, rec in enumerate(log.cpu().tolist()):
         exp = visit_order.attn_tile_work(tile_id, offsets, sizes, cums, signals)
         assert rec[:7] == [exp["wave"], exp["z"], exp["h"], exp["q_block"], exp["kv_lo"], exp["kv_hi"], exp["signal"]]
