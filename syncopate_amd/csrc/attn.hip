@@ -143,6 +143,24 @@ __device__ __forceinline__ void store_f32_through(float* ptr, float value) {
 __device__ __forceinline__ void lock_release_fence() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup"); }
 __device__ __forceinline__ void lock_taken_fence() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup"); }
 
+// max(x of this lane, x of lane ^ 32) and the same for lane ^ 16, on the vector ALU: v_permlane32_swap exchanges
+// lanes 32..63 of its first operand with lanes 0..31 of its second, v_permlane16_swap the odd rows of 16 lanes of the
+// first with the even rows of the second - given two copies of x, every lane then holds its own value in one and
+// its partner's in the other.  (__shfl_xor is an LDS instruction, ds_bpermute: in the paired kernel it would queue
+// behind the LDS reads of the four wavefronts that are in their products, and the softmax waits for it twice.)
+// Written as assembly because the compiler's own builtins for these two instructions fold max(first result, second
+// result) into the first result; the s_nop before and after are the ones it places around them itself.
+__device__ __forceinline__ float max_with_lane_xor32(float x) {
+    float a = x, b = x;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    return fmaxf(a, b);
+}
+__device__ __forceinline__ float max_with_lane_xor16(float x) {
+    float a = x, b = x;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    return fmaxf(a, b);
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
@@ -1120,12 +1138,13 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
 
         constexpr int kG = 4, kPer = 8 / kG, kGroups = 4 * kPer;          // V^T fragments per group of products, groups per step
         constexpr int kGS = 2, kPerS = 8 / kGS, kGroupsS = 4 * kPerS;     // the same for the K fragments of the scores
-        // S^T = K(n) . Q^T: 8 kv tiles x 4 k steps, each K fragment against the two halves of the q slice
+        // S^T = K(n) . Q^T: 8 kv tiles x 4 k steps, each K fragment against the two halves of the q slice.
+        // Group u = k step u / kPerS, kv tiles kGS (u % kPerS) .. + kGS.  The fragments of groups u and u + 1 are in
+        // registers; the register a pair of products has just consumed is refilled with the fragment of group u + 2, so
+        // a read has almost two groups (128 MFMA cycles) to come back.  (Asking for the first two groups' fragments
+        // sixteen products before the end of weighted_values, into registers of used-up probabilities, measured the same.)
         auto scores = [&](const int n) __attribute__((always_inline)) {
             const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
-            // group u = k step u / 2, kv tiles 4 (u % 2) .. + 4.  The fragments of groups u and u + 1 are in registers;
-            // the register a pair of products has just consumed is refilled with the fragment of group u + 2, so a
-            // read has almost two groups (256 MFMA cycles) to come back
             frag_t kf[2][kGS];
             const unsigned char* k_row = k_lds + (n & 1) * kBlockBytes + k_rd;
             // (opaque to the compiler, which would otherwise carry the four chunk offsets in registers around the loop
@@ -1189,8 +1208,7 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
             float m_new[2], alpha[2];
 #pragma unroll
             for (int b = 0; b < 2; ++b) {
-                mx[b] = fmaxf(mx[b], __shfl_xor(mx[b], 16));
-                mx[b] = fmaxf(mx[b], __shfl_xor(mx[b], 32));
+                mx[b] = max_with_lane_xor32(max_with_lane_xor16(mx[b]));
                 m_new[b] = fmaxf(m_i[b], mx[b] * p.qk_scale);
                 alpha[b] = fast_exp2(m_i[b] - m_new[b]);
             }
