@@ -718,10 +718,10 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
 //   group 1      -      S0     sm0        PV0,S1     sm1              sm(N-1)    PV(N-1)
 //
 // so in every slot the two wavefronts of a SIMD use different pipes.  Both groups read K and V
-// from the same LDS blocks (half the fills per q row); K and V are double buffered: V(n) and
-// K(n+1) are fetched at slot 2n by all eight wavefronts, into the buffers whose last readers
-// (V(n-2), K(n-1)) finished in slot 2n-1, and have landed by the end of slot 2n+1.  One barrier
-// per slot, i.e. two per kv block and wavefront instead of four.
+// from the same LDS blocks (half the fills per q row); K and V are double buffered: K(n+1) is
+// fetched in slot 2n and V(n) in slot 2n+1, each by the group that is in its softmax, into the buffers
+// whose last readers (K(n-1), V(n-2)) finished in slot 2n-1, and have landed by the end of slot 2n+1.
+// One barrier per slot, i.e. two per kv block and wavefront instead of four.
 //
 // The products are 16 x 16 x 32 MFMAs (a wavefront's 32 q rows as two halves of 16 that share every K and V
 // fragment).  With 32 x 32 x 16 products - the same flop, the same LDS reads, a third fewer vector instructions
@@ -732,13 +732,35 @@ __global__ void __launch_bounds__(kAttnThreads, 2) attn_fwd_kernel(const AttnPar
 constexpr int kPairThreads = 512;
 constexpr int kPairFills = kBlockBytes / 1024 / 8;      // 4 fills of 1 KB per wavefront and block
 
+// A fill of the paired kernel: 16 bytes per lane from `src` to LDS at `lds` + 16 * lane, written as assembly so that
+// the COMPILER DOES NOT KNOW OF IT.  Told of a load into LDS (the builtin), it makes every later LDS read wait for
+// it, s_waitcnt vmcnt(0) - it cannot tell that the read is of another buffer - and the wavefronts whose products
+// follow their fills stood still until their own fills had crossed the memory system: the slots with fills took
+// 5400 cycles, the others 2800.  What has to wait for a fill does so in the kernel's own s_waitcnt vmcnt(0): before
+// the barrier that ends an odd slot, and before the first products of a segment.  (Untold loads in flight make the
+// compiler's own vmcnt counts for its loads and stores wait for more than they need, never for less: the counter
+// retires in order.)
+__device__ __forceinline__ void fill16_untold(const unsigned char* src, const unsigned char* lds) {
+    const unsigned lds_addr = (unsigned)(uintptr_t)(lds_void_ptr)lds;
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(lds_addr) : "m0");
+}
+
 __device__ __forceinline__ void dma_kv_block8(unsigned char* lds, const unsigned char* src, size_t pitch,
                                               unsigned lane_off, int wave8) {
 #pragma unroll
     for (int i = 0; i < kPairFills; ++i) {
         const int blk = i * 8 + wave8;                  // blk % 4 == wave8 % 4: the swizzle of the 4-wave form holds
-        __builtin_amdgcn_global_load_lds((global_void_ptr)(src + (size_t)(blk * 4) * pitch + lane_off),
-                                         (lds_void_ptr)(lds + blk * 1024), 16, 0, 0);
+        fill16_untold(src + (size_t)(blk * 4) * pitch + lane_off, lds + blk * 1024);
+    }
+}
+
+// The same block by four wavefronts (`wave` = 0..3): fills wave, wave + 4, ...
+__device__ __forceinline__ void dma_kv_block4(unsigned char* lds, const unsigned char* src, size_t pitch,
+                                              unsigned lane_off, int wave) {
+#pragma unroll
+    for (int i = 0; i < 2 * kPairFills; ++i) {
+        const int blk = i * 4 + wave;
+        fill16_untold(src + (size_t)(blk * 4) * pitch + lane_off, lds + blk * 1024);
     }
 }
 
@@ -748,13 +770,12 @@ __device__ __forceinline__ void dma_kv_block8(unsigned char* lds, const unsigned
 // for every 16 columns (see the kernel's note on its layouts).
 constexpr int kPairVOddFills = kBlockBytes / 2 + 128;
 constexpr int kPairVBlockBytes = kBlockBytes + 1024;
-__device__ __forceinline__ void dma_v_block8(unsigned char* lds, const unsigned char* src, size_t pitch,
-                                             unsigned lane_off, int wave8) {
+__device__ __forceinline__ void dma_v_block4(unsigned char* lds, const unsigned char* src, size_t pitch,
+                                             unsigned lane_off, int wave) {
 #pragma unroll
-    for (int i = 0; i < kPairFills; ++i) {
-        const int blk = i * 8 + wave8;
-        __builtin_amdgcn_global_load_lds((global_void_ptr)(src + (size_t)(blk * 4) * pitch + lane_off),
-                                         (lds_void_ptr)(lds + (blk >> 1) * 1024 + (wave8 & 1) * kPairVOddFills), 16, 0, 0);
+    for (int i = 0; i < 2 * kPairFills; ++i) {
+        const int blk = i * 4 + wave;
+        fill16_untold(src + (size_t)(blk * 4) * pitch + lane_off, lds + (blk >> 1) * 1024 + (wave & 1) * kPairVOddFills);
     }
 }
 
@@ -815,7 +836,7 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
     //   K: logical chunk c of row r at physical chunk c ^ (r & 15): a 16-byte read per lane of the rows 16 a + l % 16
     //      at the chunk 4 ks + l / 16 - an A operand of S^T = K . Q^T - finds 16 distinct chunks per 16 lanes.
     //   V: logical chunk c of row r at physical chunk c ^ ((r & 3) << 1), and the fills with an odd number (rows 4..7
-    //      of every eight) half a row askew, see dma_v_block8.  A transposing read touches, per 32 lanes, 8 rows x 32
+    //      of every eight) half a row askew, see dma_v_block4.  A transposing read touches, per 32 lanes, 8 rows x 32
     //      bytes (rows 4 g + i / 4 for two values of g): rows 0..3 land in the four 32-byte granules of one half of
     //      the 64 banks, rows 4..7 in the other half.  The 16 columns a read is for enter the address as 32 t: the
     //      exclusive-or moves bits 5 and 6 only, so t / 4 is an offset in the instruction and a lane carries four
@@ -1101,13 +1122,24 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
 
-        // V(m) and K(m+1) are fetched at the start of slot 2m by every wavefront and are first read in
-        // slot 2m + 2; their buffers were last read in slot 2m - 1.  (Spreading the fills between the
-        // products or the exponentials, or leaving them all to the group that is in its softmax,
-        // measured 1-6 % slower: a wavefront stalls at every fill wherever it is placed.)
-        // Returns 1 when K(m+1) was asked for, 0 when block m is the segment's last, -1 to give up (a flag did
+        // V(m) and K(m+1) are fetched in slots 2m and 2m + 1 and are first read in slot 2m + 2; their buffers were last
+        // read in slot 2m - 1.  A wavefront stands still for some 350 cycles at every fill it issues, wherever the fill
+        // is placed, so the fills are left to the group that is in its softmax, which has a thousand cycles to spare
+        // beside the other group's products: group 1 asks for K(m+1) at the start of slot 2m (in `fetch`), group 0 for
+        // V(m) at the start of slot 2m + 1 (`fill_v`), four wavefronts a block.  Every wavefront waits for its own fills
+        // before the barrier that ends slot 2m + 1.  (Measured against every wavefront issuing an eighth of both blocks
+        // at the start of slot 2m: 1 to 3 % faster.  The softmax before the fills, or the fills spread among the
+        // products, or the next blocks touched ahead so that the fills hit in the L2: the same or slower.)
+        // `fetch` returns 1 when K(m+1) was asked for, 0 when block m is the segment's last, -1 to give up (a flag did
         // not come within the time limit, or the next visit is not one of this segment's: every wavefront is
         // told so at the same fetch, and the program ends).
+        const unsigned char* v_src_pending = nullptr;
+        int v_buf_pending = 0;
+        auto fill_v = [&]() __attribute__((always_inline)) {
+            __builtin_amdgcn_sched_barrier(0);
+            dma_v_block4(v_lds + v_buf_pending * kPairVBlockBytes, v_src_pending, v_pitch, v_fill_off, wave);
+            __builtin_amdgcn_sched_barrier(0);
+        };
         auto fetch = [&](const int m) __attribute__((always_inline)) -> int {
             __builtin_amdgcn_sched_barrier(0);
             // block m is the first of a new visit exactly when the V walk has used its visit up; the K walk
@@ -1120,15 +1152,16 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
             }
             int b = v_next + v_rot;
             b = b >= v_nkv ? b - v_nkv : b;
-            dma_v_block8(v_lds + (m & 1) * kPairVBlockBytes, v_walk + (size_t)b * kBlockN * v_pitch, v_pitch, v_fill_off, wave8);
+            v_src_pending = v_walk + (size_t)b * kBlockN * v_pitch;       // for group 0's fill_v, one slot on
+            v_buf_pending = m & 1;
             ++v_next;
             int more = 1;
             if (k_next == k_nkv) more = enter_next_visit();
             if (more > 0) {
                 b = k_next + k_rot;
                 b = b >= k_nkv ? b - k_nkv : b;
-                dma_kv_block8(k_lds + ((m + 1) & 1) * kBlockBytes, k_walk + (size_t)b * kBlockN * k_pitch, k_pitch, k_fill_off,
-                              wave8);
+                if (grp == 1)
+                    dma_kv_block4(k_lds + ((m + 1) & 1) * kBlockBytes, k_walk + (size_t)b * kBlockN * k_pitch, k_pitch, k_fill_off, wave);
                 ++k_next;
                 if constexpr (CAUSAL) m2 = beyond(k_lo + b);
             }
@@ -1312,7 +1345,8 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
             scores(0);
             end_even();
             while (more > 0) {
-                softmax(m0);                          // slot 2n + 1
+                fill_v();                             // slot 2n + 1: V(n)
+                softmax(m0);
                 end_odd();
                 more = fetch(n + 1);                     // slot 2n + 2
                 if (more < 0) return;
@@ -1323,7 +1357,8 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
                 m0 = m1;
                 m1 = m2;
             }
-            softmax(m0);                              // slot 2N - 1
+            fill_v();                                 // slot 2N - 1
+            softmax(m0);
             end_odd();
             weighted_values(n);                   // slot 2N
             end_even();
