@@ -873,7 +873,8 @@ def run_attention_a2a(device, launches=10, gated=True):
 def run_attention_slot(device, launches=10):
     """What the pieces of the paired attention kernel's slot cost beside each other (`syn_probe_attn_slot`): the 64
     MFMAs of a slot on register operands, fed from LDS through the kernel's reads, beside the other group's softmax,
-    with the fills, with the first fragments of a phase asked for early, on constant and on random operands.  Per
+    with the fills, with the first fragments of a phase asked for early, on constant and on random operands, and with
+    the products as pairs of 16x16x32 MFMAs instead of 32x32x16 ones.  Per
     configuration: time and shader-clock cycles per slot, the clock the device held (cycles / time), and the rate
     the slot's products run at, as a fraction of the matrix pipes' peak.  2048 matrix-pipe cycles per slot."""
     from syncopate_amd import _lib
@@ -884,7 +885,7 @@ def run_attention_slot(device, launches=10):
     sink = torch.empty(workgroups * 512, dtype=torch.float32, device=device)
     cycles = torch.zeros(2, dtype=torch.int64, device=device)
     stream = _lib.stream_handle(torch.cuda.current_stream())
-    PRODUCTS, SOFTMAX, LDS, FILLS, PREFETCH, RANDOM, PRIVATE = 1, 2, 4, 8, 16, 32, 64
+    PRODUCTS, SOFTMAX, LDS, FILLS, PREFETCH, RANDOM, PRIVATE, NARROW = 1, 2, 4, 8, 16, 32, 64, 128
     configs = (("products_register_operands", PRODUCTS),
                ("products_from_lds", PRODUCTS | LDS),
                ("softmax_alone", SOFTMAX),
@@ -896,7 +897,12 @@ def run_attention_slot(device, launches=10):
                ("products_from_lds_random", PRODUCTS | LDS | RANDOM),
                ("products_from_lds_beside_softmax_random", PRODUCTS | LDS | SOFTMAX | RANDOM),
                ("products_from_lds_beside_softmax_with_fills_random", PRODUCTS | LDS | SOFTMAX | FILLS | RANDOM),
-               ("same_fragments_asked_for_a_phase_early_random", PRODUCTS | LDS | SOFTMAX | FILLS | PREFETCH | RANDOM))
+               ("same_fragments_asked_for_a_phase_early_random", PRODUCTS | LDS | SOFTMAX | FILLS | PREFETCH | RANDOM),
+               # the same slot with every 32x32x16 product as two 16x16x32 products (the form the kernel uses)
+               ("narrow_products_register_operands_random", PRODUCTS | RANDOM | NARROW),
+               ("narrow_products_from_lds_beside_softmax_random", PRODUCTS | LDS | SOFTMAX | RANDOM | NARROW),
+               ("narrow_products_from_lds_beside_softmax_with_fills_random", PRODUCTS | LDS | SOFTMAX | FILLS | RANDOM | NARROW),
+               ("narrow_products_from_lds_beside_softmax_with_fills", PRODUCTS | LDS | SOFTMAX | FILLS | NARROW))
     out = {"workgroups": workgroups, "slots_per_launch": iters, "launches": launches, "matrix_pipe_cycles_per_slot": 2048}
     flop_per_slot = workgroups * 4 * 64 * 32768.0
     for name, what in (("warm-up", configs[-2][1]),) + configs:
@@ -1251,7 +1257,7 @@ def main():
         line["attn_all2all"] = run_attention_a2a(device, gated=gated)
     if "attn_slot" in only:
         line["attn_slot_probe"] = run_attention_slot(device)
-        slot = line["attn_slot_probe"]["products_from_lds_beside_softmax_with_fills_random"]["products_tflops"]
+        slot = line["attn_slot_probe"]["narrow_products_from_lds_beside_softmax_with_fills_random"]["products_tflops"]
         # the kernels' rates against the bare slot loop's (same MFMAs, LDS reads, softmax and fills on random operands,
         # nothing else): what is left is the kernels' own doing, the rest is the board's power limit
         if "attn_allgather" in line:

@@ -495,7 +495,8 @@ int syn_probe_read_streams_skewed(const void* base, int64_t stream_bytes, int64_
  * operands), 8 every wavefront issues four 1 KB LDS-DMA fills per slot from `pool`, 16 (with 4) the first
  * fragments of a phase are asked for in the tail of the previous one, 32 pseudo-random operands instead of a
  * constant, 64 a workgroup's fills read a region of its own (L2 misses; else all workgroups read the same 32 KB
- * piece per slot: L2 hits but for the first reader of an XCD).  pool: device memory of at least 65536 * workgroups + 32 MiB bytes, 16-byte aligned.  sink: device
+ * piece per slot: L2 hits but for the first reader of an XCD), 128 (with 1) every 32x32x16 MFMA is replaced by two
+ * 16x16x32 MFMAs that share its A operand - the same flop and LDS reads, the form attn_pair_kernel uses.  pool: device memory of at least 65536 * workgroups + 32 MiB bytes, 16-byte aligned.  sink: device
  * float[512 * workgroups].  cycles: device int64[2], the shader-clock cycles workgroup 0 spent in the loop
  * (wavefront 0, wavefront 4); with the launch's duration they give the clock the device held.
  * matrix-pipe cycles per slot: 2048. */

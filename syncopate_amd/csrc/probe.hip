@@ -157,9 +157,12 @@ read_streams_kernel(const u32x4_probe_t* __restrict__ base, int64_t stride_vecs,
 //   kSlotRandom     LDS and the register operands hold pseudo-random values instead of one constant
 //   kSlotPrivate    a workgroup's fills read a region of its own (misses in the L2); else every workgroup reads the
 //                   same 32 KB piece per slot - one miss per XCD, then L2 hits, like programs that walk one head's K, V
+//   kSlotNarrow     every 32x32x16 MFMA is replaced by two 16x16x32 MFMAs that share its A operand (the same flop,
+//                   the same LDS reads, half of the accumulator registers): the form attn_pair_kernel uses, whose
+//                   32 q rows per wavefront are two halves of 16
 // A slot ends like the kernel's: wait for the wavefront's own LDS reads (and fills), then the barrier.
 constexpr int kSlotProducts = 1, kSlotSoftmax = 2, kSlotLds = 4, kSlotFills = 8, kSlotPrefetch = 16, kSlotRandom = 32,
-              kSlotPrivate = 64;
+              kSlotPrivate = 64, kSlotNarrow = 128;
 constexpr int kSlotRowBytes = 256, kSlotBlockBytes = 32768;
 typedef short slot_s16x4_t __attribute__((ext_vector_type(4)));
 typedef short slot_s16x8_t __attribute__((ext_vector_type(8)));
@@ -167,8 +170,16 @@ typedef __attribute__((address_space(3))) slot_s16x4_t* slot_lds_s16x4_ptr;
 typedef __attribute__((address_space(3))) void* slot_lds_ptr;
 typedef const __attribute__((address_space(1))) void* slot_global_ptr;
 
-__device__ __forceinline__ f32x16_t slot_mfma(bf16x8_t a, bf16x8_t b, f32x16_t c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+typedef float slot_f32x4_t __attribute__((ext_vector_type(4)));
+template <bool NARROW>
+__device__ __forceinline__ f32x16_t slot_mfma(bf16x8_t a, bf16x8_t b, bf16x8_t b2, f32x16_t c) {
+    if (!NARROW) return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    slot_f32x4_t lo = {c[0], c[1], c[2], c[3]}, hi = {c[4], c[5], c[6], c[7]};
+    lo = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, lo, 0, 0, 0);
+    hi = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b2, hi, 0, 0, 0);
+    c[0] = lo[0]; c[1] = lo[1]; c[2] = lo[2]; c[3] = lo[3];
+    c[4] = hi[0]; c[5] = hi[1]; c[6] = hi[2]; c[7] = hi[3];
+    return c;
 }
 
 __device__ __forceinline__ void slot_fills(unsigned char* lds, const unsigned char* src, int wave8, int lane) {
@@ -190,7 +201,7 @@ __device__ __forceinline__ void slot_end(bool fills) {
     __builtin_amdgcn_sched_barrier(0);
 }
 
-template <bool LDS, bool PREFETCH>
+template <bool LDS, bool PREFETCH, bool NARROW>
 __device__ __forceinline__ void slot_products(int what, int iters, unsigned char* k_lds, unsigned char* v_lds,
                                               const unsigned char* pool, float* sink) {
     const int lane = threadIdx.x & 63, wave8 = threadIdx.x >> 6, r = lane & 31, half = lane >> 5;
@@ -238,11 +249,11 @@ __device__ __forceinline__ void slot_products(int what, int iters, unsigned char
 #pragma unroll
             for (int t2 = 0; t2 < 8; ++t2)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) o_acc[i] = slot_mfma(qf[t2], pf[t2], o_acc[i]);
+                for (int i = 0; i < 4; ++i) o_acc[i] = slot_mfma<NARROW>(qf[t2], pf[t2], pf[(t2 + 3) & 7], o_acc[i]);
 #pragma unroll
             for (int ks = 0; ks < 8; ++ks)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) s[j] = slot_mfma(pf[ks], qf[ks], s[j]);
+                for (int j = 0; j < 4; ++j) s[j] = slot_mfma<NARROW>(pf[ks], qf[ks], qf[(ks + 3) & 7], s[j]);
         } else {
             const unsigned char* v_blk = v_lds + (it & 1) * kSlotBlockBytes;
             const unsigned char* v_nxt = v_lds + ((it + 1) & 1) * kSlotBlockBytes;
@@ -266,7 +277,7 @@ __device__ __forceinline__ void slot_products(int what, int iters, unsigned char
                 for (int i = 0; i < 4; ++i) {
                     const slot_s16x4_t lo = vlo[t2 & 1][i], hi = vhi[t2 & 1][i];
                     const slot_s16x8_t both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                    o_acc[i] = slot_mfma(__builtin_bit_cast(bf16x8_t, both), pf[t2], o_acc[i]);
+                    o_acc[i] = slot_mfma<NARROW>(__builtin_bit_cast(bf16x8_t, both), pf[t2], pf[(t2 + 3) & 7], o_acc[i]);
                     if (t2 + 2 < 8) {
                         const unsigned char* src = v_blk + 16 * (t2 + 2) * kSlotRowBytes + v_rd[i];
                         vlo[t2 & 1][i] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((slot_lds_s16x4_ptr)src);
@@ -294,7 +305,7 @@ __device__ __forceinline__ void slot_products(int what, int iters, unsigned char
             for (int ks = 0; ks < 8; ++ks) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    s[j] = slot_mfma(kf[ks & 1][j], qf[ks], s[j]);
+                    s[j] = slot_mfma<NARROW>(kf[ks & 1][j], qf[ks], qf[(ks + 3) & 7], s[j]);
                     if (ks + 2 < 8) k_read(ks & 1, j, ks + 2);
                     else if (PREFETCH) v_first(v_nxt, ks & 1, j);   // the next slot's first two steps of P.V
                 }
@@ -357,7 +368,7 @@ __device__ __forceinline__ void slot_softmax(int what, int iters, unsigned char*
     sink[blockIdx.x * 512 + threadIdx.x] = l_i + m_i + (float)packed;
 }
 
-template <bool LDS, bool PREFETCH>
+template <bool LDS, bool PREFETCH, bool NARROW>
 __global__ void __launch_bounds__(512, 1) attn_slot_kernel(int what, int iters, const unsigned char* pool, float* sink,
                                                            long long* cycles) {
     __shared__ __attribute__((aligned(1024))) unsigned char k_lds[2 * kSlotBlockBytes];
@@ -378,7 +389,7 @@ __global__ void __launch_bounds__(512, 1) attn_slot_kernel(int what, int iters, 
     const unsigned char* mine = (what & kSlotPrivate) ? pool + (size_t)blockIdx.x * 65536 : pool;
     const long long t0 = clock64();
     if (wave8 < 4) {
-        if (what & kSlotProducts) slot_products<LDS, PREFETCH>(what, iters, k_lds, v_lds, mine, sink);
+        if (what & kSlotProducts) slot_products<LDS, PREFETCH, NARROW>(what, iters, k_lds, v_lds, mine, sink);
         else for (int it = 0; it < iters; ++it) __builtin_amdgcn_s_barrier();
     } else {
         if (what & kSlotSoftmax) slot_softmax(what, iters, k_lds, v_lds, mine, sink);
@@ -479,7 +490,8 @@ extern "C" int syn_probe_attn_slot(const void* pool, int64_t pool_bytes, int32_t
                                    float* sink, int64_t* cycles, syn_stream_t stream) {
     using namespace syn;
     if (pool == nullptr || sink == nullptr || cycles == nullptr || workgroups <= 0 || iters <= 0) return SYN_EINVAL;
-    if (what <= 0 || what >= 128 || !(what & (kSlotProducts | kSlotSoftmax))) return SYN_EINVAL;
+    if (what <= 0 || what >= 256 || !(what & (kSlotProducts | kSlotSoftmax))) return SYN_EINVAL;
+    if ((what & kSlotNarrow) && !(what & kSlotProducts)) return SYN_EINVAL;
     if ((what & kSlotPrefetch) && !(what & kSlotLds)) return SYN_EINVAL;
     // a workgroup's fills read 32 KB pieces at pool (+ 64 KB * workgroup with kSlotPrivate) + 32 KB * (slot % 1024)
     if (pool_bytes < (int64_t)workgroups * 65536 + 1024 * (int64_t)kSlotBlockBytes) return SYN_EINVAL;
@@ -488,8 +500,16 @@ extern "C" int syn_probe_attn_slot(const void* pool, int64_t pool_bytes, int32_t
     long long* c = reinterpret_cast<long long*>(cycles);
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     const dim3 grid(workgroups), block(512);
-    if (!(what & kSlotLds)) hipLaunchKernelGGL((attn_slot_kernel<false, false>), grid, block, 0, s, what, iters, g, sink, c);
-    else if (what & kSlotPrefetch) hipLaunchKernelGGL((attn_slot_kernel<true, true>), grid, block, 0, s, what, iters, g, sink, c);
-    else hipLaunchKernelGGL((attn_slot_kernel<true, false>), grid, block, 0, s, what, iters, g, sink, c);
+    const bool narrow = (what & kSlotNarrow) != 0;
+    if (!(what & kSlotLds)) {
+        if (narrow) hipLaunchKernelGGL((attn_slot_kernel<false, false, true>), grid, block, 0, s, what, iters, g, sink, c);
+        else hipLaunchKernelGGL((attn_slot_kernel<false, false, false>), grid, block, 0, s, what, iters, g, sink, c);
+    } else if (what & kSlotPrefetch) {
+        if (narrow) hipLaunchKernelGGL((attn_slot_kernel<true, true, true>), grid, block, 0, s, what, iters, g, sink, c);
+        else hipLaunchKernelGGL((attn_slot_kernel<true, true, false>), grid, block, 0, s, what, iters, g, sink, c);
+    } else {
+        if (narrow) hipLaunchKernelGGL((attn_slot_kernel<true, false, true>), grid, block, 0, s, what, iters, g, sink, c);
+        else hipLaunchKernelGGL((attn_slot_kernel<true, false, false>), grid, block, 0, s, what, iters, g, sink, c);
+    }
     return (int)hipGetLastError();
 }

@@ -142,14 +142,17 @@ def test_attention_slot_probe_runs_every_piece_and_rejects_bad_arguments(hip):
     def run(what, nbytes=needed, wg=workgroups):
         return hip.syn_probe_attn_slot(pool.data_ptr(), nbytes, wg, iters, what, sink.data_ptr(), cycles.data_ptr(), stream)
 
-    for what in (1, 2, 3, 1 | 4, 3 | 4, 3 | 4 | 8, 3 | 4 | 8 | 16, 3 | 4 | 8 | 32, 1 | 4 | 16, 2 | 8, 3 | 4 | 8 | 64):
+    for what in (1, 2, 3, 1 | 4, 3 | 4, 3 | 4 | 8, 3 | 4 | 8 | 16, 3 | 4 | 8 | 32, 1 | 4 | 16, 2 | 8, 3 | 4 | 8 | 64,
+                 1 | 128, 3 | 4 | 8 | 32 | 128, 3 | 4 | 8 | 16 | 128):
         cycles.zero_()
         _lib.check("syn_probe_attn_slot", run(what))
         torch.cuda.synchronize()
         assert min(cycles.tolist()) > 0, what
         assert torch.isfinite(sink).all()
     assert run(0) == _lib.SYN_EINVAL
-    assert run(128) == _lib.SYN_EINVAL
+    assert run(256) == _lib.SYN_EINVAL
+    assert run(128) == _lib.SYN_EINVAL               # the narrow form of products that do not run
+    assert run(2 | 128) == _lib.SYN_EINVAL
     assert run(4) == _lib.SYN_EINVAL                 # operands from LDS, but neither half runs
     assert run(1 | 16) == _lib.SYN_EINVAL            # early fragments without LDS reads
     assert run(3, nbytes=needed - 1) == _lib.SYN_EINVAL
