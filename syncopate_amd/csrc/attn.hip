@@ -1178,6 +1178,7 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
         // sixteen products before the end of weighted_values, into registers of used-up probabilities, measured the same.)
         auto scores = [&](const int n) __attribute__((always_inline)) {
             const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
+            __builtin_amdgcn_s_setprio(3);       // (the first products of a segment have no weighted_values before them)
             frag_t kf[2][kGS];
             const unsigned char* k_row = k_lds + (n & 1) * kBlockBytes + k_rd;
             // (opaque to the compiler, which would otherwise carry the four chunk offsets in registers around the loop
@@ -1220,6 +1221,7 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
         // which is at or below the lower q block), so its running maximum is finite and a wholly masked block adds
         // exact zeros.
         auto softmax = [&](const int past) __attribute__((always_inline)) {
+            __builtin_amdgcn_s_setprio(0);
             if ((CAUSAL || MODE != kPairTiles) && past > 0) {
                 // q row wave * 32 + 16 b + c16 against kv position 16 a + 4 g + i of the block
                 const int lim = wave * 32 + c16 - 4 * g - (past - 1) * kBlockN;     // mask where 16 a + i > lim + 16 b
@@ -1272,8 +1274,13 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
         };
 
         // O^T += V(n)^T . P^T: 8 d tiles x 4 kv steps of 32, each V^T fragment against the two halves of the q slice
+        // A wavefront in its products asks to be issued before the other wavefront of its SIMD, which is in its softmax
+        // (s_setprio 3 here and in `scores`, 0 in `softmax`): the matrix pipe is the one that must not wait.  1.5 to
+        // 3 % on the all-to-all tables, which run at the full clock; nothing on the all-gather table, which the board's
+        // power limit bounds.
         auto weighted_values = [&](const int n) __attribute__((always_inline)) {
             typedef short s16x8_t __attribute__((ext_vector_type(8)));
+            __builtin_amdgcn_s_setprio(3);
             const unsigned char* v_blk = v_lds + (n & 1) * kPairVBlockBytes;
             // group w = kv step w / kPer, d tiles kG (w % kPer) .. + kG
             auto v_at = [&](const int w, const int j) __attribute__((always_inline)) {
