@@ -1170,16 +1170,18 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
         };
 
         constexpr int kG = 4, kPer = 8 / kG, kGroups = 4 * kPer;          // V^T fragments per group of products, groups per step
-        constexpr int kGS = 2, kPerS = 8 / kGS, kGroupsS = 4 * kPerS;     // the same for the K fragments of the scores
+        constexpr int kGS = 2, kPerS = 8 / kGS, kGroupsS = 4 * kPerS;     // the same for the K fragments of the scores,
+        constexpr int kDS = 4;                                            // of which this many groups are in registers
         // S^T = K(n) . Q^T: 8 kv tiles x 4 k steps, each K fragment against the two halves of the q slice.
-        // Group u = k step u / kPerS, kv tiles kGS (u % kPerS) .. + kGS.  The fragments of groups u and u + 1 are in
-        // registers; the register a pair of products has just consumed is refilled with the fragment of group u + 2, so
-        // a read has almost two groups (128 MFMA cycles) to come back.  (Asking for the first two groups' fragments
+        // Group u = k step u / kPerS, kv tiles kGS (u % kPerS) .. + kGS.  The fragments of group u and of the
+        // next three are in registers; the register a pair of products has just consumed is refilled with the fragment
+        // of group u + 4, so a read has almost four groups (256 MFMA cycles) to come back - two groups ahead measured 2
+        // to 3 % slower, groups of four tiles two ahead the same as this.  (Asking for the first groups' fragments
         // sixteen products before the end of weighted_values, into registers of used-up probabilities, measured the same.)
         auto scores = [&](const int n) __attribute__((always_inline)) {
             const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
             __builtin_amdgcn_s_setprio(3);       // (the first products of a segment have no weighted_values before them)
-            frag_t kf[2][kGS];
+            frag_t kf[kDS][kGS];
             const unsigned char* k_row = k_lds + (n & 1) * kBlockBytes + k_rd;
             // (opaque to the compiler, which would otherwise carry the four chunk offsets in registers around the loop
             // over kv blocks - registers this kernel does not have)
@@ -1189,10 +1191,10 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
                 return k_row + 16 * (kGS * (u % kPerS) + j) * kRowBytes + (swz ^ (64 * (u / kPerS)));
             };
 #pragma unroll
-            for (int u = 0; u < 2; ++u)
+            for (int u = 0; u < kDS; ++u)
 #pragma unroll
                 for (int j = 0; j < kGS; ++j) kf[u][j] = *reinterpret_cast<const frag_t*>(k_at(u, j));
-            __builtin_amdgcn_sched_group_barrier(0x100, 2 * kGS, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, kDS * kGS, 0);
 #pragma unroll
             for (int u = 0; u < kGroupsS; ++u) {
                 const int ks = u / kPerS;
@@ -1200,10 +1202,10 @@ __global__ void __launch_bounds__(kPairThreads, 1) attn_pair_kernel(const AttnPa
                 for (int j = 0; j < kGS; ++j) {
                     const int a = kGS * (u % kPerS) + j;
 #pragma unroll
-                    for (int b = 0; b < 2; ++b) s[a][b] = mfma16<T>(kf[u & 1][j], qf[b][ks], ks == 0 ? zero : s[a][b]);
-                    if (u + 2 < kGroupsS) kf[u & 1][j] = *reinterpret_cast<const frag_t*>(k_at(u + 2, j));
+                    for (int b = 0; b < 2; ++b) s[a][b] = mfma16<T>(kf[u % kDS][j], qf[b][ks], ks == 0 ? zero : s[a][b]);
+                    if (u + kDS < kGroupsS) kf[u % kDS][j] = *reinterpret_cast<const frag_t*>(k_at(u + kDS, j));
                 }
-                if (u + 2 < kGroupsS) {
+                if (u + kDS < kGroupsS) {
 #pragma unroll
                     for (int j = 0; j < kGS; ++j) {
                         __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
