@@ -37,6 +37,7 @@ from .._launch import (
     host_copy,
     host_ptr,
     launches_on_stream,
+    zeroed_int32,
     remember_checked,
     require_cuda,
     status_words,
@@ -306,7 +307,7 @@ def attention_forward(
     # lse (base 2), lock and first-writer marker: the reference's M / guard / first
     # (template.py:382-384), one lock per 128-row q block
     lse = torch.empty((Z, H, Sq), device=dev, dtype=torch.float32)
-    scratch = torch.zeros((2, Z, H, Sq // BLOCK_M), device=dev, dtype=torch.int32)
+    scratch = zeroed_int32((2, Z, H, Sq // BLOCK_M), dev)
     tiles = int(cum_tiles) // BLOCK_M
     if visit_log is not None:
         if visit_log.dtype != torch.int32 or visit_log.numel() < 8 * tiles or not visit_log.is_contiguous():

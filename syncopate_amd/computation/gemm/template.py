@@ -33,6 +33,7 @@ from .._launch import (
     remember_note,
     require_cuda,
     status_words,
+    zeroed_int32,
 )
 
 from .tile_policy import choose_xcd_remap
@@ -129,7 +130,7 @@ def _launch(
     if producer:
         if counter_buffer is None:
             # equal to the number of waves (template.py:388)
-            counter_buffer = torch.zeros((num_waves,), device=dev, dtype=torch.int32)
+            counter_buffer = zeroed_int32((num_waves,), dev)
         elif counter_buffer.dtype != torch.int32 or counter_buffer.numel() < num_waves:
             raise ValueError("counter buffer must be int32 with one word per wave")
 

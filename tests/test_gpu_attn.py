@@ -553,3 +553,29 @@ def test_causal_producer_counts_tiles_above_the_diagonal(hip):
         assert counters.tolist() == [Z * H * S // 128] * 3
         assert flags.tolist() == [1, 1, 1]
         assert _rel(o, ref) <= REL_TOL
+
+
+def test_lock_areas_come_zeroed_across_many_launches(hip):
+    """The launcher's lock words come out of a pool that is zero-filled sixteen launches at a time: forty merging
+    launches in a row (the pool wraps twice), on the current stream and on another one, each against the fp32
+    reference - a launch that found a used lock word would skip or double a merge."""
+    from syncopate_amd.computation.attn import attention_forward
+    from syncopate_amd.computation._launch import check_status
+
+    Z, H, Sq, Skv = 1, 2, 512, 1024
+    q, k, v = _qkv(Z, H, Sq, Skv, torch.bfloat16, seed=77)
+    chunks = [(256, 512), (0, 256), (768, 1024), (512, 768)]
+    offsets, sizes, cums, signals, total = _kv_waves(Z, H, Sq, chunks, [-1] * 4)
+    flags = torch.ones(1, dtype=torch.int64, device="cuda")
+    sm_scale = 128 ** -0.5
+    ref = numerics.sdpa_fp32(q, k, v, sm_scale)
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    for stream in (None, side):
+        outs = [attention_forward(qd, kd, vd, sm_scale, wave_offsets=offsets, wave_sizes=sizes, cum_wave_sizes=cums,
+                                  signal_ptr=flags, signal_offsets=signals, NUM_WAVES=4, cum_tiles=total, num_programs=3,
+                                  pair_q_blocks=True, stream=stream) for _ in range(40)]
+        check_status()
+        for o in outs:
+            assert _rel(o, ref) <= REL_TOL
